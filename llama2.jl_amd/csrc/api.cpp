@@ -1,0 +1,982 @@
+// C ABI of libl2hip.so (declared in include/l2h.h): contexts, device-resident models, the
+// recorded per-token launch sequence, single-operator entry points and measurement helpers.
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <string>
+#include <vector>
+
+#include "l2h_internal.h"
+
+// ------------------------------------------------------------------------------------------
+struct l2h_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    std::string err;
+    hipDeviceProp_t prop;
+};
+
+static std::string g_create_err;
+
+static int set_err(l2h_ctx *ctx, int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx)
+        ctx->err = buf;
+    else
+        g_create_err = buf;
+    return code;
+}
+
+#define HIPCHK(ctx, call)                                                                          \
+    do {                                                                                           \
+        hipError_t e_ = (call);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            return set_err((ctx), L2H_EHIP, "%s:%d: %s failed: %s", __FILE__, __LINE__, #call,     \
+                           hipGetErrorString(e_));                                                 \
+    } while (0)
+
+static bool is_kquant(int type) {
+    return type == L2H_TYPE_Q4_K || type == L2H_TYPE_Q5_K || type == L2H_TYPE_Q6_K;
+}
+static bool type_ok(int type) { return type == L2H_TYPE_F32 || is_kquant(type); }
+
+static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
+
+// Lays out the field streams of a tensor inside one allocation (see DevTensor).
+static int dev_tensor_alloc(l2h_ctx *ctx, int type, int64_t ne0, int64_t ne1, DevTensor *t) {
+    *t = DevTensor();
+    t->type = type;
+    t->ne0 = ne0;
+    t->ne1 = ne1;
+    if (type == L2H_TYPE_F32) {
+        t->nb = 0;
+        t->gguf_bytes = ne0 * ne1 * 4;
+        t->bytes = align256(t->gguf_bytes);
+        HIPCHK(ctx, hipMalloc(&t->base, (size_t)t->bytes));
+        t->f32 = (const float *)t->base;
+        return L2H_OK;
+    }
+    t->nb = ne0 / QK_K;
+    const int64_t nblk = t->nb * ne1;
+    t->gguf_bytes = nblk * l2h_gguf_block_bytes(type);
+    int64_t off_hdr = 0, off_qs = 0, off_qh = 0, off_sc = 0, off_d = 0, total = 0;
+    if (type == L2H_TYPE_Q4_K) {
+        off_hdr = 0;
+        off_qs = align256(nblk * 16);
+        total = off_qs + align256(nblk * 128);
+    } else if (type == L2H_TYPE_Q5_K) {
+        off_hdr = 0;
+        off_qh = align256(nblk * 16);
+        off_qs = off_qh + align256(nblk * 32);
+        total = off_qs + align256(nblk * 128);
+    } else {
+        off_qs = 0;
+        off_qh = align256(nblk * 128);
+        off_sc = off_qh + align256(nblk * 64);
+        off_d = off_sc + align256(nblk * 16);
+        total = off_d + align256(nblk * 2);
+    }
+    t->bytes = total;
+    HIPCHK(ctx, hipMalloc(&t->base, (size_t)total));
+    char *b = (char *)t->base;
+    if (type != L2H_TYPE_Q6_K) t->hdr = (const uint4 *)(b + off_hdr);
+    t->qs = (const uint8_t *)(b + off_qs);
+    if (type != L2H_TYPE_Q4_K) t->qh = (const uint8_t *)(b + off_qh);
+    if (type == L2H_TYPE_Q6_K) {
+        t->sc6 = (const uint32_t *)(b + off_sc);
+        t->d6 = (const uint16_t *)(b + off_d);
+    }
+    return L2H_OK;
+}
+
+static void dev_tensor_free(DevTensor *t) {
+    if (t->base) (void)hipFree(t->base);
+    *t = DevTensor();
+}
+
+// host GGUF blocks -> device field streams
+static int dev_tensor_upload(l2h_ctx *ctx, DevTensor *t, const void *host) {
+    if (t->type == L2H_TYPE_F32) {
+        HIPCHK(ctx, hipMemcpy(t->base, host, (size_t)t->gguf_bytes, hipMemcpyHostToDevice));
+        return L2H_OK;
+    }
+    void *raw = nullptr;
+    HIPCHK(ctx, hipMalloc(&raw, (size_t)t->gguf_bytes));
+    hipError_t e = hipMemcpy(raw, host, (size_t)t->gguf_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = k_repack(ctx->stream, *t, raw, false, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    (void)hipFree(raw);
+    if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "tensor upload failed: %s", hipGetErrorString(e));
+    return L2H_OK;
+}
+
+static int dev_tensor_download(l2h_ctx *ctx, const DevTensor *t, void *host) {
+    if (t->type == L2H_TYPE_F32) {
+        HIPCHK(ctx, hipMemcpy(host, t->base, (size_t)t->gguf_bytes, hipMemcpyDeviceToHost));
+        return L2H_OK;
+    }
+    void *raw = nullptr;
+    HIPCHK(ctx, hipMalloc(&raw, (size_t)t->gguf_bytes));
+    hipError_t e = k_repack(ctx->stream, *t, nullptr, true, raw);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess) e = hipMemcpy(host, raw, (size_t)t->gguf_bytes, hipMemcpyDeviceToHost);
+    (void)hipFree(raw);
+    if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "tensor download failed: %s", hipGetErrorString(e));
+    return L2H_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// context
+// ------------------------------------------------------------------------------------------
+extern "C" int l2h_ctx_create(int device, l2h_ctx **out) {
+    if (!out) return set_err(nullptr, L2H_EINVAL, "l2h_ctx_create: out is NULL");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        return set_err(nullptr, L2H_ENODEV, "no HIP device: %s", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    if (device < 0 || device >= n) return set_err(nullptr, L2H_EINVAL, "device %d out of range (0..%d)", device, n - 1);
+    l2h_ctx *ctx = new l2h_ctx();
+    ctx->device = device;
+    e = hipSetDevice(device);
+    if (e == hipSuccess) e = hipGetDeviceProperties(&ctx->prop, device);
+    if (e == hipSuccess) e = hipStreamCreate(&ctx->stream);
+    if (e != hipSuccess) {
+        set_err(nullptr, L2H_EHIP, "context setup failed: %s", hipGetErrorString(e));
+        delete ctx;
+        return L2H_EHIP;
+    }
+    if (strncmp(ctx->prop.gcnArchName, "gfx950", 6) != 0) {
+        set_err(nullptr, L2H_ENODEV, "device %d is %s; this library is built for gfx950 only", device,
+                ctx->prop.gcnArchName);
+        (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return L2H_ENODEV;
+    }
+    *out = ctx;
+    return L2H_OK;
+}
+
+extern "C" void l2h_ctx_destroy(l2h_ctx *ctx) {
+    if (!ctx) return;
+    if (ctx->stream) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+}
+
+extern "C" const char *l2h_last_error(l2h_ctx *ctx) { return ctx ? ctx->err.c_str() : g_create_err.c_str(); }
+
+extern "C" int l2h_sync(l2h_ctx *ctx) {
+    if (!ctx) return L2H_EINVAL;
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return L2H_OK;
+}
+
+extern "C" int l2h_device_info(l2h_ctx *ctx, char *name, int name_cap, int32_t *n_cu, int64_t *hbm_bytes) {
+    if (!ctx) return L2H_EINVAL;
+    if (name && name_cap > 0) snprintf(name, (size_t)name_cap, "%s (%s)", ctx->prop.name, ctx->prop.gcnArchName);
+    if (n_cu) *n_cu = ctx->prop.multiProcessorCount;
+    if (hbm_bytes) *hbm_bytes = (int64_t)ctx->prop.totalGlobalMem;
+    return L2H_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// model
+// ------------------------------------------------------------------------------------------
+struct l2h_model {
+    l2h_ctx *ctx = nullptr;
+    l2h_config c{};
+    int hs = 0, kv_dim = 0;
+    float theta_scale = 0.0f;
+    DevTensor glob[3];
+    std::vector<DevTensor> layer;  // [n_layers][L2H_N_ROLES]
+    bool finalized = false;
+    // RunState (reference src/inference.jl:72-100) in device memory
+    float *x = nullptr, *xb = nullptr, *xb2 = nullptr, *hb = nullptr, *hb2 = nullptr, *q = nullptr, *k = nullptr,
+          *v = nullptr, *att = nullptr, *logits = nullptr;
+    double *qd = nullptr, *pd = nullptr, *part = nullptr;
+    Q8Dev xq{nullptr, nullptr, nullptr};
+    float *kc = nullptr, *vc = nullptr;  // [n_layers] x per-layer cache
+    int64_t cache_layer_elems = 0;
+    DecodeCtl *ctl = nullptr;
+    int32_t *prompt_dev = nullptr, *out_tokens = nullptr;
+    int64_t *argmax_partial = nullptr;
+    int max_out = 0;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    std::vector<void *> allocs;
+
+    DevTensor &L(int layer_idx, int role) { return layer[(size_t)layer_idx * L2H_N_ROLES + role]; }
+};
+
+static int q8_alloc(l2h_ctx *ctx, int64_t n, Q8Dev *q, std::vector<void *> *track) {
+    void *p = nullptr;
+    const int64_t o_bs = align256(n), o_d = o_bs + align256(n / 8 + 16);
+    HIPCHK(ctx, hipMalloc(&p, (size_t)(o_d + align256(n / 64 + 16))));
+    q->qs = (int8_t *)p;
+    q->bsums = (int16_t *)((char *)p + o_bs);
+    q->d = (float *)((char *)p + o_d);
+    if (track) track->push_back(p);
+    return L2H_OK;
+}
+
+extern "C" int l2h_model_create(l2h_ctx *ctx, const l2h_config *cfg, l2h_model **out) {
+    if (!ctx || !cfg || !out) return set_err(ctx, L2H_EINVAL, "l2h_model_create: NULL argument");
+    *out = nullptr;
+    const l2h_config &c = *cfg;
+    if (c.dim <= 0 || c.hidden_dim <= 0 || c.n_layers <= 0 || c.n_heads <= 0 || c.n_kv_heads <= 0 ||
+        c.vocab_size <= 0 || c.seq_len <= 0)
+        return set_err(ctx, L2H_EINVAL, "config fields must be positive");
+    if (c.dim % c.n_heads != 0) return set_err(ctx, L2H_EINVAL, "dim %d not divisible by n_heads %d", c.dim, c.n_heads);
+    if (c.n_heads % c.n_kv_heads != 0)
+        return set_err(ctx, L2H_EINVAL, "n_heads %d not divisible by n_kv_heads %d", c.n_heads, c.n_kv_heads);
+    const int hs = c.dim / c.n_heads;
+    if (hs % 4 != 0 || hs > 1024) return set_err(ctx, L2H_EINVAL, "head_size %d must be a multiple of 4, <= 1024", hs);
+    l2h_model *m = new l2h_model();
+    m->ctx = ctx;
+    m->c = c;
+    m->hs = hs;
+    m->kv_dim = hs * c.n_kv_heads;
+    // theta_scale = freq_base ^ (-1/(head_size/2)) in fp32 (reference src/inference.jl:119)
+    m->theta_scale = powf(c.rope_freq_base, -(1.0f / (float)(hs / 2)));
+    m->layer.resize((size_t)c.n_layers * L2H_N_ROLES);
+    *out = m;
+    return L2H_OK;
+}
+
+static void model_free_state(l2h_model *m) {
+    if (m->exec) (void)hipGraphExecDestroy(m->exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    m->exec = nullptr;
+    m->graph = nullptr;
+    for (void *p : m->allocs) (void)hipFree(p);
+    m->allocs.clear();
+    m->finalized = false;
+}
+
+extern "C" void l2h_model_destroy(l2h_model *m) {
+    if (!m) return;
+    (void)hipStreamSynchronize(m->ctx->stream);
+    model_free_state(m);
+    for (auto &t : m->glob) dev_tensor_free(&t);
+    for (auto &t : m->layer) dev_tensor_free(&t);
+    delete m;
+}
+
+static const char *role_name(int role) {
+    static const char *n[] = {"token_embedding_table", "rms_final_weight", "output_weight", "rms_att_weight",
+                              "rms_ffn_weight", "wq", "wk", "wv", "wo", "w1", "w2", "w3"};
+    return (role >= 0 && role < L2H_N_ROLES) ? n[role] : "?";
+}
+
+extern "C" int l2h_model_set_tensor(l2h_model *m, int role, int layer, int type, const void *host, int64_t ne0,
+                                    int64_t ne1) {
+    if (!m || !host) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "l2h_model_set_tensor: NULL argument");
+    l2h_ctx *ctx = m->ctx;
+    if (m->finalized) return set_err(ctx, L2H_ESTATE, "model already finalized");
+    if (role < 0 || role >= L2H_N_ROLES) return set_err(ctx, L2H_EINVAL, "role %d out of range", role);
+    if (!type_ok(type)) return set_err(ctx, L2H_ETYPE, "tensor type %d not implemented", type);
+    if (role >= 3 && (layer < 0 || layer >= m->c.n_layers))
+        return set_err(ctx, L2H_EINVAL, "layer %d out of range", layer);
+    const l2h_config &c = m->c;
+    int64_t e0 = 0, e1 = 0;
+    switch (role) {
+    case L2H_TOK_EMB:
+    case L2H_OUTPUT: e0 = c.dim; e1 = c.vocab_size; break;
+    case L2H_RMS_FINAL:
+    case L2H_RMS_ATT:
+    case L2H_RMS_FFN: e0 = c.dim; e1 = 1; break;
+    case L2H_WQ:
+    case L2H_WO: e0 = c.dim; e1 = c.dim; break;
+    case L2H_WK:
+    case L2H_WV: e0 = c.dim; e1 = m->kv_dim; break;
+    case L2H_W1:
+    case L2H_W3: e0 = c.dim; e1 = c.hidden_dim; break;
+    case L2H_W2: e0 = c.hidden_dim; e1 = c.dim; break;
+    }
+    if (ne0 != e0 || ne1 != e1)
+        return set_err(ctx, L2H_EINVAL, "%s: shape (%lld, %lld) does not match config (%lld, %lld)", role_name(role),
+                       (long long)ne0, (long long)ne1, (long long)e0, (long long)e1);
+    if ((role == L2H_RMS_FINAL || role == L2H_RMS_ATT || role == L2H_RMS_FFN) && type != L2H_TYPE_F32)
+        return set_err(ctx, L2H_ETYPE, "%s must be F32", role_name(role));
+    if (is_kquant(type) && ne0 % QK_K != 0)
+        return set_err(ctx, L2H_EINVAL, "%s: ne0 = %lld is not a multiple of 256", role_name(role), (long long)ne0);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevTensor &slot = role < 3 ? m->glob[role] : m->L(layer, role);
+    dev_tensor_free(&slot);
+    int rc = dev_tensor_alloc(ctx, type, ne0, ne1, &slot);
+    if (rc) return rc;
+    rc = dev_tensor_upload(ctx, &slot, host);
+    if (rc) dev_tensor_free(&slot);
+    return rc;
+}
+
+extern "C" int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t host_bytes) {
+    if (!m || !host) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "l2h_model_get_tensor: NULL argument");
+    if (role < 0 || role >= L2H_N_ROLES || (role >= 3 && (layer < 0 || layer >= m->c.n_layers)))
+        return set_err(m->ctx, L2H_EINVAL, "role/layer out of range");
+    DevTensor &t = role < 3 ? m->glob[role] : m->L(layer, role);
+    if (!t.base) return set_err(m->ctx, L2H_ESTATE, "%s not set", role_name(role));
+    if (host_bytes != t.gguf_bytes)
+        return set_err(m->ctx, L2H_EINVAL, "buffer is %lld bytes, tensor is %lld", (long long)host_bytes,
+                       (long long)t.gguf_bytes);
+    return dev_tensor_download(m->ctx, &t, host);
+}
+
+template <class T>
+static int dalloc(l2h_model *m, T **p, int64_t n, bool zero) {
+    void *v = nullptr;
+    const size_t bytes = (size_t)std::max<int64_t>(n, 1) * sizeof(T);
+    HIPCHK(m->ctx, hipMalloc(&v, bytes));
+    m->allocs.push_back(v);
+    if (zero) HIPCHK(m->ctx, hipMemset(v, 0, bytes));
+    *p = (T *)v;
+    return L2H_OK;
+}
+
+// ---- the per-token launch sequence: transformer! (reference src/inference.jl:222-315) ----------
+static hipError_t launch_matvecs(l2h_model *m, const DevTensor *const *w, float *const *y, int n, const float *xf,
+                                 const float *resid) {
+    // consecutive tensors of one type share a launch
+    hipStream_t s = m->ctx->stream;
+    int i = 0;
+    while (i < n) {
+        int j = i + 1;
+        while (j < n && j - i < 3 && w[j]->type == w[i]->type) j++;
+        MatvecArgs a{};
+        a.nseg = j - i;
+        a.total_rows = 0;
+        for (int k = i; k < j; k++) {
+            a.seg[k - i].w = *w[k];
+            a.seg[k - i].y = y[k];
+            a.total_rows += w[k]->ne1;
+        }
+        a.xq = m->xq;
+        a.xf = xf;
+        a.resid = resid;
+        a.dbg_isc = nullptr;
+        a.dbg_imin = nullptr;
+        hipError_t e = k_matvec(s, a);
+        if (e != hipSuccess) return e;
+        i = j;
+    }
+    return hipSuccess;
+}
+
+static hipError_t enqueue_token(l2h_model *m) {
+    hipStream_t s = m->ctx->stream;
+    const l2h_config &c = m->c;
+    hipError_t e;
+#define CK(call)                  \
+    do {                          \
+        e = (call);               \
+        if (e != hipSuccess) return e; \
+    } while (0)
+    CK(k_embed(s, m->glob[L2H_TOK_EMB], m->ctl, m->prompt_dev, m->x));
+    for (int l = 0; l < c.n_layers; l++) {
+        float *kc = m->kc + (int64_t)l * m->cache_layer_elems;
+        float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
+        const DevTensor &wq = m->L(l, L2H_WQ), &wk = m->L(l, L2H_WK), &wv = m->L(l, L2H_WV), &wo = m->L(l, L2H_WO),
+                        &w1 = m->L(l, L2H_W1), &w2 = m->L(l, L2H_W2), &w3 = m->L(l, L2H_W3);
+        // attention rmsnorm (:244) + q8_K image of xb for the k-quant consumers
+        CK(k_rmsnorm_quant(s, m->x, m->L(l, L2H_RMS_ATT).f32, m->xb, m->xq,
+                           is_kquant(wq.type) || is_kquant(wk.type) || is_kquant(wv.type), c.dim));
+        {  // q, k, v (:247-249)
+            const DevTensor *w[3] = {&wq, &wk, &wv};
+            float *y[3] = {m->q, m->k, m->v};
+            CK(launch_matvecs(m, w, y, 3, m->xb, nullptr));
+        }
+        // rope (:255-256) + cache append (:259-260)
+        CK(k_rope_kv(s, m->q, m->qd, m->k, m->v, kc, vc, m->ctl, m->hs, c.n_heads, c.n_kv_heads, c.seq_len,
+                     m->theta_scale, c.rope_is_neox));
+        // attention (:263-278) -> xb
+        CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->xq, is_kquant(wo.type), m->ctl, m->hs,
+                       c.n_heads, c.n_kv_heads, c.seq_len));
+        {  // x += wo * xb (:281-284)
+            const DevTensor *w[1] = {&wo};
+            float *y[1] = {m->x};
+            CK(launch_matvecs(m, w, y, 1, m->xb, m->x));
+        }
+        CK(k_rmsnorm_quant(s, m->x, m->L(l, L2H_RMS_FFN).f32, m->xb, m->xq, is_kquant(w1.type) || is_kquant(w3.type),
+                           c.dim));  // :287
+        {                            // hb = w1 xb, hb2 = w3 xb (:291-292)
+            const DevTensor *w[2] = {&w1, &w3};
+            float *y[2] = {m->hb, m->hb2};
+            CK(launch_matvecs(m, w, y, 2, m->xb, nullptr));
+        }
+        CK(k_swiglu_quant(s, m->hb, m->hb2, m->xq, is_kquant(w2.type), c.hidden_dim));  // :295-299
+        {                                                                               // x += w2 hb (:302-305)
+            const DevTensor *w[1] = {&w2};
+            float *y[1] = {m->x};
+            CK(launch_matvecs(m, w, y, 1, m->hb, m->x));
+        }
+    }
+    const DevTensor &wout = m->glob[L2H_OUTPUT];
+    CK(k_rmsnorm_quant(s, m->x, m->glob[L2H_RMS_FINAL].f32, m->x, m->xq, is_kquant(wout.type), c.dim));  // :309
+    {                                                                                                     // :312
+        const DevTensor *w[1] = {&wout};
+        float *y[1] = {m->logits};
+        CK(launch_matvecs(m, w, y, 1, m->x, nullptr));
+    }
+    CK(k_argmax(s, m->logits, c.vocab_size, m->argmax_partial, m->ctl, m->out_tokens, m->max_out));  // :360
+#undef CK
+    return hipSuccess;
+}
+
+extern "C" int l2h_model_finalize(l2h_model *m) {
+    if (!m) return L2H_EINVAL;
+    l2h_ctx *ctx = m->ctx;
+    if (m->finalized) return set_err(ctx, L2H_ESTATE, "model already finalized");
+    const l2h_config &c = m->c;
+    for (int r = 0; r < 3; r++)
+        if (!m->glob[r].base) return set_err(ctx, L2H_ESTATE, "missing tensor %s", role_name(r));
+    for (int l = 0; l < c.n_layers; l++)
+        for (int r = 3; r < L2H_N_ROLES; r++)
+            if (!m->L(l, r).base) return set_err(ctx, L2H_ESTATE, "missing blk.%d weights (%s)", l, role_name(r));
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    int rc;
+#define DA(p, n, z)                       \
+    if ((rc = dalloc(m, &(p), (n), (z)))) \
+        return rc;
+    DA(m->x, c.dim, true);
+    DA(m->xb, c.dim, true);
+    DA(m->xb2, c.dim, true);
+    DA(m->hb, c.hidden_dim, true);
+    DA(m->hb2, c.hidden_dim, true);
+    DA(m->q, c.dim, true);
+    DA(m->k, m->kv_dim, true);
+    DA(m->v, m->kv_dim, true);
+    DA(m->att, (int64_t)c.seq_len * c.n_heads, true);
+    DA(m->logits, c.vocab_size, true);
+    DA(m->qd, c.dim, true);
+    DA(m->pd, (int64_t)c.seq_len * c.n_heads, true);
+    const int ntiles = (c.seq_len + L2H_ATT_TILE - 1) / L2H_ATT_TILE;
+    DA(m->part, (int64_t)ntiles * c.dim, true);
+    m->cache_layer_elems = (int64_t)c.seq_len * m->kv_dim;
+    DA(m->kc, m->cache_layer_elems * c.n_layers, true);
+    DA(m->vc, m->cache_layer_elems * c.n_layers, true);
+    DA(m->ctl, 1, true);
+    DA(m->prompt_dev, c.seq_len, true);
+    m->max_out = c.seq_len;
+    DA(m->out_tokens, m->max_out, true);
+    DA(m->argmax_partial, L2H_ARGMAX_BLOCKS, true);
+#undef DA
+    const int64_t maxk = ((std::max(c.dim, c.hidden_dim) + 255) / 256) * 256;
+    if ((rc = q8_alloc(ctx, maxk, &m->xq, &m->allocs))) return rc;
+    HIPCHK(ctx, hipDeviceSynchronize());
+
+    // Record the launch sequence of one token; positions and tokens are read from the
+    // control block on the device, so the recording is replayed unchanged for every step.
+    if (!getenv("L2H_NO_GRAPH")) {
+        HIPCHK(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeGlobal));
+        hipError_t e = enqueue_token(m);
+        hipGraph_t g = nullptr;
+        hipError_t e2 = hipStreamEndCapture(ctx->stream, &g);
+        if (e != hipSuccess || e2 != hipSuccess) {
+            if (g) (void)hipGraphDestroy(g);
+            return set_err(ctx, L2H_EHIP, "recording the token launch sequence failed: %s",
+                           hipGetErrorString(e != hipSuccess ? e : e2));
+        }
+        m->graph = g;
+        HIPCHK(ctx, hipGraphInstantiate(&m->exec, m->graph, nullptr, nullptr, 0));
+    }
+    m->finalized = true;
+    return L2H_OK;
+}
+
+static int run_steps(l2h_model *m, int n) {
+    l2h_ctx *ctx = m->ctx;
+    for (int i = 0; i < n; i++) {
+        if (m->exec) {
+            HIPCHK(ctx, hipGraphLaunch(m->exec, ctx->stream));
+        } else {
+            hipError_t e = enqueue_token(m);
+            if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "token launch failed: %s", hipGetErrorString(e));
+        }
+    }
+    return L2H_OK;
+}
+
+extern "C" int l2h_state_reset(l2h_model *m) {
+    if (!m) return L2H_EINVAL;
+    if (!m->finalized) return set_err(m->ctx, L2H_ESTATE, "model not finalized");
+    const size_t bytes = (size_t)m->cache_layer_elems * m->c.n_layers * 4;
+    HIPCHK(m->ctx, hipMemsetAsync(m->kc, 0, bytes, m->ctx->stream));
+    HIPCHK(m->ctx, hipMemsetAsync(m->vc, 0, bytes, m->ctx->stream));
+    HIPCHK(m->ctx, hipStreamSynchronize(m->ctx->stream));
+    return L2H_OK;
+}
+
+static int kv_xfer(l2h_model *m, int layer, int pos0, int n, float *k, float *v, bool to_cache) {
+    if (!m) return L2H_EINVAL;
+    l2h_ctx *ctx = m->ctx;
+    if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
+    if (layer < 0 || layer >= m->c.n_layers || pos0 < 0 || n < 0 || pos0 + n > m->c.seq_len || !k || !v)
+        return set_err(ctx, L2H_EINVAL, "kv range out of bounds (layer %d, pos %d, n %d)", layer, pos0, n);
+    if (n == 0) return L2H_OK;
+    const size_t bytes = (size_t)n * m->kv_dim * 4;
+    float *dk = nullptr, *dv = nullptr;
+    HIPCHK(ctx, hipMalloc((void **)&dk, bytes));
+    hipError_t e = hipMalloc((void **)&dv, bytes);
+    if (e == hipSuccess && to_cache) {
+        e = hipMemcpy(dk, k, bytes, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(dv, v, bytes, hipMemcpyHostToDevice);
+    }
+    if (e == hipSuccess)
+        e = k_kv_layout(ctx->stream, m->kc + layer * m->cache_layer_elems, m->vc + layer * m->cache_layer_elems, dk, dv,
+                        pos0, n, m->hs, m->c.n_kv_heads, m->c.seq_len, to_cache);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess && !to_cache) {
+        e = hipMemcpy(k, dk, bytes, hipMemcpyDeviceToHost);
+        if (e == hipSuccess) e = hipMemcpy(v, dv, bytes, hipMemcpyDeviceToHost);
+    }
+    (void)hipFree(dk);
+    if (dv) (void)hipFree(dv);
+    if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "kv transfer failed: %s", hipGetErrorString(e));
+    return L2H_OK;
+}
+
+extern "C" int l2h_kv_write(l2h_model *m, int layer, int pos0, int n, const float *k, const float *v) {
+    return kv_xfer(m, layer, pos0, n, (float *)k, (float *)v, true);
+}
+extern "C" int l2h_kv_read(l2h_model *m, int layer, int pos0, int n, float *k, float *v) {
+    return kv_xfer(m, layer, pos0, n, k, v, false);
+}
+
+static int generate_impl(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new, int32_t *out,
+                         float *last_logits, float *decode_ms) {
+    if (!m) return L2H_EINVAL;
+    l2h_ctx *ctx = m->ctx;
+    if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
+    if (!prompt || n_prompt < 1) return set_err(ctx, L2H_EINVAL, "prompt cannot be empty");  // inference.jl:326-328
+    if (n_new < 0 || pos0 < 0) return set_err(ctx, L2H_EINVAL, "negative count");
+    const int total = n_prompt - 1 + n_new;
+    if (pos0 + total > m->c.seq_len)
+        return set_err(ctx, L2H_EINVAL, "pos0 %d + %d steps exceeds seq_len %d", pos0, total, m->c.seq_len);
+    if (n_new > 0 && !out) return set_err(ctx, L2H_EINVAL, "out is NULL");
+    for (int i = 0; i < n_prompt; i++)
+        if (prompt[i] < 0 || prompt[i] >= m->c.vocab_size)
+            return set_err(ctx, L2H_EINVAL, "prompt[%d] = %d outside vocabulary", i, prompt[i]);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DecodeCtl h{};
+    h.token = prompt[0];
+    h.pos = pos0;
+    h.step = 0;
+    h.n_prompt = n_prompt;
+    h.last_argmax = 0;
+    h.n_out = 0;
+    HIPCHK(ctx, hipMemcpyAsync(m->prompt_dev, prompt, (size_t)n_prompt * 4, hipMemcpyHostToDevice, ctx->stream));
+    HIPCHK(ctx, hipMemcpyAsync(m->ctl, &h, sizeof h, hipMemcpyHostToDevice, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    int rc;
+    if (decode_ms) {
+        hipEvent_t e0, e1;
+        HIPCHK(ctx, hipEventCreate(&e0));
+        HIPCHK(ctx, hipEventCreate(&e1));
+        if ((rc = run_steps(m, total - n_new))) return rc;
+        HIPCHK(ctx, hipEventRecord(e0, ctx->stream));
+        if ((rc = run_steps(m, n_new))) return rc;
+        HIPCHK(ctx, hipEventRecord(e1, ctx->stream));
+        HIPCHK(ctx, hipEventSynchronize(e1));
+        HIPCHK(ctx, hipEventElapsedTime(decode_ms, e0, e1));
+        (void)hipEventDestroy(e0);
+        (void)hipEventDestroy(e1);
+    } else {
+        if ((rc = run_steps(m, total))) return rc;
+    }
+    if (n_new > 0)
+        HIPCHK(ctx, hipMemcpyAsync(out, m->out_tokens, (size_t)n_new * 4, hipMemcpyDeviceToHost, ctx->stream));
+    if (last_logits)
+        HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)m->c.vocab_size * 4, hipMemcpyDeviceToHost,
+                                   ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return L2H_OK;
+}
+
+extern "C" int l2h_generate_greedy(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new,
+                                   int32_t *out, float *last_logits) {
+    return generate_impl(m, prompt, n_prompt, pos0, n_new, out, last_logits, nullptr);
+}
+
+extern "C" int l2h_generate_greedy_timed(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new,
+                                         int32_t *out, float *decode_ms) {
+    if (!decode_ms) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "decode_ms is NULL");
+    return generate_impl(m, prompt, n_prompt, pos0, n_new, out, nullptr, decode_ms);
+}
+
+extern "C" int l2h_forward(l2h_model *m, int token, int pos, float *logits, int32_t *argmax) {
+    int32_t tok = token, next = 0;
+    int rc = generate_impl(m, &tok, 1, pos, 1, &next, logits, nullptr);
+    if (rc == L2H_OK && argmax) *argmax = next;
+    return rc;
+}
+
+extern "C" int l2h_state_read(l2h_model *m, int which, float *host, int64_t n) {
+    if (!m || !host) return L2H_EINVAL;
+    if (!m->finalized) return set_err(m->ctx, L2H_ESTATE, "model not finalized");
+    const float *src = nullptr;
+    int64_t len = 0;
+    switch (which) {
+    case 0: src = m->x; len = m->c.dim; break;
+    case 1: src = m->xb; len = m->c.dim; break;
+    case 2: src = m->q; len = m->c.dim; break;
+    case 3: src = m->k; len = m->kv_dim; break;
+    case 4: src = m->v; len = m->kv_dim; break;
+    case 5: src = m->hb; len = m->c.hidden_dim; break;
+    case 6: src = m->logits; len = m->c.vocab_size; break;
+    default: return set_err(m->ctx, L2H_EINVAL, "unknown state buffer %d", which);
+    }
+    if (n != len) return set_err(m->ctx, L2H_EINVAL, "buffer %d holds %lld floats, asked for %lld", which,
+                                 (long long)len, (long long)n);
+    HIPCHK(m->ctx, hipStreamSynchronize(m->ctx->stream));
+    HIPCHK(m->ctx, hipMemcpy(host, src, (size_t)len * 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// single operators: upload, run the same kernel the model path uses, download
+// ------------------------------------------------------------------------------------------
+struct DevBuf {  // frees on scope exit
+    void *p = nullptr;
+    ~DevBuf() {
+        if (p) (void)hipFree(p);
+    }
+    hipError_t alloc(size_t bytes) { return hipMalloc(&p, bytes ? bytes : 1); }
+    template <class T>
+    T *as() { return (T *)p; }
+};
+
+static int q8_pack_blocks(l2h_ctx *ctx, const Q8Dev &q, int64_t n, void *out_blocks) {
+    const int64_t nb = n / QK_K;
+    std::vector<int8_t> qs((size_t)n);
+    std::vector<int16_t> bs((size_t)n / 16);
+    std::vector<float> d((size_t)nb);
+    HIPCHK(ctx, hipMemcpy(qs.data(), q.qs, (size_t)n, hipMemcpyDeviceToHost));
+    HIPCHK(ctx, hipMemcpy(bs.data(), q.bsums, (size_t)n / 8, hipMemcpyDeviceToHost));
+    HIPCHK(ctx, hipMemcpy(d.data(), q.d, (size_t)nb * 4, hipMemcpyDeviceToHost));
+    char *o = (char *)out_blocks;
+    for (int64_t b = 0; b < nb; b++, o += 292) {  // block_q8_K: f32 d, i8 qs[256], i16 bsums[16]
+        memcpy(o, &d[b], 4);
+        memcpy(o + 4, &qs[b * 256], 256);
+        memcpy(o + 260, &bs[b * 16], 32);
+    }
+    return L2H_OK;
+}
+
+extern "C" int l2h_quantize_q8k(l2h_ctx *ctx, const float *x, int64_t n, void *out_blocks) {
+    if (!ctx || !x || !out_blocks) return set_err(ctx, L2H_EINVAL, "l2h_quantize_q8k: NULL argument");
+    if (n < 0 || n % QK_K != 0) return set_err(ctx, L2H_EINVAL, "n = %lld is not a multiple of 256", (long long)n);
+    if (n == 0) return L2H_OK;
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf dx;
+    HIPCHK(ctx, dx.alloc((size_t)n * 4));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
+    Q8Dev q;
+    std::vector<void *> tr;
+    int rc = q8_alloc(ctx, n, &q, &tr);
+    if (rc) return rc;
+    hipError_t e = k_quant_q8(ctx->stream, dx.as<float>(), q, n);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess)
+        rc = q8_pack_blocks(ctx, q, n, out_blocks);
+    else
+        rc = set_err(ctx, L2H_EHIP, "quantize failed: %s", hipGetErrorString(e));
+    (void)hipFree(tr[0]);
+    return rc;
+}
+
+extern "C" int l2h_dequantize(l2h_ctx *ctx, int type, const void *blocks, int64_t nb, float *y) {
+    if (!ctx || !blocks || !y) return set_err(ctx, L2H_EINVAL, "l2h_dequantize: NULL argument");
+    if (!type_ok(type)) return set_err(ctx, L2H_ETYPE, "tensor type %d not implemented", type);
+    if (nb < 0) return set_err(ctx, L2H_EINVAL, "negative block count");
+    if (nb == 0) return L2H_OK;
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    const int64_t ne0 = type == L2H_TYPE_F32 ? nb : nb * QK_K;
+    DevTensor t;
+    int rc = dev_tensor_alloc(ctx, type, ne0, 1, &t);
+    if (rc) return rc;
+    rc = dev_tensor_upload(ctx, &t, blocks);
+    if (rc == L2H_OK) {
+        DevBuf dy;
+        hipError_t e = dy.alloc((size_t)ne0 * 4);
+        if (e == hipSuccess) e = k_dequant(ctx->stream, t, 0, 1, dy.as<float>());
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e == hipSuccess) e = hipMemcpy(y, dy.p, (size_t)ne0 * 4, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) rc = set_err(ctx, L2H_EHIP, "dequantize failed: %s", hipGetErrorString(e));
+    }
+    dev_tensor_free(&t);
+    return rc;
+}
+
+extern "C" int l2h_matmul(l2h_ctx *ctx, int type, const void *A, int64_t ne0, int64_t ne1, const float *x, float *y,
+                          int32_t *I_sc, int32_t *I_min) {
+    if (!ctx || !A || !x || !y) return set_err(ctx, L2H_EINVAL, "l2h_matmul: NULL argument");
+    if (!type_ok(type)) return set_err(ctx, L2H_ETYPE, "tensor type %d not implemented", type);
+    if (ne0 <= 0 || ne1 < 0) return set_err(ctx, L2H_EINVAL, "bad shape");
+    if (is_kquant(type) && ne0 % QK_K != 0)
+        return set_err(ctx, L2H_EINVAL, "ne0 = %lld is not a multiple of 256", (long long)ne0);
+    if ((I_sc == nullptr) != (I_min == nullptr)) return set_err(ctx, L2H_EINVAL, "I_sc and I_min go together");
+    if (I_sc && !is_kquant(type)) return set_err(ctx, L2H_EINVAL, "integer sums exist for k-quant types only");
+    if (ne1 == 0) return L2H_OK;
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevTensor t;
+    int rc = dev_tensor_alloc(ctx, type, ne0, ne1, &t);
+    if (rc) return rc;
+    rc = dev_tensor_upload(ctx, &t, A);
+    std::vector<void *> tr;
+    if (rc == L2H_OK) {
+        DevBuf dx, dy, di, dm;
+        Q8Dev q{nullptr, nullptr, nullptr};
+        hipError_t e = dx.alloc((size_t)ne0 * 4);
+        if (e == hipSuccess) e = dy.alloc((size_t)ne1 * 4);
+        if (e == hipSuccess) e = hipMemcpy(dx.p, x, (size_t)ne0 * 4, hipMemcpyHostToDevice);
+        const int64_t nints = ne1 * (ne0 / QK_K);
+        if (e == hipSuccess && I_sc) {
+            e = di.alloc((size_t)nints * 4);
+            if (e == hipSuccess) e = dm.alloc((size_t)nints * 4);
+        }
+        if (e == hipSuccess && is_kquant(type)) {
+            rc = q8_alloc(ctx, ne0, &q, &tr);
+            if (rc == L2H_OK) e = k_quant_q8(ctx->stream, dx.as<float>(), q, ne0);
+        }
+        if (rc == L2H_OK && e == hipSuccess) {
+            MatvecArgs a{};
+            a.nseg = 1;
+            a.seg[0].w = t;
+            a.seg[0].y = dy.as<float>();
+            a.total_rows = ne1;
+            a.xq = q;
+            a.xf = dx.as<float>();
+            a.resid = nullptr;
+            a.dbg_isc = di.as<int32_t>();
+            a.dbg_imin = dm.as<int32_t>();
+            e = k_matvec(ctx->stream, a);
+        }
+        if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+        if (e == hipSuccess) e = hipMemcpy(y, dy.p, (size_t)ne1 * 4, hipMemcpyDeviceToHost);
+        if (e == hipSuccess && I_sc) {
+            e = hipMemcpy(I_sc, di.p, (size_t)nints * 4, hipMemcpyDeviceToHost);
+            if (e == hipSuccess) e = hipMemcpy(I_min, dm.p, (size_t)nints * 4, hipMemcpyDeviceToHost);
+        }
+        if (rc == L2H_OK && e != hipSuccess) rc = set_err(ctx, L2H_EHIP, "matmul failed: %s", hipGetErrorString(e));
+    }
+    for (void *p : tr) (void)hipFree(p);
+    dev_tensor_free(&t);
+    return rc;
+}
+
+extern "C" int l2h_rmsnorm(l2h_ctx *ctx, float *o, const float *x, const float *weight, int64_t n) {
+    if (!ctx || !o || !x || !weight) return set_err(ctx, L2H_EINVAL, "l2h_rmsnorm: NULL argument");
+    if (n <= 0 || n > (1 << 30)) return set_err(ctx, L2H_EINVAL, "bad length");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf dx, dw, dout;
+    HIPCHK(ctx, dx.alloc((size_t)n * 4));
+    HIPCHK(ctx, dw.alloc((size_t)n * 4));
+    HIPCHK(ctx, dout.alloc((size_t)n * 4));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(dw.p, weight, (size_t)n * 4, hipMemcpyHostToDevice));
+    Q8Dev none{nullptr, nullptr, nullptr};
+    HIPCHK(ctx, k_rmsnorm_quant(ctx->stream, dx.as<float>(), dw.as<float>(), dout.as<float>(), none, false, (int)n));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(o, dout.p, (size_t)n * 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+extern "C" int l2h_rope(l2h_ctx *ctx, float *x, int head_size, int n_heads, int pos, float freq_base, int neox) {
+    if (!ctx || !x) return set_err(ctx, L2H_EINVAL, "l2h_rope: NULL argument");
+    if (head_size <= 0 || head_size % 2 != 0 || n_heads <= 0 || pos < 0)
+        return set_err(ctx, L2H_EINVAL, "bad rope arguments");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    const size_t bytes = (size_t)head_size * n_heads * 4;
+    DevBuf dx;
+    HIPCHK(ctx, dx.alloc(bytes));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, bytes, hipMemcpyHostToDevice));
+    const float theta_scale = powf(freq_base, -(1.0f / (float)(head_size / 2)));
+    HIPCHK(ctx, k_rope_only(ctx->stream, dx.as<float>(), head_size, n_heads, pos, theta_scale, neox));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(x, dx.p, bytes, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+extern "C" int l2h_softmax(l2h_ctx *ctx, float *x, int64_t n) {
+    if (!ctx || !x) return set_err(ctx, L2H_EINVAL, "l2h_softmax: NULL argument");
+    if (n <= 0) return set_err(ctx, L2H_EINVAL, "softmax of an empty vector");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf dx;
+    HIPCHK(ctx, dx.alloc((size_t)n * 4));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, k_softmax(ctx->stream, dx.as<float>(), n));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(x, dx.p, (size_t)n * 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+extern "C" int l2h_attention(l2h_ctx *ctx, float *out, const float *q, const float *kc, const float *vc,
+                             int head_size, int n_heads, int n_kv_heads, int pos) {
+    if (!ctx || !out || !q || !kc || !vc) return set_err(ctx, L2H_EINVAL, "l2h_attention: NULL argument");
+    if (head_size <= 0 || head_size % 4 != 0 || head_size > 1024 || n_heads <= 0 || n_kv_heads <= 0 ||
+        n_heads % n_kv_heads != 0 || pos < 0)
+        return set_err(ctx, L2H_EINVAL, "bad attention arguments");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    const int np = pos + 1;
+    const int seq_len = ((np + L2H_ATT_TILE - 1) / L2H_ATT_TILE) * L2H_ATT_TILE;
+    const int dim = head_size * n_heads, kv_dim = head_size * n_kv_heads;
+    const int ntiles = seq_len / L2H_ATT_TILE;
+    DevBuf dq, dqd, dkl, dvl, dkc, dvc, datt, dpd, dpart, dout, dctl;
+    HIPCHK(ctx, dq.alloc((size_t)dim * 4));
+    HIPCHK(ctx, dqd.alloc((size_t)dim * 8));
+    HIPCHK(ctx, dkl.alloc((size_t)np * kv_dim * 4));
+    HIPCHK(ctx, dvl.alloc((size_t)np * kv_dim * 4));
+    HIPCHK(ctx, dkc.alloc((size_t)seq_len * kv_dim * 4));
+    HIPCHK(ctx, dvc.alloc((size_t)seq_len * kv_dim * 4));
+    HIPCHK(ctx, datt.alloc((size_t)seq_len * n_heads * 4));
+    HIPCHK(ctx, dpd.alloc((size_t)seq_len * n_heads * 8));
+    HIPCHK(ctx, dpart.alloc((size_t)ntiles * dim * 8));
+    HIPCHK(ctx, dout.alloc((size_t)dim * 4));
+    HIPCHK(ctx, dctl.alloc(sizeof(DecodeCtl)));
+    DecodeCtl h{};
+    h.pos = pos;
+    HIPCHK(ctx, hipMemcpy(dctl.p, &h, sizeof h, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(dq.p, q, (size_t)dim * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(dkl.p, kc, (size_t)np * kv_dim * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(dvl.p, vc, (size_t)np * kv_dim * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, k_f32_to_f64(ctx->stream, dq.as<float>(), dqd.as<double>(), dim));
+    HIPCHK(ctx, k_kv_layout(ctx->stream, dkc.as<float>(), dvc.as<float>(), dkl.as<float>(), dvl.as<float>(), 0, np,
+                            head_size, n_kv_heads, seq_len, true));
+    Q8Dev none{nullptr, nullptr, nullptr};
+    HIPCHK(ctx, k_attention(ctx->stream, dqd.as<double>(), dkc.as<float>(), dvc.as<float>(), datt.as<float>(),
+                            dpd.as<double>(), dpart.as<double>(), dout.as<float>(), none, false,
+                            (const DecodeCtl *)dctl.p, head_size, n_heads, n_kv_heads, seq_len));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(out, dout.p, (size_t)dim * 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+extern "C" int l2h_swiglu(l2h_ctx *ctx, float *hb, const float *hb2, int64_t n) {
+    if (!ctx || !hb || !hb2) return set_err(ctx, L2H_EINVAL, "l2h_swiglu: NULL argument");
+    if (n <= 0 || n > (1 << 30)) return set_err(ctx, L2H_EINVAL, "bad length");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf a, b;
+    HIPCHK(ctx, a.alloc((size_t)n * 4));
+    HIPCHK(ctx, b.alloc((size_t)n * 4));
+    HIPCHK(ctx, hipMemcpy(a.p, hb, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(b.p, hb2, (size_t)n * 4, hipMemcpyHostToDevice));
+    Q8Dev none{nullptr, nullptr, nullptr};
+    HIPCHK(ctx, k_swiglu_quant(ctx->stream, a.as<float>(), b.as<float>(), none, false, (int)n));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(hb, a.p, (size_t)n * 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+extern "C" int l2h_argmax(l2h_ctx *ctx, const float *x, int64_t n, int32_t *out) {
+    if (!ctx || !x || !out) return set_err(ctx, L2H_EINVAL, "l2h_argmax: NULL argument");
+    if (n <= 0 || n > 0x7FFFFFFF) return set_err(ctx, L2H_EINVAL, "bad length");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf dx, dp, dctl, dout;
+    HIPCHK(ctx, dx.alloc((size_t)n * 4));
+    HIPCHK(ctx, dp.alloc((size_t)L2H_ARGMAX_BLOCKS * 8));
+    HIPCHK(ctx, dctl.alloc(sizeof(DecodeCtl)));
+    HIPCHK(ctx, dout.alloc(4));
+    DecodeCtl h{};
+    h.n_prompt = 1;
+    HIPCHK(ctx, hipMemcpy(dctl.p, &h, sizeof h, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, k_argmax(ctx->stream, dx.as<float>(), n, dp.as<int64_t>(), (DecodeCtl *)dctl.p, dout.as<int32_t>(), 1));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(out, dout.p, 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// measurement
+// ------------------------------------------------------------------------------------------
+extern "C" int l2h_profile_matvec(l2h_model *m, int role, int iters, float *avg_us, int64_t *bytes) {
+    if (!m || !avg_us) return L2H_EINVAL;
+    l2h_ctx *ctx = m->ctx;
+    if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
+    if (iters < 1) return set_err(ctx, L2H_EINVAL, "iters must be >= 1");
+    const int roles_qkv[3] = {L2H_WQ, L2H_WK, L2H_WV}, roles_13[2] = {L2H_W1, L2H_W3};
+    const int *roles;
+    int nr;
+    int single = role;
+    float *ys[3];
+    if (role == L2H_WQ) {
+        roles = roles_qkv; nr = 3; ys[0] = m->q; ys[1] = m->k; ys[2] = m->v;
+    } else if (role == L2H_W1) {
+        roles = roles_13; nr = 2; ys[0] = m->hb; ys[1] = m->hb2;
+    } else if (role == L2H_WO || role == L2H_W2 || role == L2H_OUTPUT) {
+        roles = &single; nr = 1; ys[0] = role == L2H_OUTPUT ? m->logits : m->xb2;
+    } else {
+        return set_err(ctx, L2H_EINVAL, "role %d has no matvec launch of its own", role);
+    }
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    // a defined input: zeros quantize to zero blocks, timing does not depend on values
+    const int n_layers = role == L2H_OUTPUT ? 1 : m->c.n_layers;
+    int64_t b = 0;
+    int launches_per_pass = 0;
+    hipEvent_t e0, e1;
+    HIPCHK(ctx, hipEventCreate(&e0));
+    HIPCHK(ctx, hipEventCreate(&e1));
+    for (int pass = 0; pass < 2; pass++) {  // pass 0 warms up
+        const int reps = pass == 0 ? 1 : iters;
+        if (pass == 1) HIPCHK(ctx, hipEventRecord(e0, ctx->stream));
+        for (int it = 0; it < reps; it++) {
+            launches_per_pass = 0;
+            for (int l = 0; l < n_layers; l++) {
+                const DevTensor *w[3];
+                b = 0;
+                for (int k = 0; k < nr; k++) {
+                    w[k] = role == L2H_OUTPUT ? &m->glob[L2H_OUTPUT] : &m->L(l, roles[k]);
+                    b += w[k]->gguf_bytes;
+                }
+                hipError_t e = launch_matvecs(m, w, ys, nr, m->xb, nullptr);
+                if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "matvec launch failed: %s", hipGetErrorString(e));
+                launches_per_pass++;
+            }
+        }
+        if (pass == 1) HIPCHK(ctx, hipEventRecord(e1, ctx->stream));
+        HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    }
+    float ms = 0.0f;
+    HIPCHK(ctx, hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *avg_us = ms * 1000.0f / (float)(iters * launches_per_pass);
+    if (bytes) *bytes = b;
+    return L2H_OK;
+}
+
+extern "C" int l2h_profile_stream_read(l2h_ctx *ctx, int64_t n_bytes, int iters, float *avg_us) {
+    if (!ctx || !avg_us) return L2H_EINVAL;
+    if (n_bytes < 16 || iters < 1) return set_err(ctx, L2H_EINVAL, "bad arguments");
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf buf, sink;
+    HIPCHK(ctx, buf.alloc((size_t)n_bytes));
+    HIPCHK(ctx, sink.alloc(16));
+    HIPCHK(ctx, hipMemset(buf.p, 1, (size_t)n_bytes));
+    hipEvent_t e0, e1;
+    HIPCHK(ctx, hipEventCreate(&e0));
+    HIPCHK(ctx, hipEventCreate(&e1));
+    HIPCHK(ctx, k_stream_read(ctx->stream, buf.as<uint4>(), n_bytes / 16, sink.as<uint32_t>()));
+    HIPCHK(ctx, hipEventRecord(e0, ctx->stream));
+    for (int i = 0; i < iters; i++)
+        HIPCHK(ctx, k_stream_read(ctx->stream, buf.as<uint4>(), n_bytes / 16, sink.as<uint32_t>()));
+    HIPCHK(ctx, hipEventRecord(e1, ctx->stream));
+    HIPCHK(ctx, hipEventSynchronize(e1));
+    float ms = 0.0f;
+    HIPCHK(ctx, hipEventElapsedTime(&ms, e0, e1));
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    *avg_us = ms * 1000.0f / (float)iters;
+    return L2H_OK;
+}

@@ -1,0 +1,115 @@
+// Internal declarations shared by the kernel files and the C-ABI layer of libl2hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "l2h.h"
+
+#define QK_K 256
+
+// ------------------------------------------------------------------------------------------
+// Device-resident weight tensor.  One allocation per tensor, split into field streams
+// (structure-of-arrays over the GGUF super-blocks) so that a wavefront reads every stream
+// with 16-byte lane loads over contiguous memory:
+//   F32   f32 [ne1][ne0]
+//   Q4_K  hdr  16 B/block  = {f16 d, f16 dmin, u8 scales[12]}  (the block's first 16 bytes)
+//         qs  128 B/block
+//   Q5_K  hdr  16 B/block, qh 32 B/block, qs 128 B/block
+//   Q6_K  ql  128 B/block, qh 64 B/block,
+//         sc   16 B/block  (int8 scales, byte (4*(2n+hh)+g) <- original byte (8n+hh+2g), so
+//                           the four scales one lane needs are one aligned dword)
+//         d     2 B/block  (f16)
+// Blocks keep GGUF order: block (row, b) has index row*nb + b in every stream.
+// ------------------------------------------------------------------------------------------
+struct DevTensor {
+    int type = -1;
+    int64_t ne0 = 0, ne1 = 0, nb = 0;  // nb = ne0/256 super-blocks per row (k-quants)
+    void *base = nullptr;
+    int64_t bytes = 0;                  // allocation size
+    int64_t gguf_bytes = 0;             // bytes the tensor occupies in a GGUF file
+    // stream pointers into base
+    const uint4 *hdr = nullptr;         // Q4_K, Q5_K
+    const uint8_t *qs = nullptr;        // Q4_K, Q5_K (128 B/block); Q6_K: ql
+    const uint8_t *qh = nullptr;        // Q5_K (32 B/block); Q6_K (64 B/block)
+    const uint32_t *sc6 = nullptr;      // Q6_K permuted scales, 4 dwords/block
+    const uint16_t *d6 = nullptr;       // Q6_K f16 d
+    const float *f32 = nullptr;         // F32
+};
+
+// q8_K activations on the device: structure-of-arrays over the block_q8_K fields.
+struct Q8Dev {
+    int8_t *qs;      // [n]
+    int16_t *bsums;  // [n/16]
+    float *d;        // [n/256]
+};
+
+// Per-sequence control block in device memory, read and advanced by the kernels so that
+// a recorded launch sequence can be replayed for every token without host involvement.
+struct DecodeCtl {
+    int32_t token;      // input token of the current step
+    int32_t pos;        // 0-based position of the current step
+    int32_t step;       // index of the current step within the generate call
+    int32_t n_prompt;   // prompt length of the generate call
+    int32_t last_argmax;
+    int32_t n_out;      // number of generated ids written so far
+    int32_t pad[2];
+};
+
+// One matvec launch covers up to 3 weight matrices that consume the same input vector.
+struct MatvecSeg {
+    DevTensor w;
+    float *y;        // output rows of this segment
+};
+struct MatvecArgs {
+    MatvecSeg seg[3];
+    int nseg;
+    int64_t total_rows;
+    Q8Dev xq;              // k-quant input
+    const float *xf;       // F32 input
+    const float *resid;    // epilogue: y = resid + result (may equal y), or nullptr
+    int32_t *dbg_isc;      // debug: per (row, block) integer sums, or nullptr
+    int32_t *dbg_imin;
+};
+
+// ---- launchers (kernel files) ----------------------------------------------------------------
+// Each returns hipGetLastError() of its launch.
+hipError_t k_repack(hipStream_t s, const DevTensor &t, const void *raw_dev, bool inverse, void *raw_out);
+hipError_t k_embed(hipStream_t s, const DevTensor &emb, const DecodeCtl *ctl, const int32_t *prompt, float *x);
+hipError_t k_dequant(hipStream_t s, const DevTensor &t, int64_t row0, int64_t nrows, float *y);
+hipError_t k_rmsnorm_quant(hipStream_t s, const float *x, const float *w, float *o, Q8Dev q8, bool do_q8, int n);
+hipError_t k_quant_q8(hipStream_t s, const float *x, Q8Dev q8, int64_t n);
+hipError_t k_swiglu_quant(hipStream_t s, float *hb, const float *hb2, Q8Dev q8, bool do_q8, int n);
+hipError_t k_matvec(hipStream_t s, const MatvecArgs &a);
+hipError_t k_rope_kv(hipStream_t s, float *q, double *qd, const float *k, const float *v, float *kc, float *vc,
+                     const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads, int seq_len,
+                     float theta_scale, int neox);
+hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
+hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
+                       double *part, float *out, Q8Dev q8, bool do_q8, const DecodeCtl *ctl, int head_size,
+                       int n_heads, int n_kv_heads, int seq_len);
+hipError_t k_softmax(hipStream_t s, float *x, int64_t n);
+hipError_t k_argmax(hipStream_t s, const float *x, int64_t n, int64_t *partial, DecodeCtl *ctl, int32_t *out_tokens,
+                    int max_out);
+hipError_t k_kv_layout(hipStream_t s, float *kc, float *vc, float *k_lin, float *v_lin, int pos0, int n, int head_size,
+                       int n_kv_heads, int seq_len, bool to_cache);
+hipError_t k_stream_read(hipStream_t s, const uint4 *p, int64_t n16, uint32_t *sink);
+hipError_t k_f32_to_f64(hipStream_t s, const float *x, double *y, int64_t n);
+
+static inline int64_t l2h_gguf_block_bytes(int type) {
+    switch (type) {
+    case L2H_TYPE_F32: return 4;
+    case L2H_TYPE_Q4_K: return 144;
+    case L2H_TYPE_Q5_K: return 176;
+    case L2H_TYPE_Q6_K: return 210;
+    }
+    return -1;
+}
+
+// number of argmax partial slots
+#define L2H_ARGMAX_BLOCKS 256
+// timesteps handled per attention work item
+#define L2H_ATT_TILE 64
