@@ -1,0 +1,178 @@
+#!/usr/bin/env python3
+"""Decode benchmark: batch-1 greedy decode of a synthetic Llama-3-8B-shaped Q4_K_S model on one
+MI355X (the configuration the headline metric is quoted on).
+
+    python bench.py [--gpus 1] [--steps 128] [--warmup 8] [--workload 8b-q4ks]
+
+A step is one decode token (one pass of the per-token path).  The model (q4_K layers, q6_K output
+projection, N(0, 0.02) weights, norms 1) is generated and quantized on the host cores, uploaded
+once, then: a 32-token seeded prompt is fed (untimed), W warm-up tokens are decoded (untimed) and
+exactly K tokens are decoded inside the timed region, with the weights and KV cache resident in
+HBM.  One JSON line is printed on stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
+
+WORKLOADS = {
+    # name: (plan, config kwargs, prompt length)
+    "8b-q4ks": ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
+                                    vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
+    "8b-q5km": ("PLAN_Q5_K_M", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
+                                    vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
+    "llama2c-f32": ("PLAN_F32", dict(dim=512, hidden_dim=1376, n_layers=8, n_heads=8, n_kv_heads=8, vocab_size=32000,
+                                     seq_len=1024, rope_freq_base=10000.0, rope_is_neox=False), 16),
+    # small shape for a quick functional run of this script
+    "tiny-q4ks": ("PLAN_Q4_K_S", dict(dim=512, hidden_dim=1024, n_layers=4, n_heads=8, n_kv_heads=2, vocab_size=2048,
+                                      seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--workload", default="8b-q4ks", choices=sorted(WORKLOADS))
+    ap.add_argument("--repeats", type=int, default=3, help="timed regions; the median is reported")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 = skip)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on exactly one GPU (batch-1 decode does not shard; see DESIGN.md); "
+            "--gpus %d is not supported" % args.gpus)
+        sys.exit(2)
+
+    pkg = entry.load_package()
+    from llama2_jl_amd import _lib, synth
+    plan_name, kw, n_prompt = WORKLOADS[args.workload]
+    cfg = pkg.ModelConfig(**kw)
+    K, W = args.steps, args.warmup
+    if n_prompt - 1 + W + K > cfg.seq_len:
+        log("steps + warmup + prompt exceed seq_len %d" % cfg.seq_len)
+        sys.exit(2)
+
+    ctx = pkg.default_context()
+    info = ctx.device_info()
+    log("device:", info)
+    t0 = time.time()
+    lm = synth.synthetic_model(cfg, getattr(synth, plan_name), seed=20240607,
+                               share_classifier=(plan_name == "PLAN_F32"))
+    log("model generated + quantized on %d host threads in %.1f s" % (synth._threads(), time.time() - t0))
+    t0 = time.time()
+    dev = lm.device()
+    ctx.sync()
+    log("uploaded in %.1f s" % (time.time() - t0))
+
+    w_bytes = synth.weight_bytes_per_token(lm)
+    kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads
+    prompt = synth.seeded_prompt(99, n_prompt, cfg.vocab_size)
+
+    # ---- timed region: K decode tokens after the prompt and W warm-up tokens --------------------
+    times, tokens = [], None
+    for rep in range(args.repeats):
+        dev.reset()
+        # prompt + warm-up tokens, untimed
+        warm = dev.generate_greedy(prompt, W) if W > 0 else np.zeros(0, np.int32)
+        # next step: position pos0, fed with the last warm-up token (or the last prompt token)
+        pos0 = n_prompt - 1 + W
+        first = int(warm[-1]) if W > 0 else int(prompt[-1])
+        ctx.sync()
+        t_start = time.perf_counter()
+        ids = dev.generate_greedy([first], K, pos0=pos0)
+        ctx.sync()
+        dt = time.perf_counter() - t_start
+        times.append(dt)
+        if tokens is None:
+            tokens = ids.tolist()
+        elif tokens != ids.tolist():
+            log("WARNING: repeat %d produced different tokens" % rep)
+        log("repeat %d: %d tokens in %.2f ms -> %.1f tok/s" % (rep, K, dt * 1e3, K / dt))
+    dt = float(np.median(times))
+    tok_s = K / dt
+    # positions read by the timed steps: pos0 .. pos0+K-1, each reads pos+1 cache rows
+    kv_bytes = 2 * cfg.n_layers * kv_dim * 4 * (pos0 + 1 + (K - 1) / 2.0)
+    bytes_per_token = w_bytes + kv_bytes
+    roofline_tok_s = HBM_PEAK_GBS * 1e9 / bytes_per_token
+
+    # ---- dominant kernel: the k-quant (or fp32) matvec, timed with HIP events on the library's
+    # stream, every layer's tensor in turn so that nothing is cache-resident ----------------------
+    roles = [("qkv", _lib.WQ), ("wo", _lib.WO), ("w1w3", _lib.W1), ("w2", _lib.W2), ("output", _lib.OUTPUT)]
+    per_kernel, tot_us, tot_b, n_launch = {}, 0.0, 0, 0
+    dominant_type = lm.weights.layers[0].w1.type if hasattr(lm.weights.layers[0].w1, "type") else 0
+    for name, role in roles:
+        us, b = dev.profile_matvec(role, iters=10)
+        per_kernel[name] = {"us": round(us, 2), "MB": round(b / 1e6, 2), "GB/s": round(b / us / 1e3, 1)}
+        out_type = lm.weights.output_weight.type if hasattr(lm.weights.output_weight, "type") else 0
+        if name != "output" or out_type == dominant_type:
+            mult = cfg.n_layers if name != "output" else 1
+            tot_us += us * mult
+            tot_b += b * mult
+            n_launch += mult
+    log("per-launch matvec timings:", json.dumps(per_kernel))
+    achieved = tot_b / tot_us / 1e3  # GB/s over the launches of the dominant kernel within one token
+    stream_us = pkg.lib().l2h_profile_stream_read
+    import ctypes
+    us = ctypes.c_float()
+    ctx.check(stream_us(ctx.handle, 2 << 30, 5, ctypes.byref(us)))
+    stream_gbs = (2 << 30) / us.value / 1e3
+    log("plain streaming read of 2 GiB: %.0f GB/s" % stream_gbs)
+
+    # ---- CPU baseline: the oracle in the reference's own arithmetic (float activations, fp32
+    # sums), rows split over the host threads like Threads.@threads; a bounded number of tokens ---
+    cpu = None
+    if args.cpu_seconds > 0:
+        orc = entry.load_oracle()
+        cores = synth._threads()
+        om = orc.model_from_language_model(lm, nthreads=cores)
+        n_tok, t_cpu = 0, 0.0
+        t_begin = time.perf_counter()
+        while n_tok < 16 and (n_tok < 2 or t_cpu < args.cpu_seconds):
+            om.forward(int(prompt[n_tok % n_prompt]), n_tok, orc.REFERENCE)
+            n_tok += 1
+            t_cpu = time.perf_counter() - t_begin
+        cpu = {"value": round(n_tok / t_cpu, 3), "unit": "tok/s", "cores": cores, "kind": "port",
+               "sample": "%d decode steps (positions 0..%d) of the same model, C restatement of the Julia CPU path "
+                         "(float activations, fp32 sums, rows split over %d threads); Julia itself is not installed"
+                         % (n_tok, n_tok - 1, cores)}
+        log("cpu baseline:", cpu)
+        om.close()
+
+    result = {
+        "metric": "decode tok/s, Llama-3-8B-shape Q4_K_S, batch 1; % of HBM-BW roofline",
+        "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": round(dt * 1e3 / K, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 dot products (q4_K/q6_K x q8_K), fp64 accumulation, fp32 activations",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "shape": kw, "plan": plan_name, "prompt_tokens": n_prompt,
+                   "decode_positions": [pos0, pos0 + K - 1], "repeats": args.repeats,
+                   "bytes_per_token": int(bytes_per_token), "weight_bytes_per_token": int(w_bytes),
+                   "roofline_tok_s_at_8TBs": round(roofline_tok_s, 1),
+                   "frac_of_roofline": round(tok_s / roofline_tok_s, 4),
+                   "tokens_head": tokens[:8]},
+        "roofline": {"bound": "hbm", "kernel": "matvec_kq_kernel (k-quant x q8_K dequant-matvec)",
+                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "bytes_per_launch": int(tot_b / max(1, n_launch)), "launches_per_token": n_launch,
+                     "avg_launch_us": round(tot_us / max(1, n_launch), 2), "per_launch": per_kernel,
+                     "measured_stream_read_GBs": round(stream_gbs, 1)},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
