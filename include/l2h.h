@@ -111,8 +111,8 @@ int l2h_generate_greedy(l2h_model *m, const int32_t *prompt, int n_prompt, int p
  * measured with HIP events on the context's stream. */
 int l2h_generate_greedy_timed(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new,
                               int32_t *out, float *decode_ms);
-/* Copies an activation of the last forward call: which = 0 x, 1 xb, 2 q, 3 k, 4 v,
- * 5 hb, 6 logits (RunState fields, src/inference.jl:72-86). */
+/* Copies an activation of the last forward call: which = 0 x, 1 xb, 2 q (rotated), 5 hb,
+ * 6 logits (RunState fields, src/inference.jl:72-86; k and v go straight into the cache). */
 int l2h_state_read(l2h_model *m, int which, float *host, int64_t n);
 
 /* ---- single operators (each is the device form of one reference function) ----------- */
@@ -128,8 +128,11 @@ int l2h_dequantize(l2h_ctx *ctx, int ggml_type, const void *blocks, int64_t nb, 
  * sums the kernel formed: [ne1][ne0/256] int32 each. */
 int l2h_matmul(l2h_ctx *ctx, int ggml_type, const void *A, int64_t ne0, int64_t ne1, const float *x, float *y,
                int32_t *I_sc, int32_t *I_min);
-/* rmsnorm!(o, x, weight) (src/inference.jl:102-110). o may alias x. */
+/* rmsnorm!(o, x, weight) (src/inference.jl:102-110). o may alias x. n <= 15360. */
 int l2h_rmsnorm(l2h_ctx *ctx, float *o, const float *x, const float *weight, int64_t n);
+/* rmsnorm! followed by q8_K quantization of the result, exactly as the matvec kernels do it in
+ * their prologue (src/inference.jl:244 then the activation quantizer); n % 256 == 0. */
+int l2h_rmsnorm_q8k(l2h_ctx *ctx, const float *x, const float *weight, int64_t n, void *out_blocks);
 /* rope!(x, pos, config) (src/inference.jl:112-167) on x[n_heads][head_size]. */
 int l2h_rope(l2h_ctx *ctx, float *x, int head_size, int n_heads, int pos, float freq_base, int neox);
 /* softmax!(x) (src/inference.jl:169-174) */

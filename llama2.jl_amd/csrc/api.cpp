@@ -205,7 +205,7 @@ struct l2h_model {
     float *x = nullptr, *xb = nullptr, *xb2 = nullptr, *hb = nullptr, *hb2 = nullptr, *q = nullptr, *k = nullptr,
           *v = nullptr, *att = nullptr, *logits = nullptr;
     double *qd = nullptr, *pd = nullptr, *part = nullptr;
-    Q8Dev xq{nullptr, nullptr, nullptr};
+    float *rope_cs = nullptr;  // cos/sin of the current position's RoPE angles, [hs/2][2]
     float *kc = nullptr, *vc = nullptr;  // [n_layers] x per-layer cache
     int64_t cache_layer_elems = 0;
     DecodeCtl *ctl = nullptr;
@@ -345,89 +345,126 @@ static int dalloc(l2h_model *m, T **p, int64_t n, bool zero) {
 }
 
 // ---- the per-token launch sequence: transformer! (reference src/inference.jl:222-315) ----------
-static hipError_t launch_matvecs(l2h_model *m, const DevTensor *const *w, float *const *y, int n, const float *xf,
-                                 const float *resid) {
-    // consecutive tensors of one type share a launch
+static PhaseArgs base_args(l2h_model *m) {
+    PhaseArgs a{};
+    a.max_grid = m->ctx->prop.multiProcessorCount;
+    a.ctl = m->ctl;
+    a.hs = m->hs;
+    a.seq_len = m->c.seq_len;
+    a.neox = m->c.rope_is_neox;
+    a.rope_cs = m->rope_cs;
+    a.qd = m->qd;
+    return a;
+}
+
+// rmsnorm (:244) + q, k, v (:247-249) + rope (:255-256) + cache append (:259-260)
+static hipError_t launch_qkv(l2h_model *m, int l) {
     hipStream_t s = m->ctx->stream;
+    const DevTensor *w[3] = {&m->L(l, L2H_WQ), &m->L(l, L2H_WK), &m->L(l, L2H_WV)};
+    float *y[3] = {m->q, nullptr, nullptr};
+    PhaseArgs a = base_args(m);
+    a.xf = m->x;
+    a.normw = m->L(l, L2H_RMS_ATT).f32;
+    a.kc = m->kc + (int64_t)l * m->cache_layer_elems;
+    a.vc = m->vc + (int64_t)l * m->cache_layer_elems;
     int i = 0;
-    while (i < n) {
+    while (i < 3) {  // consecutive tensors of one type share a launch
         int j = i + 1;
-        while (j < n && j - i < 3 && w[j]->type == w[i]->type) j++;
-        MatvecArgs a{};
+        while (j < 3 && w[j]->type == w[i]->type) j++;
         a.nseg = j - i;
-        a.total_rows = 0;
         for (int k = i; k < j; k++) {
-            a.seg[k - i].w = *w[k];
-            a.seg[k - i].y = y[k];
-            a.total_rows += w[k]->ne1;
+            a.w[k - i] = *w[k];
+            a.y[k - i] = y[k];
+            a.seg_role[k - i] = k;
         }
-        a.xq = m->xq;
-        a.xf = xf;
-        a.resid = resid;
-        a.dbg_isc = nullptr;
-        a.dbg_imin = nullptr;
-        hipError_t e = k_matvec(s, a);
+        hipError_t e = k_matvec(s, a, PRO_RMSNORM, EPI_ROPE_KV);
         if (e != hipSuccess) return e;
         i = j;
     }
     return hipSuccess;
 }
 
+// x += wo * xb (:281-284); the prologue quantizes the attention output
+static hipError_t launch_wo(l2h_model *m, int l) {
+    PhaseArgs a = base_args(m);
+    a.nseg = 1;
+    a.w[0] = m->L(l, L2H_WO);
+    a.y[0] = m->x;
+    a.resid = m->x;
+    a.xf = m->xb;
+    return k_matvec(m->ctx->stream, a, PRO_QUANT, EPI_RESID);
+}
+
+// rmsnorm (:287) + w1, w3 (:291-292) + SwiGLU (:295-299) -> hb
+static hipError_t launch_w13(l2h_model *m, int l) {
+    hipStream_t s = m->ctx->stream;
+    const DevTensor &w1 = m->L(l, L2H_W1), &w3 = m->L(l, L2H_W3);
+    PhaseArgs a = base_args(m);
+    a.xf = m->x;
+    a.normw = m->L(l, L2H_RMS_FFN).f32;
+    if (w1.type == w3.type) {
+        a.nseg = 2;
+        a.w[0] = w1;
+        a.w[1] = w3;
+        a.y[0] = m->hb;
+        return k_matvec(s, a, PRO_RMSNORM, EPI_SWIGLU);
+    }
+    a.nseg = 1;
+    a.w[0] = w1;
+    a.y[0] = m->hb;
+    hipError_t e = k_matvec(s, a, PRO_RMSNORM, EPI_STORE);
+    if (e != hipSuccess) return e;
+    a.w[0] = w3;
+    a.y[0] = m->hb2;
+    e = k_matvec(s, a, PRO_RMSNORM, EPI_STORE);
+    if (e != hipSuccess) return e;
+    return k_swiglu(s, m->hb, m->hb2, m->c.hidden_dim);
+}
+
+// x += w2 * hb (:302-305)
+static hipError_t launch_w2(l2h_model *m, int l) {
+    PhaseArgs a = base_args(m);
+    a.nseg = 1;
+    a.w[0] = m->L(l, L2H_W2);
+    a.y[0] = m->x;
+    a.resid = m->x;
+    a.xf = m->hb;
+    return k_matvec(m->ctx->stream, a, PRO_QUANT, EPI_RESID);
+}
+
+// final rmsnorm (:309) + classifier (:312)
+static hipError_t launch_output(l2h_model *m) {
+    PhaseArgs a = base_args(m);
+    a.nseg = 1;
+    a.w[0] = m->glob[L2H_OUTPUT];
+    a.y[0] = m->logits;
+    a.xf = m->x;
+    a.normw = m->glob[L2H_RMS_FINAL].f32;
+    return k_matvec(m->ctx->stream, a, PRO_RMSNORM, EPI_STORE);
+}
+
 static hipError_t enqueue_token(l2h_model *m) {
     hipStream_t s = m->ctx->stream;
     const l2h_config &c = m->c;
     hipError_t e;
-#define CK(call)                  \
-    do {                          \
-        e = (call);               \
+#define CK(call)                       \
+    do {                               \
+        e = (call);                    \
         if (e != hipSuccess) return e; \
     } while (0)
-    CK(k_embed(s, m->glob[L2H_TOK_EMB], m->ctl, m->prompt_dev, m->x));
+    // token embedding (:236) and this position's RoPE table
+    CK(k_embed(s, m->glob[L2H_TOK_EMB], m->ctl, m->prompt_dev, m->x, m->rope_cs, m->hs, m->theta_scale));
     for (int l = 0; l < c.n_layers; l++) {
         float *kc = m->kc + (int64_t)l * m->cache_layer_elems;
         float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
-        const DevTensor &wq = m->L(l, L2H_WQ), &wk = m->L(l, L2H_WK), &wv = m->L(l, L2H_WV), &wo = m->L(l, L2H_WO),
-                        &w1 = m->L(l, L2H_W1), &w2 = m->L(l, L2H_W2), &w3 = m->L(l, L2H_W3);
-        // attention rmsnorm (:244) + q8_K image of xb for the k-quant consumers
-        CK(k_rmsnorm_quant(s, m->x, m->L(l, L2H_RMS_ATT).f32, m->xb, m->xq,
-                           is_kquant(wq.type) || is_kquant(wk.type) || is_kquant(wv.type), c.dim));
-        {  // q, k, v (:247-249)
-            const DevTensor *w[3] = {&wq, &wk, &wv};
-            float *y[3] = {m->q, m->k, m->v};
-            CK(launch_matvecs(m, w, y, 3, m->xb, nullptr));
-        }
-        // rope (:255-256) + cache append (:259-260)
-        CK(k_rope_kv(s, m->q, m->qd, m->k, m->v, kc, vc, m->ctl, m->hs, c.n_heads, c.n_kv_heads, c.seq_len,
-                     m->theta_scale, c.rope_is_neox));
-        // attention (:263-278) -> xb
-        CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->xq, is_kquant(wo.type), m->ctl, m->hs,
-                       c.n_heads, c.n_kv_heads, c.seq_len));
-        {  // x += wo * xb (:281-284)
-            const DevTensor *w[1] = {&wo};
-            float *y[1] = {m->x};
-            CK(launch_matvecs(m, w, y, 1, m->xb, m->x));
-        }
-        CK(k_rmsnorm_quant(s, m->x, m->L(l, L2H_RMS_FFN).f32, m->xb, m->xq, is_kquant(w1.type) || is_kquant(w3.type),
-                           c.dim));  // :287
-        {                            // hb = w1 xb, hb2 = w3 xb (:291-292)
-            const DevTensor *w[2] = {&w1, &w3};
-            float *y[2] = {m->hb, m->hb2};
-            CK(launch_matvecs(m, w, y, 2, m->xb, nullptr));
-        }
-        CK(k_swiglu_quant(s, m->hb, m->hb2, m->xq, is_kquant(w2.type), c.hidden_dim));  // :295-299
-        {                                                                               // x += w2 hb (:302-305)
-            const DevTensor *w[1] = {&w2};
-            float *y[1] = {m->x};
-            CK(launch_matvecs(m, w, y, 1, m->hb, m->x));
-        }
+        CK(launch_qkv(m, l));
+        CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->ctl, m->hs, c.n_heads, c.n_kv_heads,
+                       c.seq_len));  // :263-278 -> xb
+        CK(launch_wo(m, l));
+        CK(launch_w13(m, l));
+        CK(launch_w2(m, l));
     }
-    const DevTensor &wout = m->glob[L2H_OUTPUT];
-    CK(k_rmsnorm_quant(s, m->x, m->glob[L2H_RMS_FINAL].f32, m->x, m->xq, is_kquant(wout.type), c.dim));  // :309
-    {                                                                                                     // :312
-        const DevTensor *w[1] = {&wout};
-        float *y[1] = {m->logits};
-        CK(launch_matvecs(m, w, y, 1, m->x, nullptr));
-    }
+    CK(launch_output(m));
     CK(k_argmax(s, m->logits, c.vocab_size, m->argmax_partial, m->ctl, m->out_tokens, m->max_out));  // :360
 #undef CK
     return hipSuccess;
@@ -459,6 +496,7 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     DA(m->att, (int64_t)c.seq_len * c.n_heads, true);
     DA(m->logits, c.vocab_size, true);
     DA(m->qd, c.dim, true);
+    DA(m->rope_cs, m->hs, true);
     DA(m->pd, (int64_t)c.seq_len * c.n_heads, true);
     const int ntiles = (c.seq_len + L2H_ATT_TILE - 1) / L2H_ATT_TILE;
     DA(m->part, (int64_t)ntiles * c.dim, true);
@@ -471,8 +509,6 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     DA(m->out_tokens, m->max_out, true);
     DA(m->argmax_partial, L2H_ARGMAX_BLOCKS, true);
 #undef DA
-    const int64_t maxk = ((std::max(c.dim, c.hidden_dim) + 255) / 256) * 256;
-    if ((rc = q8_alloc(ctx, maxk, &m->xq, &m->allocs))) return rc;
     HIPCHK(ctx, hipDeviceSynchronize());
 
     // Record the launch sequence of one token; positions and tokens are read from the
@@ -630,8 +666,6 @@ extern "C" int l2h_state_read(l2h_model *m, int which, float *host, int64_t n) {
     case 0: src = m->x; len = m->c.dim; break;
     case 1: src = m->xb; len = m->c.dim; break;
     case 2: src = m->q; len = m->c.dim; break;
-    case 3: src = m->k; len = m->kv_dim; break;
-    case 4: src = m->v; len = m->kv_dim; break;
     case 5: src = m->hb; len = m->c.hidden_dim; break;
     case 6: src = m->logits; len = m->c.vocab_size; break;
     default: return set_err(m->ctx, L2H_EINVAL, "unknown state buffer %d", which);
@@ -685,7 +719,7 @@ extern "C" int l2h_quantize_q8k(l2h_ctx *ctx, const float *x, int64_t n, void *o
     std::vector<void *> tr;
     int rc = q8_alloc(ctx, n, &q, &tr);
     if (rc) return rc;
-    hipError_t e = k_quant_q8(ctx->stream, dx.as<float>(), q, n);
+    hipError_t e = k_stage_dump(ctx->stream, dx.as<float>(), nullptr, n, PRO_QUANT, q, nullptr);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess)
         rc = q8_pack_blocks(ctx, q, n, out_blocks);
@@ -733,10 +767,8 @@ extern "C" int l2h_matmul(l2h_ctx *ctx, int type, const void *A, int64_t ne0, in
     int rc = dev_tensor_alloc(ctx, type, ne0, ne1, &t);
     if (rc) return rc;
     rc = dev_tensor_upload(ctx, &t, A);
-    std::vector<void *> tr;
     if (rc == L2H_OK) {
         DevBuf dx, dy, di, dm;
-        Q8Dev q{nullptr, nullptr, nullptr};
         hipError_t e = dx.alloc((size_t)ne0 * 4);
         if (e == hipSuccess) e = dy.alloc((size_t)ne1 * 4);
         if (e == hipSuccess) e = hipMemcpy(dx.p, x, (size_t)ne0 * 4, hipMemcpyHostToDevice);
@@ -745,22 +777,16 @@ extern "C" int l2h_matmul(l2h_ctx *ctx, int type, const void *A, int64_t ne0, in
             e = di.alloc((size_t)nints * 4);
             if (e == hipSuccess) e = dm.alloc((size_t)nints * 4);
         }
-        if (e == hipSuccess && is_kquant(type)) {
-            rc = q8_alloc(ctx, ne0, &q, &tr);
-            if (rc == L2H_OK) e = k_quant_q8(ctx->stream, dx.as<float>(), q, ne0);
-        }
-        if (rc == L2H_OK && e == hipSuccess) {
-            MatvecArgs a{};
+        if (e == hipSuccess) {
+            PhaseArgs a{};
+            a.max_grid = ctx->prop.multiProcessorCount;
             a.nseg = 1;
-            a.seg[0].w = t;
-            a.seg[0].y = dy.as<float>();
-            a.total_rows = ne1;
-            a.xq = q;
+            a.w[0] = t;
+            a.y[0] = dy.as<float>();
             a.xf = dx.as<float>();
-            a.resid = nullptr;
             a.dbg_isc = di.as<int32_t>();
             a.dbg_imin = dm.as<int32_t>();
-            e = k_matvec(ctx->stream, a);
+            e = k_matvec(ctx->stream, a, PRO_QUANT, EPI_STORE);
         }
         if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
         if (e == hipSuccess) e = hipMemcpy(y, dy.p, (size_t)ne1 * 4, hipMemcpyDeviceToHost);
@@ -768,16 +794,15 @@ extern "C" int l2h_matmul(l2h_ctx *ctx, int type, const void *A, int64_t ne0, in
             e = hipMemcpy(I_sc, di.p, (size_t)nints * 4, hipMemcpyDeviceToHost);
             if (e == hipSuccess) e = hipMemcpy(I_min, dm.p, (size_t)nints * 4, hipMemcpyDeviceToHost);
         }
-        if (rc == L2H_OK && e != hipSuccess) rc = set_err(ctx, L2H_EHIP, "matmul failed: %s", hipGetErrorString(e));
+        if (e != hipSuccess) rc = set_err(ctx, L2H_EHIP, "matmul failed: %s", hipGetErrorString(e));
     }
-    for (void *p : tr) (void)hipFree(p);
     dev_tensor_free(&t);
     return rc;
 }
 
 extern "C" int l2h_rmsnorm(l2h_ctx *ctx, float *o, const float *x, const float *weight, int64_t n) {
     if (!ctx || !o || !x || !weight) return set_err(ctx, L2H_EINVAL, "l2h_rmsnorm: NULL argument");
-    if (n <= 0 || n > (1 << 30)) return set_err(ctx, L2H_EINVAL, "bad length");
+    if (n <= 0 || n > 15360) return set_err(ctx, L2H_EINVAL, "length %lld outside 1..15360", (long long)n);
     HIPCHK(ctx, hipSetDevice(ctx->device));
     DevBuf dx, dw, dout;
     HIPCHK(ctx, dx.alloc((size_t)n * 4));
@@ -786,10 +811,35 @@ extern "C" int l2h_rmsnorm(l2h_ctx *ctx, float *o, const float *x, const float *
     HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
     HIPCHK(ctx, hipMemcpy(dw.p, weight, (size_t)n * 4, hipMemcpyHostToDevice));
     Q8Dev none{nullptr, nullptr, nullptr};
-    HIPCHK(ctx, k_rmsnorm_quant(ctx->stream, dx.as<float>(), dw.as<float>(), dout.as<float>(), none, false, (int)n));
+    HIPCHK(ctx, k_stage_dump(ctx->stream, dx.as<float>(), dw.as<float>(), n, PRO_RMSNORM, none, dout.as<float>()));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(o, dout.p, (size_t)n * 4, hipMemcpyDeviceToHost));
     return L2H_OK;
+}
+
+// rmsnorm!(o, x, weight) followed by q8_K quantization of o, as the matvec prologue does it
+extern "C" int l2h_rmsnorm_q8k(l2h_ctx *ctx, const float *x, const float *weight, int64_t n, void *out_blocks) {
+    if (!ctx || !x || !weight || !out_blocks) return set_err(ctx, L2H_EINVAL, "l2h_rmsnorm_q8k: NULL argument");
+    if (n <= 0 || n % QK_K != 0 || n > 15360)
+        return set_err(ctx, L2H_EINVAL, "length %lld must be a multiple of 256, at most 15360", (long long)n);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf dx, dw;
+    HIPCHK(ctx, dx.alloc((size_t)n * 4));
+    HIPCHK(ctx, dw.alloc((size_t)n * 4));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)n * 4, hipMemcpyHostToDevice));
+    HIPCHK(ctx, hipMemcpy(dw.p, weight, (size_t)n * 4, hipMemcpyHostToDevice));
+    Q8Dev q;
+    std::vector<void *> tr;
+    int rc = q8_alloc(ctx, n, &q, &tr);
+    if (rc) return rc;
+    hipError_t e = k_stage_dump(ctx->stream, dx.as<float>(), dw.as<float>(), n, PRO_RMSNORM, q, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
+    if (e == hipSuccess)
+        rc = q8_pack_blocks(ctx, q, n, out_blocks);
+    else
+        rc = set_err(ctx, L2H_EHIP, "rmsnorm+quantize failed: %s", hipGetErrorString(e));
+    (void)hipFree(tr[0]);
+    return rc;
 }
 
 extern "C" int l2h_rope(l2h_ctx *ctx, float *x, int head_size, int n_heads, int pos, float freq_base, int neox) {
@@ -853,10 +903,9 @@ extern "C" int l2h_attention(l2h_ctx *ctx, float *out, const float *q, const flo
     HIPCHK(ctx, k_f32_to_f64(ctx->stream, dq.as<float>(), dqd.as<double>(), dim));
     HIPCHK(ctx, k_kv_layout(ctx->stream, dkc.as<float>(), dvc.as<float>(), dkl.as<float>(), dvl.as<float>(), 0, np,
                             head_size, n_kv_heads, seq_len, true));
-    Q8Dev none{nullptr, nullptr, nullptr};
     HIPCHK(ctx, k_attention(ctx->stream, dqd.as<double>(), dkc.as<float>(), dvc.as<float>(), datt.as<float>(),
-                            dpd.as<double>(), dpart.as<double>(), dout.as<float>(), none, false,
-                            (const DecodeCtl *)dctl.p, head_size, n_heads, n_kv_heads, seq_len));
+                            dpd.as<double>(), dpart.as<double>(), dout.as<float>(), (const DecodeCtl *)dctl.p,
+                            head_size, n_heads, n_kv_heads, seq_len));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(out, dout.p, (size_t)dim * 4, hipMemcpyDeviceToHost));
     return L2H_OK;
@@ -871,8 +920,7 @@ extern "C" int l2h_swiglu(l2h_ctx *ctx, float *hb, const float *hb2, int64_t n) 
     HIPCHK(ctx, b.alloc((size_t)n * 4));
     HIPCHK(ctx, hipMemcpy(a.p, hb, (size_t)n * 4, hipMemcpyHostToDevice));
     HIPCHK(ctx, hipMemcpy(b.p, hb2, (size_t)n * 4, hipMemcpyHostToDevice));
-    Q8Dev none{nullptr, nullptr, nullptr};
-    HIPCHK(ctx, k_swiglu_quant(ctx->stream, a.as<float>(), b.as<float>(), none, false, (int)n));
+    HIPCHK(ctx, k_swiglu(ctx->stream, a.as<float>(), b.as<float>(), (int)n));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(hb, a.p, (size_t)n * 4, hipMemcpyDeviceToHost));
     return L2H_OK;
@@ -905,25 +953,21 @@ extern "C" int l2h_profile_matvec(l2h_model *m, int role, int iters, float *avg_
     l2h_ctx *ctx = m->ctx;
     if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
     if (iters < 1) return set_err(ctx, L2H_EINVAL, "iters must be >= 1");
-    const int roles_qkv[3] = {L2H_WQ, L2H_WK, L2H_WV}, roles_13[2] = {L2H_W1, L2H_W3};
-    const int *roles;
-    int nr;
-    int single = role;
-    float *ys[3];
-    if (role == L2H_WQ) {
-        roles = roles_qkv; nr = 3; ys[0] = m->q; ys[1] = m->k; ys[2] = m->v;
-    } else if (role == L2H_W1) {
-        roles = roles_13; nr = 2; ys[0] = m->hb; ys[1] = m->hb2;
-    } else if (role == L2H_WO || role == L2H_W2 || role == L2H_OUTPUT) {
-        roles = &single; nr = 1; ys[0] = role == L2H_OUTPUT ? m->logits : m->xb2;
-    } else {
+    if (role != L2H_WQ && role != L2H_WO && role != L2H_W1 && role != L2H_W2 && role != L2H_OUTPUT)
         return set_err(ctx, L2H_EINVAL, "role %d has no matvec launch of its own", role);
-    }
     HIPCHK(ctx, hipSetDevice(ctx->device));
-    // a defined input: zeros quantize to zero blocks, timing does not depend on values
+    DecodeCtl h{};  // position 0: the q/k/v launch appends to cache row 0
+    HIPCHK(ctx, hipMemcpy(m->ctl, &h, sizeof h, hipMemcpyHostToDevice));
     const int n_layers = role == L2H_OUTPUT ? 1 : m->c.n_layers;
     int64_t b = 0;
-    int launches_per_pass = 0;
+    if (role == L2H_WQ)
+        b = m->L(0, L2H_WQ).gguf_bytes + m->L(0, L2H_WK).gguf_bytes + m->L(0, L2H_WV).gguf_bytes;
+    else if (role == L2H_W1)
+        b = m->L(0, L2H_W1).gguf_bytes + m->L(0, L2H_W3).gguf_bytes;
+    else if (role == L2H_OUTPUT)
+        b = m->glob[L2H_OUTPUT].gguf_bytes;
+    else
+        b = m->L(0, role).gguf_bytes;
     hipEvent_t e0, e1;
     HIPCHK(ctx, hipEventCreate(&e0));
     HIPCHK(ctx, hipEventCreate(&e1));
@@ -931,17 +975,16 @@ extern "C" int l2h_profile_matvec(l2h_model *m, int role, int iters, float *avg_
         const int reps = pass == 0 ? 1 : iters;
         if (pass == 1) HIPCHK(ctx, hipEventRecord(e0, ctx->stream));
         for (int it = 0; it < reps; it++) {
-            launches_per_pass = 0;
             for (int l = 0; l < n_layers; l++) {
-                const DevTensor *w[3];
-                b = 0;
-                for (int k = 0; k < nr; k++) {
-                    w[k] = role == L2H_OUTPUT ? &m->glob[L2H_OUTPUT] : &m->L(l, roles[k]);
-                    b += w[k]->gguf_bytes;
+                hipError_t e;
+                switch (role) {
+                case L2H_WQ: e = launch_qkv(m, l); break;
+                case L2H_WO: e = launch_wo(m, l); break;
+                case L2H_W1: e = launch_w13(m, l); break;
+                case L2H_W2: e = launch_w2(m, l); break;
+                default: e = launch_output(m); break;
                 }
-                hipError_t e = launch_matvecs(m, w, ys, nr, m->xb, nullptr);
                 if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "matvec launch failed: %s", hipGetErrorString(e));
-                launches_per_pass++;
             }
         }
         if (pass == 1) HIPCHK(ctx, hipEventRecord(e1, ctx->stream));
@@ -951,7 +994,7 @@ extern "C" int l2h_profile_matvec(l2h_model *m, int role, int iters, float *avg_
     HIPCHK(ctx, hipEventElapsedTime(&ms, e0, e1));
     (void)hipEventDestroy(e0);
     (void)hipEventDestroy(e1);
-    *avg_us = ms * 1000.0f / (float)(iters * launches_per_pass);
+    *avg_us = ms * 1000.0f / (float)(iters * n_layers);
     if (bytes) *bytes = b;
     return L2H_OK;
 }

@@ -75,60 +75,6 @@ __device__ __forceinline__ void kq_scale_min(const uint4 hdr, int s, int &sc, in
     m = (s & 1) ? mb : ma;
 }
 
-// ------------------------------------------------------------------------------------------
-// q8_K quantization of 256 values held by 16 consecutive lanes, 16 values each (lane `sub`
-// of the group holds elements 16*sub .. 16*sub+15).  llama.cpp's quantize_row_q8_K rule:
-// the FIRST element of largest magnitude fixes the scale (ties go to the lowest index),
-// iscale = -127/max, q = min(127, round-half-even(iscale*x)), d = 1/iscale.
-// Returns the 16 quants packed in a uint4, their sum, and d (same on all 16 lanes).
-// ------------------------------------------------------------------------------------------
-__device__ __forceinline__ void q8k_quantize_group(const float v[16], int sub, uint4 &packed, int &bsum, float &d) {
-    float amax = 0.0f, mx = 0.0f;
-#pragma unroll
-    for (int k = 0; k < 16; k++) {
-        const float ax = fabsf(v[k]);
-        if (ax > amax) {
-            amax = ax;
-            mx = v[k];
-        }
-    }
-#pragma unroll
-    for (int m = 1; m < 16; m <<= 1) {
-        const float oa = __shfl_xor(amax, m, WAVE), om = __shfl_xor(mx, m, WAVE);
-        const bool other_is_lower = (sub & m) != 0;
-        // combine(lower range, upper range): the upper one wins only if strictly larger
-        const bool take_other = other_is_lower ? !(amax > oa) : (oa > amax);
-        if (take_other) {
-            amax = oa;
-            mx = om;
-        }
-    }
-    if (amax == 0.0f) {
-        packed = make_uint4(0, 0, 0, 0);
-        bsum = 0;
-        d = 0.0f;
-        return;
-    }
-    const float iscale = -127.0f / mx;
-    uint32_t w[4];
-    int sum = 0;
-#pragma unroll
-    for (int k4 = 0; k4 < 4; k4++) {
-        uint32_t word = 0;
-#pragma unroll
-        for (int b = 0; b < 4; b++) {
-            int q = (int)rintf(iscale * v[4 * k4 + b]);
-            q = q < 127 ? q : 127;
-            sum += (int)(int8_t)q;
-            word |= ((uint32_t)(q & 0xFF)) << (8 * b);
-        }
-        w[k4] = word;
-    }
-    packed = make_uint4(w[0], w[1], w[2], w[3]);
-    bsum = sum;
-    d = 1.0f / iscale;
-}
-
 // Weight value of element e (0..ne0) of row `row`, formed with the reference's fp32
 // expressions (src/kquants.jl:93,97 q4_K; :213,217 q5_K; :340-343 q6_K).
 __device__ __forceinline__ float dequant_elem(const DevTensor &t, int64_t row, int64_t e) {

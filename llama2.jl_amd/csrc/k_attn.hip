@@ -125,17 +125,10 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
 }
 
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
-                       double *part, float *out, Q8Dev q8, bool do_q8, const DecodeCtl *ctl, int head_size,
-                       int n_heads, int n_kv_heads, int seq_len) {
+                       double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads,
+                       int seq_len) {
     const int G = n_heads / n_kv_heads;
-    hipError_t e;
-    if (G % 4 == 0)
-        e = launch_attn<4>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    else if (G % 2 == 0)
-        e = launch_attn<2>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    else
-        e = launch_attn<1>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    if (e != hipSuccess) return e;
-    if (do_q8) e = k_quant_q8(s, out, q8, (int64_t)head_size * n_heads);
-    return e;
+    if (G % 4 == 0) return launch_attn<4>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    if (G % 2 == 0) return launch_attn<2>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    return launch_attn<1>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
 }

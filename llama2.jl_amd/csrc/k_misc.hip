@@ -73,15 +73,25 @@ hipError_t k_repack(hipStream_t s, const DevTensor &t, const void *raw_dev, bool
 // (src/inference.jl:354-360,385).
 // ------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void embed_kernel(DevTensor emb, const DecodeCtl *ctl, const int32_t *prompt,
-                                                    float *x) {
+                                                    float *x, float *rope_cs, int hs, float theta_scale) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (blockIdx.x == 0 && threadIdx.x < (hs >> 1)) {
+        // cos/sin of this position's RoPE angles, shared by all layers and heads: theta_i is
+        // fp32(pos) advanced by i fp32 multiplications (reference src/inference.jl:122-127)
+        float theta = 1.0f * (float)ctl->pos;
+        for (int k = 0; k < (int)threadIdx.x; k++) theta *= theta_scale;
+        rope_cs[2 * threadIdx.x] = (float)cos((double)theta);
+        rope_cs[2 * threadIdx.x + 1] = (float)sin((double)theta);
+    }
     if (i >= emb.ne0) return;
     const int tok = ctl->step < ctl->n_prompt ? prompt[ctl->step] : ctl->last_argmax;
     x[i] = dequant_elem(emb, tok, i);
 }
 
-hipError_t k_embed(hipStream_t s, const DevTensor &emb, const DecodeCtl *ctl, const int32_t *prompt, float *x) {
-    hipLaunchKernelGGL(embed_kernel, dim3((unsigned)((emb.ne0 + 255) / 256)), dim3(256), 0, s, emb, ctl, prompt, x);
+hipError_t k_embed(hipStream_t s, const DevTensor &emb, const DecodeCtl *ctl, const int32_t *prompt, float *x,
+                   float *rope_cs, int head_size, float theta_scale) {
+    hipLaunchKernelGGL(embed_kernel, dim3((unsigned)((emb.ne0 + 255) / 256)), dim3(256), 0, s, emb, ctl, prompt, x,
+                       rope_cs, head_size, theta_scale);
     return hipGetLastError();
 }
 
@@ -98,135 +108,26 @@ hipError_t k_dequant(hipStream_t s, const DevTensor &t, int64_t row0, int64_t nr
 }
 
 // ------------------------------------------------------------------------------------------
-// rmsnorm!(o, x, weight) (reference src/inference.jl:102-110) fused with the q8_K
-// quantization of o.  One workgroup: the sum of squares spans the whole vector.
-//   ss = fp32(sum_fp64 x*x); ss /= n; ss += 1e-5; ss = 1/sqrt(ss); o = w * (ss * x)
-// ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void rmsnorm_quant_kernel(const float *x, const float *w, float *o, Q8Dev q8,
-                                                             int do_q8, int n) {
-    __shared__ double red[16];
-    const int tid = threadIdx.x;
-    double acc = 0.0;
-    for (int i = tid; i < n; i += blockDim.x) {
-        const double v = (double)x[i];
-        acc = fma(v, v, acc);
-    }
-    float ss = (float)block_sum_f64(acc, red);
-    ss /= (float)n;
-    ss += 1e-5f;
-    ss = 1.0f / sqrtf(ss);
-    if (!do_q8) {
-        for (int i = tid; i < n; i += blockDim.x) o[i] = w[i] * (ss * x[i]);
-        return;
-    }
-    // n % 256 == 0: 16 lanes per q8_K block, 16 consecutive elements per lane
-    for (int base = 16 * tid; base < n; base += 16 * blockDim.x) {
-        float v[16];
-#pragma unroll
-        for (int k4 = 0; k4 < 4; k4++) {
-            const float4 xv = *(const float4 *)(x + base + 4 * k4);
-            const float4 wv = *(const float4 *)(w + base + 4 * k4);
-            v[4 * k4 + 0] = wv.x * (ss * xv.x);
-            v[4 * k4 + 1] = wv.y * (ss * xv.y);
-            v[4 * k4 + 2] = wv.z * (ss * xv.z);
-            v[4 * k4 + 3] = wv.w * (ss * xv.w);
-        }
-#pragma unroll
-        for (int k4 = 0; k4 < 4; k4++)
-            *(float4 *)(o + base + 4 * k4) = make_float4(v[4 * k4], v[4 * k4 + 1], v[4 * k4 + 2], v[4 * k4 + 3]);
-        uint4 packed;
-        int bsum;
-        float d;
-        q8k_quantize_group(v, tid & 15, packed, bsum, d);
-        *(uint4 *)(q8.qs + base) = packed;
-        q8.bsums[base >> 4] = (int16_t)bsum;
-        if ((tid & 15) == 0) q8.d[base >> 8] = d;
-    }
-}
-
-hipError_t k_rmsnorm_quant(hipStream_t s, const float *x, const float *w, float *o, Q8Dev q8, bool do_q8, int n) {
-    hipLaunchKernelGGL(rmsnorm_quant_kernel, dim3(1), dim3(1024), 0, s, x, w, o, q8, do_q8 ? 1 : 0, n);
-    return hipGetLastError();
-}
-
-// q8_K quantization of a plain fp32 vector, n % 256 == 0.
-__global__ __launch_bounds__(256) void quant_q8_kernel(const float *x, Q8Dev q8, int64_t n) {
-    const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t base = 16 * t;
-    if (base >= n) return;  // uniform per 16-lane group since n % 256 == 0
-    float v[16];
-#pragma unroll
-    for (int k4 = 0; k4 < 4; k4++) {
-        const float4 xv = *(const float4 *)(x + base + 4 * k4);
-        v[4 * k4 + 0] = xv.x;
-        v[4 * k4 + 1] = xv.y;
-        v[4 * k4 + 2] = xv.z;
-        v[4 * k4 + 3] = xv.w;
-    }
-    uint4 packed;
-    int bsum;
-    float d;
-    q8k_quantize_group(v, threadIdx.x & 15, packed, bsum, d);
-    *(uint4 *)(q8.qs + base) = packed;
-    q8.bsums[base >> 4] = (int16_t)bsum;
-    if ((threadIdx.x & 15) == 0) q8.d[base >> 8] = d;
-}
-
-hipError_t k_quant_q8(hipStream_t s, const float *x, Q8Dev q8, int64_t n) {
-    const int64_t threads = n / 16;
-    hipLaunchKernelGGL(quant_q8_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, x, q8, n);
-    return hipGetLastError();
-}
-
-// ------------------------------------------------------------------------------------------
 // hb[i] = hb[i] * (1/(1+exp(-hb[i]))) * hb2[i]  (reference src/inference.jl:295-299),
-// exp evaluated in fp64 and rounded to fp32; optionally followed by q8_K quantization.
+// exp evaluated in fp64 and rounded to fp32.  Stand-alone form, used when w1 and w3 differ in
+// type and cannot share one launch.
 // ------------------------------------------------------------------------------------------
-__device__ __forceinline__ float swiglu_one(float a, float b) {
+__global__ __launch_bounds__(256) void swiglu_kernel(float *hb, const float *hb2, int n) {
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n) return;
+    const float a = hb[t];
     const float e = (float)exp((double)(-a));
     const float v = a * (1.0f / (1.0f + e));
-    return v * b;
+    hb[t] = v * hb2[t];
 }
 
-__global__ __launch_bounds__(256) void swiglu_quant_kernel(float *hb, const float *hb2, Q8Dev q8, int do_q8, int n) {
-    const int t = blockIdx.x * blockDim.x + threadIdx.x;
-    if (!do_q8) {
-        if (t < n) hb[t] = swiglu_one(hb[t], hb2[t]);
-        return;
-    }
-    const int base = 16 * t;
-    if (base >= n) return;
-    float v[16];
-#pragma unroll
-    for (int k4 = 0; k4 < 4; k4++) {
-        const float4 a = *(const float4 *)(hb + base + 4 * k4);
-        const float4 b = *(const float4 *)(hb2 + base + 4 * k4);
-        v[4 * k4 + 0] = swiglu_one(a.x, b.x);
-        v[4 * k4 + 1] = swiglu_one(a.y, b.y);
-        v[4 * k4 + 2] = swiglu_one(a.z, b.z);
-        v[4 * k4 + 3] = swiglu_one(a.w, b.w);
-    }
-#pragma unroll
-    for (int k4 = 0; k4 < 4; k4++)
-        *(float4 *)(hb + base + 4 * k4) = make_float4(v[4 * k4], v[4 * k4 + 1], v[4 * k4 + 2], v[4 * k4 + 3]);
-    uint4 packed;
-    int bsum;
-    float d;
-    q8k_quantize_group(v, threadIdx.x & 15, packed, bsum, d);
-    *(uint4 *)(q8.qs + base) = packed;
-    q8.bsums[base >> 4] = (int16_t)bsum;
-    if ((threadIdx.x & 15) == 0) q8.d[base >> 8] = d;
-}
-
-hipError_t k_swiglu_quant(hipStream_t s, float *hb, const float *hb2, Q8Dev q8, bool do_q8, int n) {
-    const int threads = do_q8 ? n / 16 : n;
-    hipLaunchKernelGGL(swiglu_quant_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, hb, hb2, q8,
-                       do_q8 ? 1 : 0, n);
+hipError_t k_swiglu(hipStream_t s, float *hb, const float *hb2, int n) {
+    hipLaunchKernelGGL(swiglu_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, hb, hb2, n);
     return hipGetLastError();
 }
 
 // ------------------------------------------------------------------------------------------
-// rope!(q), rope!(k) (reference src/inference.jl:112-167) + KV append (:259-260).
+// rope!(x) (reference src/inference.jl:112-167), stand-alone form.
 // theta of pair i is fp32(pos) advanced by i fp32 multiplications with theta_scale
 // (:122-127); cos/sin are evaluated in fp64 and rounded to fp32; the complex product
 // rounds each of its four products (Complex{Float32} multiplication).
@@ -244,46 +145,6 @@ __device__ __forceinline__ void rope_pair(float a, float b, int i, int pos, floa
 
 __device__ __forceinline__ int64_t kc_index(int kvh, int i, int t, int hs, int seq_len) {
     return (((int64_t)kvh * (hs >> 2) + (i >> 2)) * seq_len + t) * 4 + (i & 3);
-}
-
-__global__ __launch_bounds__(256) void rope_kv_kernel(float *q, double *qd, const float *k, const float *v, float *kc,
-                                                      float *vc, const DecodeCtl *ctl, int hs, int n_heads,
-                                                      int n_kv_heads, int seq_len, float theta_scale, int neox) {
-    const int gid = blockIdx.x * blockDim.x + threadIdx.x;
-    const int half = hs >> 1;
-    const int nq = n_heads * half, nk = n_kv_heads * half, nv = n_kv_heads * hs;
-    const int pos = ctl->pos;
-    if (gid < nq + nk) {
-        const bool is_q = gid < nq;
-        const int p = is_q ? gid : gid - nq;
-        const int h = p / half, i = p % half;
-        const int e0 = neox ? i : 2 * i, e1 = neox ? half + i : 2 * i + 1;
-        const float *src = is_q ? q : k;
-        float re, im;
-        rope_pair(src[h * hs + e0], src[h * hs + e1], i, pos, theta_scale, re, im);
-        if (is_q) {
-            q[h * hs + e0] = re;
-            q[h * hs + e1] = im;
-            qd[h * hs + e0] = (double)re;
-            qd[h * hs + e1] = (double)im;
-        } else {
-            kc[kc_index(h, e0, pos, hs, seq_len)] = re;
-            kc[kc_index(h, e1, pos, hs, seq_len)] = im;
-        }
-    } else if (gid < nq + nk + nv) {
-        const int e = gid - nq - nk;
-        const int h = e / hs, i = e % hs;
-        vc[((int64_t)h * seq_len + pos) * hs + i] = v[e];
-    }
-}
-
-hipError_t k_rope_kv(hipStream_t s, float *q, double *qd, const float *k, const float *v, float *kc, float *vc,
-                     const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads, int seq_len,
-                     float theta_scale, int neox) {
-    const int total = n_heads * head_size / 2 + n_kv_heads * head_size / 2 + n_kv_heads * head_size;
-    hipLaunchKernelGGL(rope_kv_kernel, dim3((total + 255) / 256), dim3(256), 0, s, q, qd, k, v, kc, vc, ctl,
-                       head_size, n_heads, n_kv_heads, seq_len, theta_scale, neox);
-    return hipGetLastError();
 }
 
 __global__ __launch_bounds__(256) void rope_only_kernel(float *x, int hs, int n_heads, int pos, float theta_scale,

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <algorithm>
 #include <string>
 #include <vector>
 
@@ -59,38 +60,51 @@ struct DecodeCtl {
     int32_t pad[2];
 };
 
-// One matvec launch covers up to 3 weight matrices that consume the same input vector.
-struct MatvecSeg {
-    DevTensor w;
-    float *y;        // output rows of this segment
-};
-struct MatvecArgs {
-    MatvecSeg seg[3];
+// One matvec launch covers up to 3 weight matrices of one type that consume the same input
+// vector, with a fused prologue (how the activations reach LDS) and epilogue.
+enum { PRO_Q8 = 0, PRO_QUANT = 1, PRO_RMSNORM = 2 };
+enum { EPI_STORE = 0, EPI_RESID = 1, EPI_SWIGLU = 2, EPI_ROPE_KV = 3 };
+enum { SEG_Q = 0, SEG_K = 1, SEG_V = 2 };
+struct PhaseArgs {
+    DevTensor w[3];
+    float *y[3];           // STORE/RESID: output rows of each segment; SWIGLU: y[0] = hb; ROPE_KV: q rows
     int nseg;
-    int64_t total_rows;
-    Q8Dev xq;              // k-quant input
-    const float *xf;       // F32 input
-    const float *resid;    // epilogue: y = resid + result (may equal y), or nullptr
-    int32_t *dbg_isc;      // debug: per (row, block) integer sums, or nullptr
-    int32_t *dbg_imin;
+    int seg_role[3];       // ROPE_KV: SEG_Q / SEG_K / SEG_V
+    // filled by k_matvec: logical rows in total and per workgroup (even), tile shape
+    int64_t n_rows;
+    int rows_per_wg, rt, st, ntpr;
+    int max_grid;          // workgroups to use at most (number of compute units)
+    Q8Dev xq;              // PRO_Q8: quantized input
+    const float *xf;       // PRO_QUANT / PRO_RMSNORM: fp32 input
+    const float *normw;    // PRO_RMSNORM: norm weights
+    const float *resid;    // EPI_RESID: y = resid + result (may alias y)
+    // EPI_ROPE_KV
+    const float *rope_cs;  // [hs/2][2] cos, sin of the current position
+    double *qd;            // rotated q widened to fp64
+    float *kc, *vc;        // this layer's caches
+    const DecodeCtl *ctl;
+    int hs, seq_len, neox;
+    // debug: per (row, block) integer sums (EPI_STORE only), or nullptr
+    int32_t *dbg_isc, *dbg_imin;
+    int64_t dbg_row0[3];
+#ifdef L2H_TIMELINE
+    long long *timeline;   // profiling build only: [workgroup][8] wall-clock stamps
+#endif
 };
 
 // ---- launchers (kernel files) ----------------------------------------------------------------
 // Each returns hipGetLastError() of its launch.
 hipError_t k_repack(hipStream_t s, const DevTensor &t, const void *raw_dev, bool inverse, void *raw_out);
-hipError_t k_embed(hipStream_t s, const DevTensor &emb, const DecodeCtl *ctl, const int32_t *prompt, float *x);
+hipError_t k_embed(hipStream_t s, const DevTensor &emb, const DecodeCtl *ctl, const int32_t *prompt, float *x,
+                   float *rope_cs, int head_size, float theta_scale);
 hipError_t k_dequant(hipStream_t s, const DevTensor &t, int64_t row0, int64_t nrows, float *y);
-hipError_t k_rmsnorm_quant(hipStream_t s, const float *x, const float *w, float *o, Q8Dev q8, bool do_q8, int n);
-hipError_t k_quant_q8(hipStream_t s, const float *x, Q8Dev q8, int64_t n);
-hipError_t k_swiglu_quant(hipStream_t s, float *hb, const float *hb2, Q8Dev q8, bool do_q8, int n);
-hipError_t k_matvec(hipStream_t s, const MatvecArgs &a);
-hipError_t k_rope_kv(hipStream_t s, float *q, double *qd, const float *k, const float *v, float *kc, float *vc,
-                     const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads, int seq_len,
-                     float theta_scale, int neox);
+hipError_t k_swiglu(hipStream_t s, float *hb, const float *hb2, int n);
+hipError_t k_matvec(hipStream_t s, PhaseArgs a, int pro, int epi);
+hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64_t n, int pro, Q8Dev q8_out, float *f32_out);
 hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
-                       double *part, float *out, Q8Dev q8, bool do_q8, const DecodeCtl *ctl, int head_size,
-                       int n_heads, int n_kv_heads, int seq_len);
+                       double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads,
+                       int seq_len);
 hipError_t k_softmax(hipStream_t s, float *x, int64_t n);
 hipError_t k_argmax(hipStream_t s, const float *x, int64_t n, int64_t *partial, DecodeCtl *ctl, int32_t *out_tokens,
                     int max_out);

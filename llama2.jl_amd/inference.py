@@ -146,13 +146,12 @@ class DeviceModel:
         self.ctx.check(_lib.lib().l2h_model_get_tensor(self.handle, role, layer, _lib.ptr(out), nbytes))
         return out
 
-    _STATE = {"x": 0, "xb": 1, "q": 2, "k": 3, "v": 4, "hb": 5, "logits": 6}
+    _STATE = {"x": 0, "xb": 1, "q": 2, "hb": 5, "logits": 6}
 
     def state(self, name):
         c = self.config
         kv_dim = c.dim // c.n_heads * c.n_kv_heads
-        n = {"x": c.dim, "xb": c.dim, "q": c.dim, "k": kv_dim, "v": kv_dim, "hb": c.hidden_dim,
-             "logits": c.vocab_size}[name]
+        n = {"x": c.dim, "xb": c.dim, "q": c.dim, "hb": c.hidden_dim, "logits": c.vocab_size}[name]
         out = np.empty(n, np.float32)
         self.ctx.check(_lib.lib().l2h_state_read(self.handle, self._STATE[name], _lib.ptr(out), n))
         return out

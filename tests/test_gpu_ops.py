@@ -122,6 +122,18 @@ def test_rmsnorm(pkg, orc, ctx, rng, n):
     assert _rel(o, closed.astype(np.float32)) <= 1e-5
 
 
+@pytest.mark.parametrize("n", [256, 4096, 14336])
+def test_rmsnorm_then_q8k_bit_exact(pkg, orc, ctx, rng, n):
+    """The matvec prologue: rmsnorm then q8_K quantization, block for block."""
+    from llama2_jl_amd import _lib, kquants
+    x = (rng.standard_normal(n) * 2).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, n).astype(np.float32)
+    got = np.zeros(n // 256, kquants.block_q8_K)
+    ctx.check(_lib.lib().l2h_rmsnorm_q8k(ctx.handle, _lib.ptr(x), _lib.ptr(w), n, _lib.ptr(got)))
+    want = orc.quantize_q8_K(orc.rmsnorm(x, w, orc.GPU_SPEC))
+    assert got.tobytes() == want.tobytes()
+
+
 @pytest.mark.parametrize("hs,neox,base", [(64, 0, 10000.0), (128, 0, 500000.0), (96, 1, 10000.0)])
 @pytest.mark.parametrize("pos", [0, 1, 17, 4095])
 def test_rope(pkg, orc, ctx, rng, hs, neox, base, pos):
