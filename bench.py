@@ -49,6 +49,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="8b-q4ks", choices=sorted(WORKLOADS))
     ap.add_argument("--repeats", type=int, default=3, help="timed regions; the median is reported")
+    ap.add_argument("--path", type=int, default=0, help="0 auto, 1 kernel per phase, 2 persistent kernel")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -73,9 +74,9 @@ def main():
                                share_classifier=(plan_name == "PLAN_F32"))
     log("model generated + quantized on %d host threads in %.1f s" % (synth._threads(), time.time() - t0))
     t0 = time.time()
-    dev = lm.device()
+    dev = lm.device(path=args.path)
     ctx.sync()
-    log("uploaded in %.1f s" % (time.time() - t0))
+    log("uploaded in %.1f s; launch path %d (1 = kernel per phase, 2 = persistent kernel)" % (time.time() - t0, dev.path))
 
     w_bytes = synth.weight_bytes_per_token(lm)
     kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads
@@ -158,7 +159,7 @@ def main():
         "dtype": "int8 dot products (q4_K/q6_K x q8_K), fp64 accumulation, fp32 activations",
         "data": "synthetic",
         "config": {"workload": args.workload, "shape": kw, "plan": plan_name, "prompt_tokens": n_prompt,
-                   "decode_positions": [pos0, pos0 + K - 1], "repeats": args.repeats,
+                   "decode_positions": [pos0, pos0 + K - 1], "repeats": args.repeats, "launch_path": dev.path,
                    "bytes_per_token": int(bytes_per_token), "weight_bytes_per_token": int(w_bytes),
                    "roofline_tok_s_at_8TBs": round(roofline_tok_s, 1),
                    "frac_of_roofline": round(tok_s / roofline_tok_s, 4),

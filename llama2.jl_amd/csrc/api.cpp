@@ -120,7 +120,7 @@ static int dev_tensor_upload(l2h_ctx *ctx, DevTensor *t, const void *host) {
 
 static int dev_tensor_download(l2h_ctx *ctx, const DevTensor *t, void *host) {
     if (t->type == L2H_TYPE_F32) {
-        HIPCHK(ctx, hipMemcpy(host, t->base, (size_t)t->gguf_bytes, hipMemcpyDeviceToHost));
+        HIPCHK(ctx, hipMemcpy(host, t->f32, (size_t)t->gguf_bytes, hipMemcpyDeviceToHost));
         return L2H_OK;
     }
     void *raw = nullptr;
@@ -193,6 +193,9 @@ extern "C" int l2h_device_info(l2h_ctx *ctx, char *name, int name_cap, int32_t *
 // ------------------------------------------------------------------------------------------
 // model
 // ------------------------------------------------------------------------------------------
+struct l2h_model;
+static l2h_model *g_bound_model = nullptr;  // whose phase arguments the persistent kernel's constant memory holds
+
 struct l2h_model {
     l2h_ctx *ctx = nullptr;
     l2h_config c{};
@@ -214,6 +217,18 @@ struct l2h_model {
     int max_out = 0;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
+    // persistent decode kernel
+    int path_request = 0;  // 0 auto, 1 one kernel per phase, 2 persistent kernel required
+    bool mega = false;
+    PhaseArgs mega_ph[5];  // q/k/v, wo, w1+w3, w2 of layer 0 and the classifier, planned for the persistent grid
+    GridBar *bar = nullptr;
+    unsigned long long bar_gen = 0;
+    int mega_grid = 0;
+    size_t mega_lds = 0;
+    int mega_types[5] = {0, 0, 0, 0, 0};
+#ifdef L2H_TIMELINE
+    long long *timeline = nullptr, *timeline2 = nullptr;
+#endif
     std::vector<void *> allocs;
 
     DevTensor &L(int layer_idx, int role) { return layer[(size_t)layer_idx * L2H_N_ROLES + role]; }
@@ -266,6 +281,7 @@ static void model_free_state(l2h_model *m) {
 
 extern "C" void l2h_model_destroy(l2h_model *m) {
     if (!m) return;
+    if (g_bound_model == m) g_bound_model = nullptr;
     (void)hipStreamSynchronize(m->ctx->stream);
     model_free_state(m);
     for (auto &t : m->glob) dev_tensor_free(&t);
@@ -321,12 +337,22 @@ extern "C" int l2h_model_set_tensor(l2h_model *m, int role, int layer, int type,
     return rc;
 }
 
+extern "C" int l2h_model_set_path(l2h_model *m, int path) {
+    if (!m) return L2H_EINVAL;
+    if (m->finalized) return set_err(m->ctx, L2H_ESTATE, "model already finalized");
+    if (path < 0 || path > 2) return set_err(m->ctx, L2H_EINVAL, "path must be 0, 1 or 2");
+    m->path_request = path;
+    return L2H_OK;
+}
+
+extern "C" int l2h_model_path(l2h_model *m) { return (m && m->finalized) ? (m->mega ? 2 : 1) : 0; }
+
 extern "C" int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t host_bytes) {
     if (!m || !host) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "l2h_model_get_tensor: NULL argument");
     if (role < 0 || role >= L2H_N_ROLES || (role >= 3 && (layer < 0 || layer >= m->c.n_layers)))
         return set_err(m->ctx, L2H_EINVAL, "role/layer out of range");
     DevTensor &t = role < 3 ? m->glob[role] : m->L(layer, role);
-    if (!t.base) return set_err(m->ctx, L2H_ESTATE, "%s not set", role_name(role));
+    if (t.type < 0) return set_err(m->ctx, L2H_ESTATE, "%s not set", role_name(role));
     if (host_bytes != t.gguf_bytes)
         return set_err(m->ctx, L2H_EINVAL, "buffer is %lld bytes, tensor is %lld", (long long)host_bytes,
                        (long long)t.gguf_bytes);
@@ -354,12 +380,14 @@ static PhaseArgs base_args(l2h_model *m) {
     a.neox = m->c.rope_is_neox;
     a.rope_cs = m->rope_cs;
     a.qd = m->qd;
+    a.normw_stride = m->L(0, L2H_RMS_ATT).layer_stride;
+    a.cache_stride = m->cache_layer_elems * 4;
     return a;
 }
 
-// rmsnorm (:244) + q, k, v (:247-249) + rope (:255-256) + cache append (:259-260)
-static hipError_t launch_qkv(l2h_model *m, int l) {
-    hipStream_t s = m->ctx->stream;
+// rmsnorm (:244) + q, k, v (:247-249) + rope (:255-256) + cache append (:259-260); tensors
+// first..last-1 of {wq, wk, wv} in one launch (they must share a type)
+static PhaseArgs make_qkv(l2h_model *m, int l, int first, int last) {
     const DevTensor *w[3] = {&m->L(l, L2H_WQ), &m->L(l, L2H_WK), &m->L(l, L2H_WV)};
     float *y[3] = {m->q, nullptr, nullptr};
     PhaseArgs a = base_args(m);
@@ -367,17 +395,23 @@ static hipError_t launch_qkv(l2h_model *m, int l) {
     a.normw = m->L(l, L2H_RMS_ATT).f32;
     a.kc = m->kc + (int64_t)l * m->cache_layer_elems;
     a.vc = m->vc + (int64_t)l * m->cache_layer_elems;
+    a.nseg = last - first;
+    a.seg_roles = 0;
+    for (int k = first; k < last; k++) {
+        a.w[k - first] = *w[k];
+        a.y[k - first] = y[k];
+        a.seg_roles |= k << (2 * (k - first));
+    }
+    return a;
+}
+
+static hipError_t launch_qkv(l2h_model *m, int l) {
+    const int t[3] = {m->L(l, L2H_WQ).type, m->L(l, L2H_WK).type, m->L(l, L2H_WV).type};
     int i = 0;
     while (i < 3) {  // consecutive tensors of one type share a launch
         int j = i + 1;
-        while (j < 3 && w[j]->type == w[i]->type) j++;
-        a.nseg = j - i;
-        for (int k = i; k < j; k++) {
-            a.w[k - i] = *w[k];
-            a.y[k - i] = y[k];
-            a.seg_role[k - i] = k;
-        }
-        hipError_t e = k_matvec(s, a, PRO_RMSNORM, EPI_ROPE_KV);
+        while (j < 3 && t[j] == t[i]) j++;
+        hipError_t e = k_matvec(m->ctx->stream, make_qkv(m, l, i, j), PRO_RMSNORM, EPI_ROPE_KV);
         if (e != hipSuccess) return e;
         i = j;
     }
@@ -385,33 +419,37 @@ static hipError_t launch_qkv(l2h_model *m, int l) {
 }
 
 // x += wo * xb (:281-284); the prologue quantizes the attention output
-static hipError_t launch_wo(l2h_model *m, int l) {
+static PhaseArgs make_wo(l2h_model *m, int l) {
     PhaseArgs a = base_args(m);
     a.nseg = 1;
     a.w[0] = m->L(l, L2H_WO);
     a.y[0] = m->x;
     a.resid = m->x;
     a.xf = m->xb;
-    return k_matvec(m->ctx->stream, a, PRO_QUANT, EPI_RESID);
+    return a;
+}
+static hipError_t launch_wo(l2h_model *m, int l) {
+    return k_matvec(m->ctx->stream, make_wo(m, l), PRO_QUANT, EPI_RESID);
 }
 
 // rmsnorm (:287) + w1, w3 (:291-292) + SwiGLU (:295-299) -> hb
-static hipError_t launch_w13(l2h_model *m, int l) {
-    hipStream_t s = m->ctx->stream;
-    const DevTensor &w1 = m->L(l, L2H_W1), &w3 = m->L(l, L2H_W3);
+static PhaseArgs make_w13(l2h_model *m, int l) {
     PhaseArgs a = base_args(m);
     a.xf = m->x;
     a.normw = m->L(l, L2H_RMS_FFN).f32;
-    if (w1.type == w3.type) {
-        a.nseg = 2;
-        a.w[0] = w1;
-        a.w[1] = w3;
-        a.y[0] = m->hb;
-        return k_matvec(s, a, PRO_RMSNORM, EPI_SWIGLU);
-    }
-    a.nseg = 1;
-    a.w[0] = w1;
+    a.nseg = 2;
+    a.w[0] = m->L(l, L2H_W1);
+    a.w[1] = m->L(l, L2H_W3);
     a.y[0] = m->hb;
+    return a;
+}
+static hipError_t launch_w13(l2h_model *m, int l) {
+    hipStream_t s = m->ctx->stream;
+    PhaseArgs a = make_w13(m, l);
+    if (a.w[0].type == a.w[1].type) return k_matvec(s, a, PRO_RMSNORM, EPI_SWIGLU);
+    // different types: two launches, then the stand-alone SwiGLU
+    const DevTensor w3 = a.w[1];
+    a.nseg = 1;
     hipError_t e = k_matvec(s, a, PRO_RMSNORM, EPI_STORE);
     if (e != hipSuccess) return e;
     a.w[0] = w3;
@@ -422,25 +460,167 @@ static hipError_t launch_w13(l2h_model *m, int l) {
 }
 
 // x += w2 * hb (:302-305)
-static hipError_t launch_w2(l2h_model *m, int l) {
+static PhaseArgs make_w2(l2h_model *m, int l) {
     PhaseArgs a = base_args(m);
     a.nseg = 1;
     a.w[0] = m->L(l, L2H_W2);
     a.y[0] = m->x;
     a.resid = m->x;
     a.xf = m->hb;
-    return k_matvec(m->ctx->stream, a, PRO_QUANT, EPI_RESID);
+    return a;
+}
+static hipError_t launch_w2(l2h_model *m, int l) {
+    return k_matvec(m->ctx->stream, make_w2(m, l), PRO_QUANT, EPI_RESID);
 }
 
 // final rmsnorm (:309) + classifier (:312)
-static hipError_t launch_output(l2h_model *m) {
+static PhaseArgs make_output(l2h_model *m) {
     PhaseArgs a = base_args(m);
     a.nseg = 1;
     a.w[0] = m->glob[L2H_OUTPUT];
     a.y[0] = m->logits;
     a.xf = m->x;
     a.normw = m->glob[L2H_RMS_FINAL].f32;
-    return k_matvec(m->ctx->stream, a, PRO_RMSNORM, EPI_STORE);
+    return a;
+}
+static hipError_t launch_output(l2h_model *m) {
+    return k_matvec(m->ctx->stream, make_output(m), PRO_RMSNORM, EPI_STORE);
+}
+
+// Moves the per-layer tensors of each role into one slab per role, layer l at base + l * stride,
+// so that a kernel can address any layer from the layer-0 pointers.
+static int rehome_layers(l2h_model *m) {
+    l2h_ctx *ctx = m->ctx;
+    const int L = m->c.n_layers;
+    for (int role = 3; role < L2H_N_ROLES; role++) {
+        const DevTensor &t0 = m->L(0, role);
+        bool same = true;
+        for (int l = 1; l < L; l++) same = same && m->L(l, role).type == t0.type && m->L(l, role).bytes == t0.bytes;
+        if (!same) continue;  // mixed types across layers: tensors stay where they are
+        char *slab = nullptr;
+        HIPCHK(ctx, hipMalloc((void **)&slab, (size_t)t0.bytes * L));
+        for (int l = 0; l < L; l++) {
+            DevTensor &t = m->L(l, role);
+            char *nb = slab + (int64_t)l * t.bytes;
+            HIPCHK(ctx, hipMemcpy(nb, t.base, (size_t)t.bytes, hipMemcpyDeviceToDevice));
+            const char *ob = (const char *)t.base;
+#define MOVE(F) if (t.F) t.F = (decltype(t.F))(nb + ((const char *)t.F - ob))
+            MOVE(hdr); MOVE(qs); MOVE(qh); MOVE(sc6); MOVE(d6); MOVE(f32);
+#undef MOVE
+            (void)hipFree(t.base);
+            t.base = l == 0 ? (void *)slab : nullptr;  // the slab is freed through layer 0
+            t.slab_member = true;
+            t.layer_stride = t.bytes;
+        }
+    }
+    return L2H_OK;
+}
+
+// ---- persistent decode kernel: plan + launch -------------------------------------------------
+static MegaArgs mega_args(l2h_model *m) {
+    MegaArgs g{};
+    g.bar = m->bar;
+    g.gen0 = m->bar_gen;
+    g.emb = m->glob[L2H_TOK_EMB];
+    g.ctl = m->ctl;
+    g.prompt = m->prompt_dev;
+    g.x = m->x;
+    g.xb = m->xb;
+    g.q = m->q;
+    g.rope_cs = m->rope_cs;
+    g.logits = m->logits;
+    g.kc = m->kc;
+    g.vc = m->vc;
+    g.cache_layer_elems = m->cache_layer_elems;
+    g.argmax_partial = (unsigned long long *)m->argmax_partial;
+    g.out_tokens = m->out_tokens;
+    g.max_out = m->max_out;
+    g.theta_scale = m->theta_scale;
+    g.hs = m->hs;
+    g.n_heads = m->c.n_heads;
+    g.n_kv_heads = m->c.n_kv_heads;
+    g.seq_len = m->c.seq_len;
+    g.n_layers = m->c.n_layers;
+    g.dim = m->c.dim;
+    g.vocab = m->c.vocab_size;
+    g.spin_limit = 1u << 22;
+#ifdef L2H_TIMELINE
+    g.timeline = m->timeline;
+#endif
+    return g;
+}
+
+// Decides whether this model can run on the persistent kernel and, if so, builds its plan.
+static int mega_setup(l2h_model *m) {
+    l2h_ctx *ctx = m->ctx;
+    const l2h_config &c = m->c;
+    m->mega = false;
+    if (m->path_request == 1 || getenv("L2H_NO_MEGA")) return L2H_OK;
+    const char *why = nullptr;
+    const int t_qkv = m->L(0, L2H_WQ).type, t_wo = m->L(0, L2H_WO).type, t_w13 = m->L(0, L2H_W1).type,
+              t_w2 = m->L(0, L2H_W2).type, t_out = m->glob[L2H_OUTPUT].type;
+    for (int l = 0; l < c.n_layers && !why; l++) {
+        if (m->L(l, L2H_WQ).type != t_qkv || m->L(l, L2H_WK).type != t_qkv || m->L(l, L2H_WV).type != t_qkv ||
+            m->L(l, L2H_WO).type != t_wo || m->L(l, L2H_W1).type != t_w13 || m->L(l, L2H_W3).type != t_w13 ||
+            m->L(l, L2H_W2).type != t_w2)
+            why = "tensor types differ between layers or inside a fused launch";
+    }
+    if (!why && !k_mega_supported(t_qkv, t_wo, t_w13, t_w2, t_out)) why = "no kernel for this combination of tensor types";
+    if (!why && std::max(c.dim, c.hidden_dim) > 16384) why = "activation vector longer than 16384";
+    const int grid = ctx->prop.multiProcessorCount;
+    if (!why) {
+        PhaseArgs a[5] = {make_qkv(m, 0, 0, 3), make_wo(m, 0), make_w13(m, 0), make_w2(m, 0), make_output(m)};
+        const int epi[5] = {EPI_ROPE_KV, EPI_RESID, EPI_SWIGLU, EPI_RESID, EPI_STORE};
+        for (int k = 0; k < 5; k++) {
+            a[k].max_grid = grid;
+            if (k_matvec_plan(a[k], epi[k]) <= 0) why = "phase cannot be planned";
+            m->mega_ph[k] = a[k];
+        }
+        if (m->L(0, L2H_RMS_ATT).layer_stride != m->L(0, L2H_RMS_FFN).layer_stride) why = "norm weight slabs differ";
+    }
+    size_t lds = 0;
+    if (!why) {
+        MegaArgs g = mega_args(m);
+        lds = k_mega_lds_bytes(g, m->mega_ph);
+        if (lds > 64 * 1024) why = "needs more than 64 KiB of LDS (sequence too long for the one-head-per-workgroup attention)";
+    }
+    if (why) {
+        if (m->path_request == 2) return set_err(ctx, L2H_EINVAL, "persistent kernel not available: %s", why);
+        return L2H_OK;
+    }
+    int rc;
+    if ((rc = dalloc(m, &m->bar, 1, true))) return rc;
+    m->bar_gen = 0;
+    m->mega_grid = grid;
+    m->mega_lds = lds;
+    m->mega_types[0] = t_qkv;
+    m->mega_types[1] = t_wo;
+    m->mega_types[2] = t_w13;
+    m->mega_types[3] = t_w2;
+    m->mega_types[4] = t_out;
+#ifdef L2H_TIMELINE
+    if ((rc = dalloc(m, &m->timeline, (int64_t)grid * 64, true))) return rc;
+    if ((rc = dalloc(m, &m->timeline2, (int64_t)grid * 8, true))) return rc;
+    {
+        const char *ph = getenv("L2H_TL_PHASE");
+        m->mega_ph[ph ? atoi(ph) : 2].timeline = m->timeline2;
+    }
+#endif
+    m->mega = true;
+    return L2H_OK;
+}
+
+static hipError_t mega_launch_token(l2h_model *m) {
+    if (g_bound_model != m) {
+        hipError_t e = k_mega_bind(m->ctx->stream, m->mega_ph);
+        if (e != hipSuccess) return e;
+        g_bound_model = m;
+    }
+    MegaArgs g = mega_args(m);
+    hipError_t e = k_mega_launch(m->ctx->stream, g, m->mega_types[0], m->mega_types[1], m->mega_types[2],
+                                 m->mega_types[3], m->mega_types[4], m->mega_grid, m->mega_lds);
+    if (e == hipSuccess) m->bar_gen += 2ull + 5ull * (unsigned long long)m->c.n_layers;
+    return e;
 }
 
 static hipError_t enqueue_token(l2h_model *m) {
@@ -482,6 +662,7 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
             if (!m->L(l, r).base) return set_err(ctx, L2H_ESTATE, "missing blk.%d weights (%s)", l, role_name(r));
     HIPCHK(ctx, hipSetDevice(ctx->device));
     int rc;
+    if ((rc = rehome_layers(m))) return rc;
 #define DA(p, n, z)                       \
     if ((rc = dalloc(m, &(p), (n), (z)))) \
         return rc;
@@ -507,13 +688,14 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     DA(m->prompt_dev, c.seq_len, true);
     m->max_out = c.seq_len;
     DA(m->out_tokens, m->max_out, true);
-    DA(m->argmax_partial, L2H_ARGMAX_BLOCKS, true);
+    DA(m->argmax_partial, std::max(L2H_ARGMAX_BLOCKS, ctx->prop.multiProcessorCount), true);
 #undef DA
     HIPCHK(ctx, hipDeviceSynchronize());
+    if ((rc = mega_setup(m))) return rc;
 
     // Record the launch sequence of one token; positions and tokens are read from the
     // control block on the device, so the recording is replayed unchanged for every step.
-    if (!getenv("L2H_NO_GRAPH")) {
+    if (!m->mega && !getenv("L2H_NO_GRAPH")) {
         HIPCHK(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeGlobal));
         hipError_t e = enqueue_token(m);
         hipGraph_t g = nullptr;
@@ -533,7 +715,10 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
 static int run_steps(l2h_model *m, int n) {
     l2h_ctx *ctx = m->ctx;
     for (int i = 0; i < n; i++) {
-        if (m->exec) {
+        if (m->mega) {
+            hipError_t e = mega_launch_token(m);
+            if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "decode kernel launch failed: %s", hipGetErrorString(e));
+        } else if (m->exec) {
             HIPCHK(ctx, hipGraphLaunch(m->exec, ctx->stream));
         } else {
             hipError_t e = enqueue_token(m);
@@ -541,6 +726,17 @@ static int run_steps(l2h_model *m, int n) {
         }
     }
     return L2H_OK;
+}
+
+// after the stream has drained: did a workgroup of the persistent kernel give up at a barrier?
+static int mega_check(l2h_model *m) {
+    if (!m->mega) return L2H_OK;
+    unsigned int ab = 0;
+    HIPCHK(m->ctx, hipMemcpy(&ab, &m->bar->abort, 4, hipMemcpyDeviceToHost));
+    if (!ab) return L2H_OK;
+    HIPCHK(m->ctx, hipMemset(m->bar, 0, sizeof(GridBar)));
+    m->bar_gen = 0;
+    return set_err(m->ctx, L2H_EHIP, "persistent decode kernel: a grid barrier timed out (workgroups not co-resident?)");
 }
 
 extern "C" int l2h_state_reset(l2h_model *m) {
@@ -636,7 +832,7 @@ static int generate_impl(l2h_model *m, const int32_t *prompt, int n_prompt, int 
         HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)m->c.vocab_size * 4, hipMemcpyDeviceToHost,
                                    ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    return L2H_OK;
+    return mega_check(m);
 }
 
 extern "C" int l2h_generate_greedy(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new,
@@ -1023,3 +1219,17 @@ extern "C" int l2h_profile_stream_read(l2h_ctx *ctx, int64_t n_bytes, int iters,
     *avg_us = ms * 1000.0f / (float)iters;
     return L2H_OK;
 }
+
+#ifdef L2H_TIMELINE
+// profiling build only: wall-clock stamps (100 MHz) of the last persistent-kernel launch
+extern "C" int l2h_debug_timeline(l2h_model *m, long long *out, int n_wg) {
+    if (!m || !m->mega || !m->timeline) return L2H_ESTATE;
+    HIPCHK(m->ctx, hipMemcpy(out, m->timeline, (size_t)n_wg * 64 * 8, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+extern "C" int l2h_debug_timeline2(l2h_model *m, long long *out, int n_wg) {
+    if (!m || !m->mega || !m->timeline2) return L2H_ESTATE;
+    HIPCHK(m->ctx, hipMemcpy(out, m->timeline2, (size_t)n_wg * 8 * 8, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+#endif

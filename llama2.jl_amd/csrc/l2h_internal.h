@@ -32,6 +32,8 @@ struct DevTensor {
     void *base = nullptr;
     int64_t bytes = 0;                  // allocation size
     int64_t gguf_bytes = 0;             // bytes the tensor occupies in a GGUF file
+    bool slab_member = false;           // lives inside a per-role slab (owned by layer 0's tensor)
+    int64_t layer_stride = 0;           // bytes from this tensor to the same tensor of the next layer (slab), or 0
     // stream pointers into base
     const uint4 *hdr = nullptr;         // Q4_K, Q5_K
     const uint8_t *qs = nullptr;        // Q4_K, Q5_K (128 B/block); Q6_K: ql
@@ -69,7 +71,7 @@ struct PhaseArgs {
     DevTensor w[3];
     float *y[3];           // STORE/RESID: output rows of each segment; SWIGLU: y[0] = hb; ROPE_KV: q rows
     int nseg;
-    int seg_role[3];       // ROPE_KV: SEG_Q / SEG_K / SEG_V
+    int seg_roles;         // ROPE_KV: SEG_Q / SEG_K / SEG_V of segment s in bits 2s, 2s+1
     // filled by k_matvec: logical rows in total and per workgroup (even), tile shape
     int64_t n_rows;
     int rows_per_wg, rt, st, ntpr;
@@ -77,6 +79,8 @@ struct PhaseArgs {
     Q8Dev xq;              // PRO_Q8: quantized input
     const float *xf;       // PRO_QUANT / PRO_RMSNORM: fp32 input
     const float *normw;    // PRO_RMSNORM: norm weights
+    int64_t normw_stride;  // bytes to the next layer's norm weights
+    int64_t cache_stride;  // bytes to the next layer's kc / vc
     const float *resid;    // EPI_RESID: y = resid + result (may alias y)
     // EPI_ROPE_KV
     const float *rope_cs;  // [hs/2][2] cos, sin of the current position
@@ -92,6 +96,38 @@ struct PhaseArgs {
 #endif
 };
 
+// State of the grid-wide barrier of the persistent decode kernel: 16 arrival counters (one per
+// 16 workgroups) feeding a root counter, and 8 copies of the release flag; every word sits in
+// its own 128-byte line.  Counters only grow: barrier number g completes when they reach g times
+// their arrival count.
+struct GridBar {
+    unsigned long long count[17 * 16];
+    unsigned long long flag[8 * 16];
+    unsigned int abort;  // set when a workgroup gave up waiting; the kernel then drains
+    unsigned int pad[31];
+};
+
+// Arguments of the persistent decode kernel (one launch = one token).
+struct MegaArgs {
+    GridBar *bar;
+    unsigned long long gen0;  // barriers completed by earlier launches
+    DevTensor emb;
+    DecodeCtl *ctl;
+    const int32_t *prompt;
+    float *x, *xb, *q, *rope_cs, *logits;
+    float *kc, *vc;  // layer 0; layer l at + l * cache_layer_elems
+    int64_t cache_layer_elems;
+    unsigned long long *argmax_partial;  // one slot per workgroup
+    int32_t *out_tokens;
+    int max_out;
+    float theta_scale;
+    int hs, n_heads, n_kv_heads, seq_len, n_layers, dim, vocab;
+    unsigned int spin_limit;  // polls before a barrier wait gives up
+#ifdef L2H_TIMELINE
+    long long *timeline;      // profiling build only: [workgroup][64] wall-clock stamps of the first phases
+#endif
+};
+
 // ---- launchers (kernel files) ----------------------------------------------------------------
 // Each returns hipGetLastError() of its launch.
 hipError_t k_repack(hipStream_t s, const DevTensor &t, const void *raw_dev, bool inverse, void *raw_out);
@@ -100,6 +136,15 @@ hipError_t k_embed(hipStream_t s, const DevTensor &emb, const DecodeCtl *ctl, co
 hipError_t k_dequant(hipStream_t s, const DevTensor &t, int64_t row0, int64_t nrows, float *y);
 hipError_t k_swiglu(hipStream_t s, float *hb, const float *hb2, int n);
 hipError_t k_matvec(hipStream_t s, PhaseArgs a, int pro, int epi);
+// fills the row split and tile shape of a phase for a grid of at most a.max_grid workgroups; returns the grid
+int k_matvec_plan(PhaseArgs &a, int epi);
+// persistent decode kernel: supported for the given tensor types?  LDS bytes it needs; launch
+bool k_mega_supported(int t_qkv, int t_wo, int t_w13, int t_w2, int t_out);
+size_t k_mega_lds_bytes(const MegaArgs &g, const PhaseArgs *ph);
+// ph: q/k/v, wo, w1+w3, w2 of layer 0 (later layers are addressed by stride) and the classifier
+hipError_t k_mega_bind(hipStream_t s, const PhaseArgs *ph);
+hipError_t k_mega_launch(hipStream_t s, const MegaArgs &g, int t_qkv, int t_wo, int t_w13, int t_w2, int t_out, int grid,
+                         size_t lds);
 hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64_t n, int pro, Q8Dev q8_out, float *f32_out);
 hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,

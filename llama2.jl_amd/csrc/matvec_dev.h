@@ -1,0 +1,741 @@
+// Device code of the k-quant / fp32 matvec phases, shared by the per-phase kernels and the
+// persistent decode kernel.
+#pragma once
+#include "dev_common.h"
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ uint4 ldg_nt(const uint4 *p) {
+    const u32x4 t = __builtin_nontemporal_load((const u32x4 *)p);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+
+// ------------------------------------------------------------------------------------------
+// Activations exchanged between workgroups INSIDE one kernel (the persistent decode kernel) are
+// written and read with device-scope relaxed atomics: such stores go through to memory and such
+// loads do not hit a stale line of another XCD's L2.  COH = false (one kernel per phase) uses
+// plain accesses; the kernel boundary orders them.
+// ------------------------------------------------------------------------------------------
+template <bool COH>
+__device__ __forceinline__ float ld_f32(const float *p) {
+    if (COH) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
+template <bool COH>
+__device__ __forceinline__ float4 ld_f32x4(const float *p) {
+    if (COH) {
+        const unsigned long long lo =
+            __hip_atomic_load((const unsigned long long *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned long long hi =
+            __hip_atomic_load((const unsigned long long *)p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return make_float4(__uint_as_float((uint32_t)lo), __uint_as_float((uint32_t)(lo >> 32)),
+                           __uint_as_float((uint32_t)hi), __uint_as_float((uint32_t)(hi >> 32)));
+    }
+    return *(const float4 *)p;
+}
+template <bool COH>
+__device__ __forceinline__ void st_f32(float *p, float v) {
+    if (COH)
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *p = v;
+}
+template <bool COH>
+__device__ __forceinline__ void st_f64(double *p, double v) {
+    if (COH)
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+        *p = v;
+}
+
+__device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// Activations staged in LDS for one workgroup.
+struct XLds {
+    const int8_t *qs;
+    const int16_t *bsums;
+    const float *d;
+    const float *xf;  // F32 weights: the fp32 input vector
+};
+
+// ---- what one lane loads for one chunk of a row ------------------------------------------------
+// q4_K: chunk c (0..7) of a block = qs bytes [16c, 16c+16): low nibbles are elements 64j+16h+k of
+// sub-block 2j, high nibbles elements 64j+32+16h+k of sub-block 2j+1 (j = c>>1, h = c&1;
+// reference src/kquants.jl:92-98).
+// q5_K: as q4_K plus bit 2j / 2j+1 of qh[16h+k] (src/kquants.jl:213,217,220-221).
+// q6_K: chunk c (0..3) = ql bytes [64n+16h,+16) and [64n+32+16h,+16) with qh bytes [32n+16h,+16),
+// n = c>>1, h = c&1: four groups of 16 elements at 128n+32g+16h (src/kquants.jl:333-343).
+template <int TYPE>
+struct Chunk;
+template <>
+struct Chunk<L2H_TYPE_Q4_K> {
+    uint4 w, hdr;
+};
+template <>
+struct Chunk<L2H_TYPE_Q5_K> {
+    uint4 w, qh, hdr;
+};
+template <>
+struct Chunk<L2H_TYPE_Q6_K> {
+    uint4 la, lb, qh;
+    uint32_t sc;
+    uint32_t d;
+};
+
+__device__ __forceinline__ void zero_chunk(Chunk<L2H_TYPE_Q4_K> &c) {
+    c.w = make_uint4(0, 0, 0, 0);
+    c.hdr = make_uint4(0, 0, 0, 0);
+}
+__device__ __forceinline__ void zero_chunk(Chunk<L2H_TYPE_Q5_K> &c) {
+    c.w = make_uint4(0, 0, 0, 0);
+    c.qh = make_uint4(0, 0, 0, 0);
+    c.hdr = make_uint4(0, 0, 0, 0);
+}
+__device__ __forceinline__ void zero_chunk(Chunk<L2H_TYPE_Q6_K> &c) {
+    c.la = make_uint4(0, 0, 0, 0);
+    c.lb = make_uint4(0, 0, 0, 0);
+    c.qh = make_uint4(0, 0, 0, 0);
+    c.sc = 0;
+    c.d = 0;
+}
+
+template <int TYPE>
+__device__ __forceinline__ int chunks_per_block() {
+    return TYPE == L2H_TYPE_Q6_K ? 4 : 8;
+}
+
+// Stream pointers of the segment a row lives in, picked with selects so that the kernel
+// arguments are only ever read at fixed offsets (one batch of scalar loads at kernel entry).
+struct SegPtrs {
+    const uint4 *hdr, *qs, *qh;
+    const uint32_t *sc6;
+    const uint16_t *d6;
+    int64_t nb;
+};
+template <class T>
+__device__ __forceinline__ T *at_layer(T *p, int64_t stride_bytes, int layer) {
+    return (T *)((char *)p + stride_bytes * layer);
+}
+// `layer` selects the copy inside a per-role slab (0 when the pointers already name the layer)
+__device__ __forceinline__ SegPtrs seg_ptrs(const PhaseArgs &a, int seg, int layer) {
+    SegPtrs p;
+#define PICK(F) (seg == 0 ? a.w[0].F : (seg == 1 ? a.w[1].F : a.w[2].F))
+    const int64_t off = PICK(layer_stride) * layer;
+    p.hdr = (const uint4 *)((const char *)PICK(hdr) + off);
+    p.qs = (const uint4 *)((const char *)PICK(qs) + off);
+    p.qh = (const uint4 *)((const char *)PICK(qh) + off);
+    p.sc6 = (const uint32_t *)((const char *)PICK(sc6) + off);
+    p.d6 = (const uint16_t *)((const char *)PICK(d6) + off);
+#undef PICK
+    p.nb = a.w[0].nb;
+    return p;
+}
+
+template <int TYPE>
+__device__ __forceinline__ void load_chunk(Chunk<TYPE> &c, const SegPtrs &t, int64_t row, int g);
+
+template <>
+__device__ __forceinline__ void load_chunk<L2H_TYPE_Q4_K>(Chunk<L2H_TYPE_Q4_K> &c, const SegPtrs &t, int64_t row,
+                                                          int g) {
+    c.w = ldg_nt(t.qs + row * t.nb * 8 + g);
+    c.hdr = ldg_nt(t.hdr + row * t.nb + (g >> 3));
+}
+template <>
+__device__ __forceinline__ void load_chunk<L2H_TYPE_Q5_K>(Chunk<L2H_TYPE_Q5_K> &c, const SegPtrs &t, int64_t row,
+                                                          int g) {
+    c.w = ldg_nt(t.qs + row * t.nb * 8 + g);
+    c.qh = ldg_nt(t.qh + (row * t.nb + (g >> 3)) * 2 + (g & 1));
+    c.hdr = ldg_nt(t.hdr + row * t.nb + (g >> 3));
+}
+template <>
+__device__ __forceinline__ void load_chunk<L2H_TYPE_Q6_K>(Chunk<L2H_TYPE_Q6_K> &c, const SegPtrs &t, int64_t row,
+                                                          int g) {
+    const int64_t blk = row * t.nb + (g >> 2);
+    const int n = (g >> 1) & 1, h = g & 1;
+    c.la = ldg_nt(t.qs + blk * 8 + 4 * n + h);
+    c.lb = ldg_nt(t.qs + blk * 8 + 4 * n + 2 + h);
+    c.qh = ldg_nt(t.qh + blk * 4 + 2 * n + h);
+    c.sc = __builtin_nontemporal_load(t.sc6 + blk * 4 + 2 * n + h);
+    c.d = (uint32_t)__builtin_nontemporal_load(t.d6 + blk);
+}
+
+// ---- this lane's fp64 share of one chunk; DEBUG also stores the per-block integer sums ----------
+template <bool DEBUG>
+__device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q4_K> &ch, int g, const XLds &x, int32_t *dbg_isc,
+                                             int32_t *dbg_imin, int64_t dbg_base) {
+    const int b = g >> 3, c = g & 7, j = c >> 1, h = c & 1;
+    int sc_a, sc_b, m_a, m_b;
+    kq_scales_pair(ch.hdr, j, sc_a, sc_b, m_a, m_b);
+    const int8_t *xb = x.qs + b * 256 + 64 * j + 16 * h;
+    const uint4 xlo = *(const uint4 *)xb;
+    const uint4 xhi = *(const uint4 *)(xb + 32);
+    const uint4 w = ch.w;
+    int dot_a = 0, dot_b = 0;
+    dot_a = sdot4(w.x & 0x0F0F0F0Fu, xlo.x, dot_a);
+    dot_a = sdot4(w.y & 0x0F0F0F0Fu, xlo.y, dot_a);
+    dot_a = sdot4(w.z & 0x0F0F0F0Fu, xlo.z, dot_a);
+    dot_a = sdot4(w.w & 0x0F0F0F0Fu, xlo.w, dot_a);
+    dot_b = sdot4((w.x >> 4) & 0x0F0F0F0Fu, xhi.x, dot_b);
+    dot_b = sdot4((w.y >> 4) & 0x0F0F0F0Fu, xhi.y, dot_b);
+    dot_b = sdot4((w.z >> 4) & 0x0F0F0F0Fu, xhi.z, dot_b);
+    dot_b = sdot4((w.w >> 4) & 0x0F0F0F0Fu, xhi.w, dot_b);
+    const int16_t *bs = x.bsums + b * 16 + 4 * j + h;
+    int i_sc = sc_a * dot_a + sc_b * dot_b;
+    int i_min = m_a * (int)bs[0] + m_b * (int)bs[2];
+    const float yd = x.d[b];
+    const float dy = half_bits_to_float((uint16_t)(ch.hdr.x & 0xFFFF)) * yd;
+    const float my = half_bits_to_float((uint16_t)(ch.hdr.x >> 16)) * yd;
+    double t = (double)dy * (double)i_sc;
+    t = fma(-(double)my, (double)i_min, t);
+    if (DEBUG) {
+        i_sc += __shfl_xor(i_sc, 1, WAVE);
+        i_min += __shfl_xor(i_min, 1, WAVE);
+        i_sc += __shfl_xor(i_sc, 2, WAVE);
+        i_min += __shfl_xor(i_min, 2, WAVE);
+        i_sc += __shfl_xor(i_sc, 4, WAVE);
+        i_min += __shfl_xor(i_min, 4, WAVE);
+        if (c == 0) {
+            dbg_isc[dbg_base + b] = i_sc;
+            dbg_imin[dbg_base + b] = i_min;
+        }
+    }
+    return t;
+}
+
+template <bool DEBUG>
+__device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q5_K> &ch, int g, const XLds &x, int32_t *dbg_isc,
+                                             int32_t *dbg_imin, int64_t dbg_base) {
+    const int b = g >> 3, c = g & 7, j = c >> 1, h = c & 1;
+    int sc_a, sc_b, m_a, m_b;
+    kq_scales_pair(ch.hdr, j, sc_a, sc_b, m_a, m_b);
+    const int8_t *xb = x.qs + b * 256 + 64 * j + 16 * h;
+    const uint4 xlo = *(const uint4 *)xb;
+    const uint4 xhi = *(const uint4 *)(xb + 32);
+    const uint4 w = ch.w, qh = ch.qh;
+    const int sa = 2 * j, sb = 2 * j + 1;
+    int dot_a = 0, dot_b = 0;
+#define Q5LO(W, H) (((W)&0x0F0F0F0Fu) | ((((H) >> sa) & 0x01010101u) << 4))
+#define Q5HI(W, H) ((((W) >> 4) & 0x0F0F0F0Fu) | ((((H) >> sb) & 0x01010101u) << 4))
+    dot_a = sdot4(Q5LO(w.x, qh.x), xlo.x, dot_a);
+    dot_a = sdot4(Q5LO(w.y, qh.y), xlo.y, dot_a);
+    dot_a = sdot4(Q5LO(w.z, qh.z), xlo.z, dot_a);
+    dot_a = sdot4(Q5LO(w.w, qh.w), xlo.w, dot_a);
+    dot_b = sdot4(Q5HI(w.x, qh.x), xhi.x, dot_b);
+    dot_b = sdot4(Q5HI(w.y, qh.y), xhi.y, dot_b);
+    dot_b = sdot4(Q5HI(w.z, qh.z), xhi.z, dot_b);
+    dot_b = sdot4(Q5HI(w.w, qh.w), xhi.w, dot_b);
+#undef Q5LO
+#undef Q5HI
+    const int16_t *bs = x.bsums + b * 16 + 4 * j + h;
+    int i_sc = sc_a * dot_a + sc_b * dot_b;
+    int i_min = m_a * (int)bs[0] + m_b * (int)bs[2];
+    const float yd = x.d[b];
+    const float dy = half_bits_to_float((uint16_t)(ch.hdr.x & 0xFFFF)) * yd;
+    const float my = half_bits_to_float((uint16_t)(ch.hdr.x >> 16)) * yd;
+    double t = (double)dy * (double)i_sc;
+    t = fma(-(double)my, (double)i_min, t);
+    if (DEBUG) {
+        i_sc += __shfl_xor(i_sc, 1, WAVE);
+        i_min += __shfl_xor(i_min, 1, WAVE);
+        i_sc += __shfl_xor(i_sc, 2, WAVE);
+        i_min += __shfl_xor(i_min, 2, WAVE);
+        i_sc += __shfl_xor(i_sc, 4, WAVE);
+        i_min += __shfl_xor(i_min, 4, WAVE);
+        if (c == 0) {
+            dbg_isc[dbg_base + b] = i_sc;
+            dbg_imin[dbg_base + b] = i_min;
+        }
+    }
+    return t;
+}
+
+// q-32 is folded in through the q8_K group sums: sum (q-32)*x = sum q*x - 32*bsum.
+template <bool DEBUG>
+__device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q6_K> &ch, int g, const XLds &x, int32_t *dbg_isc,
+                                             int32_t *dbg_imin, int64_t dbg_base) {
+    const int b = g >> 2, c = g & 3, n = c >> 1, h = c & 1;
+    const int8_t *xb = x.qs + b * 256 + 128 * n + 16 * h;
+    const uint4 x0 = *(const uint4 *)xb, x1 = *(const uint4 *)(xb + 32), x2 = *(const uint4 *)(xb + 64),
+                x3 = *(const uint4 *)(xb + 96);
+    const uint4 la = ch.la, lb = ch.lb, qh = ch.qh;
+    int d0 = 0, d1 = 0, d2 = 0, d3 = 0;
+#define Q6STEP(A, B, H, X0, X1, X2, X3)                                 \
+    d0 = sdot4(((A)&0x0F0F0F0Fu) | (((H) << 4) & 0x30303030u), X0, d0); \
+    d1 = sdot4(((B)&0x0F0F0F0Fu) | (((H) << 2) & 0x30303030u), X1, d1); \
+    d2 = sdot4((((A) >> 4) & 0x0F0F0F0Fu) | ((H)&0x30303030u), X2, d2); \
+    d3 = sdot4((((B) >> 4) & 0x0F0F0F0Fu) | (((H) >> 2) & 0x30303030u), X3, d3);
+    Q6STEP(la.x, lb.x, qh.x, x0.x, x1.x, x2.x, x3.x)
+    Q6STEP(la.y, lb.y, qh.y, x0.y, x1.y, x2.y, x3.y)
+    Q6STEP(la.z, lb.z, qh.z, x0.z, x1.z, x2.z, x3.z)
+    Q6STEP(la.w, lb.w, qh.w, x0.w, x1.w, x2.w, x3.w)
+#undef Q6STEP
+    const int16_t *bs = x.bsums + b * 16 + 8 * n + h;
+    const uint32_t scw = ch.sc;
+    const int s0 = (int)(int8_t)(scw & 0xFF), s1 = (int)(int8_t)((scw >> 8) & 0xFF),
+              s2 = (int)(int8_t)((scw >> 16) & 0xFF), s3 = (int)(int8_t)(scw >> 24);
+    int i_sc = s0 * (d0 - 32 * (int)bs[0]) + s1 * (d1 - 32 * (int)bs[2]) + s2 * (d2 - 32 * (int)bs[4]) +
+               s3 * (d3 - 32 * (int)bs[6]);
+    const float dy = half_bits_to_float((uint16_t)ch.d) * x.d[b];
+    const double t = (double)dy * (double)i_sc;
+    if (DEBUG) {
+        i_sc += __shfl_xor(i_sc, 1, WAVE);
+        i_sc += __shfl_xor(i_sc, 2, WAVE);
+        if (c == 0) {
+            dbg_isc[dbg_base + b] = i_sc;
+            dbg_imin[dbg_base + b] = 0;
+        }
+    }
+    return t;
+}
+
+// ------------------------------------------------------------------------------------------
+// wavefront reductions on DPP row operations (ALU latency, no LDS crossbar round trips)
+// ------------------------------------------------------------------------------------------
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, 0xF, 0xF, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, 0xF, 0xF, false);
+    return __hiloint2double(hi, lo);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+    const int lo = __builtin_amdgcn_readlane(__double2loint(v), lane);
+    const int hi = __builtin_amdgcn_readlane(__double2hiint(v), lane);
+    return __hiloint2double(hi, lo);
+}
+#define DPP_QUAD_SWAP1 0xB1     // quad_perm [1,0,3,2]
+#define DPP_QUAD_SWAP2 0x4E     // quad_perm [2,3,0,1]
+#define DPP_ROW_HALF_MIRROR 0x141
+#define DPP_ROW_MIRROR 0x140
+
+// Sum over the 64 lanes; the same value is returned on every lane.  Fixed order.
+__device__ __forceinline__ double wave_sum_f64_dpp(double v) {
+    v += dpp_f64<DPP_QUAD_SWAP1>(v);
+    v += dpp_f64<DPP_QUAD_SWAP2>(v);
+    v += dpp_f64<DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f64<DPP_ROW_MIRROR>(v);
+    return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
+}
+__device__ __forceinline__ float wave_max_f32_dpp(float v) {
+    v = fmaxf(v, dpp_f32<DPP_QUAD_SWAP1>(v));
+    v = fmaxf(v, dpp_f32<DPP_QUAD_SWAP2>(v));
+    v = fmaxf(v, dpp_f32<DPP_ROW_HALF_MIRROR>(v));
+    v = fmaxf(v, dpp_f32<DPP_ROW_MIRROR>(v));
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+// sum within aligned groups of 4 lanes
+__device__ __forceinline__ int quad_sum_i32(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, DPP_QUAD_SWAP1, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(0, v, DPP_QUAD_SWAP2, 0xF, 0xF, false);
+    return v;
+}
+
+// ------------------------------------------------------------------------------------------
+// prologue: activations -> this workgroup's LDS
+// ------------------------------------------------------------------------------------------
+// One wavefront quantizes one q8_K block; lane l holds elements 4l..4l+3.  llama.cpp's
+// quantize_row_q8_K rule: the FIRST element of largest magnitude fixes the scale (ties go to the
+// lowest index), iscale = -127/max, q = min(127, round-half-even(iscale*x)), d = 1/iscale.
+__device__ __forceinline__ void q8k_quantize_wave(const float v[4], uint32_t &packed, int &bsum16, float &d) {
+    float amax = 0.0f, mx = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const float ax = fabsf(v[k]);
+        if (ax > amax) {
+            amax = ax;
+            mx = v[k];
+        }
+    }
+    const float wmax = wave_max_f32_dpp(amax);
+    if (wmax == 0.0f) {
+        packed = 0;
+        bsum16 = 0;
+        d = 0.0f;
+        return;
+    }
+    // lowest lane whose own extreme reaches the block's: its first such element is the block's first
+    const unsigned long long holders = __ballot(amax == wmax);
+    const int first = __builtin_ctzll(holders);
+    const float bmx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx), first));
+    const float iscale = -127.0f / bmx;
+    uint32_t word = 0;
+    int sum = 0;
+#pragma unroll
+    for (int b = 0; b < 4; b++) {
+        int q = (int)rintf(iscale * v[b]);
+        q = q < 127 ? q : 127;
+        sum += (int)(int8_t)q;
+        word |= ((uint32_t)(q & 0xFF)) << (8 * b);
+    }
+    packed = word;
+    bsum16 = quad_sum_i32(sum);
+    d = 1.0f / iscale;
+}
+
+#define STAGE_MAX_ROUNDS 4  // q8_K blocks per wavefront: K <= 4 * 16 * 256
+
+template <int PRO, bool KQ, bool COH>
+__device__ __forceinline__ void stage_activations(const PhaseArgs &a, int layer, int64_t K, int8_t *s_qs, int16_t *s_bs,
+                                                  float *s_d, float *s_xf, double *red) {
+    const float *normw = at_layer(a.normw, a.normw_stride, layer);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    if (PRO == PRO_Q8) {
+        const uint4 *g_qs = (const uint4 *)a.xq.qs;
+        for (int i = tid; i < K / 16; i += blockDim.x) ((uint4 *)s_qs)[i] = g_qs[i];
+        const uint4 *g_bs = (const uint4 *)a.xq.bsums;
+        for (int i = tid; i < K / 128; i += blockDim.x) ((uint4 *)s_bs)[i] = g_bs[i];
+        for (int i = tid; i < K / 256; i += blockDim.x) s_d[i] = a.xq.d[i];
+        return;
+    }
+    if (!KQ) {  // F32 weights consume fp32 activations
+        float ss = 1.0f;
+        if (PRO == PRO_RMSNORM) {
+            double acc = 0.0;
+            for (int64_t i = tid; i < K; i += blockDim.x) {
+                const double v = (double)ld_f32<COH>(a.xf + i);
+                acc = fma(v, v, acc);
+            }
+            ss = (float)block_sum_f64(acc, red);
+            ss /= (float)K;
+            ss += 1e-5f;
+            ss = 1.0f / sqrtf(ss);
+        }
+        for (int64_t i = tid; i < K; i += blockDim.x)
+            s_xf[i] = PRO == PRO_RMSNORM ? normw[i] * (ss * ld_f32<COH>(a.xf + i)) : ld_f32<COH>(a.xf + i);
+        return;
+    }
+    // k-quant weights: wavefront w takes q8_K blocks w, w+nwaves, ...; all loads issued first
+    const int nb = (int)(K >> 8);
+    float4 xv[STAGE_MAX_ROUNDS], wv[STAGE_MAX_ROUNDS];
+#pragma unroll
+    for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+        const int b = wave + r * nwaves;
+        if (b < nb) {
+            xv[r] = ld_f32x4<COH>(a.xf + 256 * b + 4 * lane);
+            if (PRO == PRO_RMSNORM) wv[r] = *(const float4 *)(normw + 256 * b + 4 * lane);
+        }
+    }
+    float ss = 1.0f;
+    if (PRO == PRO_RMSNORM) {  // rmsnorm! (reference src/inference.jl:102-110)
+        double acc = 0.0;
+#pragma unroll
+        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+            const int b = wave + r * nwaves;
+            if (b < nb) {
+                acc = fma((double)xv[r].x, (double)xv[r].x, acc);
+                acc = fma((double)xv[r].y, (double)xv[r].y, acc);
+                acc = fma((double)xv[r].z, (double)xv[r].z, acc);
+                acc = fma((double)xv[r].w, (double)xv[r].w, acc);
+            }
+        }
+        acc = wave_sum_f64_dpp(acc);
+        if (lane == 0) red[wave] = acc;
+        __syncthreads();
+        double t = 0.0;
+        for (int w = 0; w < nwaves; w++) t += red[w];
+        ss = (float)t;
+        ss /= (float)K;
+        ss += 1e-5f;
+        ss = 1.0f / sqrtf(ss);
+    }
+#pragma unroll
+    for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+        const int b = wave + r * nwaves;
+        if (b < nb) {
+            float v[4] = {xv[r].x, xv[r].y, xv[r].z, xv[r].w};
+            if (PRO == PRO_RMSNORM) {
+                v[0] = wv[r].x * (ss * v[0]);
+                v[1] = wv[r].y * (ss * v[1]);
+                v[2] = wv[r].z * (ss * v[2]);
+                v[3] = wv[r].w * (ss * v[3]);
+            }
+            uint32_t packed;
+            int bsum;
+            float d;
+            q8k_quantize_wave(v, packed, bsum, d);
+            ((uint32_t *)s_qs)[64 * b + lane] = packed;
+            if ((lane & 3) == 0) s_bs[16 * b + (lane >> 2)] = (int16_t)bsum;
+            if (lane == 0) s_d[b] = d;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// logical rows.  Rows are numbered so that the two rows an epilogue combines are neighbours
+// (2i, 2i+1): a w1/w3 pair, a RoPE pair; otherwise the concatenation of the segments' rows.
+// ------------------------------------------------------------------------------------------
+struct RowRef {
+    int seg;      // segment index, -1 = no such row
+    int64_t row;  // row inside the segment
+};
+
+// the row of a tile is the same on every lane: say so, and the address arithmetic and the
+// selection of the segment's pointers run on the scalar unit
+__device__ __forceinline__ RowRef uniform_row(RowRef r) {
+    RowRef u;
+    u.seg = __builtin_amdgcn_readfirstlane(r.seg);
+    const int lo = __builtin_amdgcn_readfirstlane((int)(r.row & 0xFFFFFFFFll));
+    const int hi = __builtin_amdgcn_readfirstlane((int)(r.row >> 32));
+    u.row = ((int64_t)hi << 32) | (uint32_t)lo;
+    return u;
+}
+
+template <int EPI>
+__device__ __forceinline__ RowRef logical_row(const PhaseArgs &a, int64_t L) {
+    RowRef rr;
+    if (EPI == EPI_SWIGLU) {  // (w1 row g, w3 row g)
+        rr.seg = (int)(L & 1);
+        rr.row = L >> 1;
+        return rr;
+    }
+    const int64_t n0 = a.w[0].ne1, n1 = a.nseg > 1 ? a.w[1].ne1 : 0, n2 = a.nseg > 2 ? a.w[2].ne1 : 0;
+    if (L < n0) {
+        rr.seg = 0;
+    } else if (L < n0 + n1) {
+        rr.seg = 1;
+        L -= n0;
+    } else if (L < n0 + n1 + n2) {
+        rr.seg = 2;
+        L -= n0 + n1;
+    } else {
+        rr.seg = -1;
+    }
+    rr.row = L;
+    if (EPI == EPI_ROPE_KV && rr.seg >= 0 && a.neox) {
+        const int role = (a.seg_roles >> (2 * rr.seg)) & 3;
+        if (role != SEG_V) {  // neox pairs element i with i + hs/2 (reference src/inference.jl:146)
+            const int half = a.hs >> 1;
+            const int64_t h = L / a.hs;
+            const int e = (int)(L % a.hs);
+            rr.row = h * a.hs + (e >> 1) + ((e & 1) ? half : 0);
+        }
+    }
+    return rr;
+}
+
+// exp evaluated in fp64 and rounded to fp32 (reference src/inference.jl:296)
+__device__ __forceinline__ float swiglu_val(float h1, float h3) {
+    const float e = (float)exp((double)(-h1));
+    const float v = h1 * (1.0f / (1.0f + e));
+    return v * h3;
+}
+
+// One thread finishes logical row L; `other` is the value of its neighbour row L^1.
+template <int EPI, bool COH>
+__device__ __forceinline__ void finish_row(const PhaseArgs &a, int layer, int64_t L, float val, float other) {
+    const RowRef rr = logical_row<EPI>(a, L);
+    if (rr.seg < 0) return;
+    const int r = (int)(L & 1);
+    if (EPI == EPI_STORE) {
+        float *y = rr.seg == 0 ? a.y[0] : (rr.seg == 1 ? a.y[1] : a.y[2]);
+        st_f32<COH>(y + rr.row, val);
+    } else if (EPI == EPI_RESID) {  // x .+= ... (src/inference.jl:284,305)
+        st_f32<COH>(a.y[0] + rr.row, ld_f32<COH>(a.resid + rr.row) + val);
+    } else if (EPI == EPI_SWIGLU) {  // src/inference.jl:295-299
+        if (r == 0) st_f32<COH>(a.y[0] + rr.row, swiglu_val(val, other));
+    } else {  // EPI_ROPE_KV: rope! (src/inference.jl:112-157) and cache append (:259-260)
+        const int role = (a.seg_roles >> (2 * rr.seg)) & 3;
+        const int pos = a.ctl->pos;
+        const int h = (int)(rr.row / a.hs), e = (int)(rr.row % a.hs);
+        if (role == SEG_V) {
+            st_f32<COH>(at_layer(a.vc, a.cache_stride, layer) + ((int64_t)h * a.seq_len + pos) * a.hs + e, val);
+            return;
+        }
+        const int half = a.hs >> 1;
+        const int i = a.neox ? (e % half) : (e >> 1);
+        const float c = ld_f32<COH>(a.rope_cs + 2 * i), s = ld_f32<COH>(a.rope_cs + 2 * i + 1);
+        // complex product (re + i im)(c + i s), each of the four products rounded
+        const float re = r == 0 ? val : other, im = r == 0 ? other : val;
+        const float out = r == 0 ? (re * c) - (im * s) : (re * s) + (im * c);
+        if (role == SEG_Q) {
+            st_f32<COH>(a.y[0] + rr.row, out);  // q is always the first segment of its launch
+            st_f64<COH>(a.qd + rr.row, (double)out);
+        } else {
+            st_f32<COH>(at_layer(a.kc, a.cache_stride, layer) + (((int64_t)h * (a.hs >> 2) + (e >> 2)) * a.seq_len + pos) * 4 + (e & 3), out);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// the k-quant kernel.  A workgroup owns a contiguous range of logical rows.  Its work is cut
+// into tiles of rt rows x st chunk-steps (rt*st <= NSLOT; a chunk-step = 64 lanes x one chunk);
+// the 16 wavefronts take tiles round-robin with the next tile's loads in flight, reduce each
+// tile's rows over the lanes and leave fp64 partial sums in LDS; then one thread per row adds
+// that row's partials in a fixed order and runs the epilogue.
+// ------------------------------------------------------------------------------------------
+template <int TYPE>
+struct Tile {
+    static constexpr int NSLOT = TYPE == L2H_TYPE_Q4_K ? 4 : 2;
+    Chunk<TYPE> c[NSLOT];
+};
+
+// profiling builds (-DL2H_TIMELINE) stamp the phases of every workgroup with the 100 MHz wall clock
+#ifdef L2H_TIMELINE
+#define TL(i)                                                                                 \
+    if (a.timeline && threadIdx.x == 0) a.timeline[blockIdx.x * 8 + (i)] = wall_clock64();
+#else
+#define TL(i)
+#endif
+
+// One phase of one workgroup `wg`.  `smem` is the dynamic LDS area, `red` 16 doubles, `s_next` the
+// tile counter.  If `preloaded`, `cur` already holds tile number `wave` of this phase (its loads
+// were issued before the caller waited on the previous phase).
+template <int TYPE, int PRO, int EPI, bool DEBUG, bool COH>
+__device__ __forceinline__ void matvec_phase(const PhaseArgs &a, int layer, int wg, uint4 *smem, double *red,
+                                             int *s_next_p, Tile<TYPE> &cur, bool preloaded) {
+    TL(0)
+    constexpr int NSLOT = Tile<TYPE>::NSLOT;
+    constexpr int CPB = TYPE == L2H_TYPE_Q6_K ? 4 : 8;
+    const int64_t K = a.w[0].ne0;
+    int8_t *s_qs = (int8_t *)smem;
+    int16_t *s_bs = (int16_t *)(s_qs + K);
+    float *s_d = (float *)(s_qs + K + K / 8);
+    double *s_part = (double *)(s_qs + ((K + K / 8 + K / 64 + 15) & ~(int64_t)15));  // [rows_per_wg][ntpr]
+    float *s_val = (float *)(s_part + (int64_t)a.rows_per_wg * a.ntpr);              // [rows_per_wg]
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
+    const int rt = a.rt, st = a.st, ntpr = a.ntpr;
+    const int64_t L_lo = (int64_t)wg * a.rows_per_wg;
+    const int64_t L_hi = min(a.n_rows, L_lo + a.rows_per_wg);
+    const int n_local = L_hi > L_lo ? (int)(L_hi - L_lo) : 0;
+    const int nchunks = (int)a.w[0].nb * CPB;
+    const int nsteps = (nchunks + WAVE - 1) / WAVE;
+    const int n_rowblocks = (n_local + rt - 1) / rt;
+    const int ntiles = n_rowblocks * ntpr;
+
+    // slot k of a tile: row offset k / st, step offset k % st
+    auto load_tile = [&](Tile<TYPE> &t, int tt) {
+        const int rb = tt / ntpr, sb = tt % ntpr;
+#pragma unroll
+        for (int k = 0; k < NSLOT; k++) {
+            const int ro = k / st, so = k % st;
+            const int lr = rb * rt + ro, step = sb * st + so;
+            const int ci = lane + WAVE * step;
+            if (ro < rt && lr < n_local && step < nsteps && ci < nchunks) {
+                const RowRef rr = uniform_row(logical_row<EPI>(a, L_lo + lr));
+                if (rr.seg >= 0) load_chunk<TYPE>(t.c[k], seg_ptrs(a, rr.seg, layer), rr.row, ci);
+            }
+        }
+    };
+
+    // the first 16 tiles are handed out statically, the rest on demand (equalises the finish
+    // times of the wavefronts); every tile's partial sums have their own LDS slots, so the
+    // result does not depend on which wavefront ran which tile
+    if (threadIdx.x == 0) *s_next_p = nwaves;
+    Tile<TYPE> nxt;
+    int tt = wave;
+    if (!preloaded && tt < ntiles) load_tile(cur, tt);  // in flight while the activations are staged
+    TL(1)
+
+    stage_activations<PRO, true, COH>(a, layer, K, s_qs, s_bs, s_d, nullptr, red);
+    TL(2)
+    __syncthreads();
+    TL(3)
+    XLds x{s_qs, s_bs, s_d, nullptr};
+
+    while (tt < ntiles) {
+        int tn = 0;
+        if (lane == 0) tn = atomicAdd(s_next_p, 1);
+        tn = __builtin_amdgcn_readfirstlane(tn);
+        if (tn < ntiles) load_tile(nxt, tn);
+        const int rb = tt / ntpr, sb = tt % ntpr;
+        double acc[NSLOT];
+#pragma unroll
+        for (int k = 0; k < NSLOT; k++) {
+            acc[k] = 0.0;
+            const int ro = k / st, so = k % st;
+            const int lr = rb * rt + ro, step = sb * st + so;
+            const int ci = lane + WAVE * step;
+            if (ro < rt && lr < n_local && step < nsteps && ci < nchunks) {
+                const RowRef rr = uniform_row(logical_row<EPI>(a, L_lo + lr));
+                if (rr.seg >= 0) {
+                    int64_t dbg_base = 0;
+                    if (DEBUG) dbg_base = rr.row * a.w[0].nb;  // debug launches have one segment
+                    acc[k] = chunk_term<DEBUG>(cur.c[k], ci, x, a.dbg_isc, a.dbg_imin, dbg_base);
+                }
+            }
+        }
+        // fold the slots of each row, reduce over the lanes, park the partial sum
+#pragma unroll
+        for (int ro = 0; ro < NSLOT; ro++) {
+            if (ro < rt) {  // uniform
+                double v = 0.0;
+#pragma unroll
+                for (int k = 0; k < NSLOT; k++)
+                    if (k / st == ro) v += acc[k];
+                v = wave_sum_f64_dpp(v);
+                const int lr = rb * rt + ro;
+                if (lane == 0 && lr < n_local) s_part[lr * ntpr + sb] = v;
+            }
+        }
+        cur = nxt;
+        tt = tn;
+    }
+    TL(4)
+    __syncthreads();
+    TL(5)
+    // one thread per logical row
+    for (int lr = threadIdx.x; lr < n_local; lr += blockDim.x) {
+        double v = 0.0;
+        for (int p = 0; p < ntpr; p++) v += s_part[lr * ntpr + p];
+        s_val[lr] = (float)v;
+    }
+    if (EPI == EPI_SWIGLU || EPI == EPI_ROPE_KV) __syncthreads();
+    for (int lr = threadIdx.x; lr < n_local; lr += blockDim.x) {
+        const float other = (EPI == EPI_SWIGLU || EPI == EPI_ROPE_KV) ? s_val[lr ^ 1] : 0.0f;
+        finish_row<EPI, COH>(a, layer, L_lo + lr, s_val[lr], other);
+    }
+    TL(6)
+}
+
+
+// Issue the loads of tile number `wave` of a phase (what matvec_phase would do first).
+template <int TYPE, int EPI>
+__device__ __forceinline__ void matvec_prefetch(const PhaseArgs &a, int layer, int wg, Tile<TYPE> &t) {
+    constexpr int NSLOT = Tile<TYPE>::NSLOT;
+    constexpr int CPB = TYPE == L2H_TYPE_Q6_K ? 4 : 8;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int rt = a.rt, st = a.st, ntpr = a.ntpr;
+    const int64_t L_lo = (int64_t)wg * a.rows_per_wg;
+    const int64_t L_hi = min(a.n_rows, L_lo + a.rows_per_wg);
+    const int n_local = L_hi > L_lo ? (int)(L_hi - L_lo) : 0;
+    const int nchunks = (int)a.w[0].nb * CPB;
+    const int nsteps = (nchunks + WAVE - 1) / WAVE;
+    const int ntiles = ((n_local + rt - 1) / rt) * ntpr;
+    // every register of the tile is defined here, so the tile is dead before this call
+#pragma unroll
+    for (int k = 0; k < NSLOT; k++) zero_chunk(t.c[k]);
+    if (wave >= ntiles) return;
+    const int rb = wave / ntpr, sb = wave % ntpr;
+#pragma unroll
+    for (int k = 0; k < NSLOT; k++) {
+        const int ro = k / st, so = k % st;
+        const int lr = rb * rt + ro, step = sb * st + so;
+        const int ci = lane + WAVE * step;
+        if (ro < rt && lr < n_local && step < nsteps && ci < nchunks) {
+            const RowRef rr = uniform_row(logical_row<EPI>(a, L_lo + lr));
+            if (rr.seg >= 0) load_chunk<TYPE>(t.c[k], seg_ptrs(a, rr.seg, layer), rr.row, ci);
+        }
+    }
+}
+
+// Where matvec_phase left the finished fp32 row values of workgroup `wg` (LDS), and how many.
+__device__ __forceinline__ const float *matvec_phase_vals(const PhaseArgs &a, int wg, uint4 *smem, int &n_local,
+                                                          int64_t &L_lo) {
+    const int64_t K = a.w[0].ne0;
+    int8_t *s_qs = (int8_t *)smem;
+    double *s_part = (double *)(s_qs + ((K + K / 8 + K / 64 + 15) & ~(int64_t)15));
+    L_lo = (int64_t)wg * a.rows_per_wg;
+    const int64_t L_hi = min(a.n_rows, L_lo + a.rows_per_wg);
+    n_local = L_hi > L_lo ? (int)(L_hi - L_lo) : 0;
+    return (const float *)(s_part + (int64_t)a.rows_per_wg * a.ntpr);
+}

@@ -64,7 +64,7 @@ _LAYER_ROLES = [("rms_att_weight", _lib.RMS_ATT), ("rms_ffn_weight", _lib.RMS_FF
 class DeviceModel:
     """l2h_model: the weights in HBM plus the RunState (activations, KV cache)."""
 
-    def __init__(self, config, weights, ctx=None):
+    def __init__(self, config, weights, ctx=None, path=0):
         self.ctx = ctx or _lib.default_context()
         self.config = config
         cfg = _lib.Config(config.dim, config.hidden_dim, config.n_layers, config.n_heads, config.n_kv_heads,
@@ -81,7 +81,9 @@ class DeviceModel:
             for l, lw in enumerate(weights.layers):
                 for name, role in _LAYER_ROLES:
                     self._set(role, l, getattr(lw, name))
+            self.ctx.check(_lib.lib().l2h_model_set_path(self.handle, path))
             self.ctx.check(_lib.lib().l2h_model_finalize(self.handle))
+            self.path = _lib.lib().l2h_model_path(self.handle)  # 1 = kernel per phase, 2 = persistent kernel
         except Exception:
             self.close()
             raise
@@ -167,10 +169,10 @@ class LanguageModel:  # src/inference.jl:50-54
         self.config, self.tokenizer, self.weights = config, tokenizer, weights
         self._device = None
 
-    def device(self, ctx=None):
-        """Upload once; later calls reuse the resident copy."""
+    def device(self, ctx=None, path=0):
+        """Upload once; later calls reuse the resident copy.  path: see l2h_model_set_path."""
         if self._device is None:
-            self._device = DeviceModel(self.config, self.weights, ctx)
+            self._device = DeviceModel(self.config, self.weights, ctx, path)
         return self._device
 
     def __str__(self):  # src/inference.jl:56-60

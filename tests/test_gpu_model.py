@@ -38,15 +38,20 @@ CASES = {
 }
 
 
-@pytest.mark.parametrize("case", list(CASES))
-def test_forward_and_greedy(pkg, orc, case):
+# launch paths: 1 = one kernel per phase (replayed recording), 2 = persistent one-launch-per-token kernel
+PATHS = [(c, p) for c in CASES for p in (1, 2) if not (c == "f32" and p == 2)]
+
+
+@pytest.mark.parametrize("case,path", PATHS)
+def test_forward_and_greedy(pkg, orc, case, path):
     from llama2_jl_amd import synth
     plan, kw = CASES[case]
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
     prompt = synth.seeded_prompt(5, 6, cfg.vocab_size)
     n_new = min(40, cfg.seq_len - len(prompt))
-    dev = lm.device()
+    dev = lm.device(path=path)
+    assert dev.path == path
     om = orc.model_from_language_model(lm, nthreads=8)
 
     # single steps: logits of the first three positions
@@ -71,13 +76,36 @@ def test_forward_and_greedy(pkg, orc, case):
     om.reset()
     f_ids, f_logits = om.generate_greedy(prompt, n_new, orc.REFERENCE)
     agree = int(np.argmax(np.append(ids != f_ids, True)))
-    print("\n[%s] logits rel err vs oracle(q8k,fp64 sums) %.3g; vs reference float path: %d/%d tokens agree, "
-          "final-logit rel diff %.3g" % (case, err, agree, n_new, _rel(logits, f_logits)))
+    print("\n[%s path %d] logits rel err vs oracle(q8k,fp64 sums) %.3g; vs reference float path: %d/%d tokens agree, "
+          "final-logit rel diff %.3g" % (case, path, err, agree, n_new, _rel(logits, f_logits)))
     assert ids.tolist() == ref_ids.tolist(), case
     assert err <= 1e-3, case
 
 
-def test_kv_prefill_and_long_context(pkg, orc, rng):
+def test_paths_agree_bit_for_bit(pkg):
+    """Both launch paths run the same device functions: identical logits and tokens."""
+    from llama2_jl_amd import synth
+    plan, kw = CASES["q4ks_gqa"]
+    prompt = synth.seeded_prompt(8, 5, kw["vocab_size"])
+    outs = []
+    for path in (1, 2):
+        lm = _model(pkg, plan, **kw)
+        ids, logits = lm.device(path=path).generate_greedy(prompt, 30, want_logits=True)
+        outs.append((ids, logits))
+    assert outs[0][0].tolist() == outs[1][0].tolist()
+    assert np.array_equal(outs[0][1].view(np.uint32), outs[1][1].view(np.uint32))
+
+
+def test_automatic_path_choice(pkg):
+    from llama2_jl_amd import synth
+    assert _model(pkg, *[CASES["q4ks_gqa"][0]], **CASES["q4ks_gqa"][1]).device().path == 2
+    assert _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device().path == 1  # no persistent kernel for F32
+    with pytest.raises(pkg.L2HError):
+        _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device(path=2)
+
+
+@pytest.mark.parametrize("path", [1, 2])
+def test_kv_prefill_and_long_context(pkg, orc, rng, path):
     """Decode into a cache pre-filled with seeded rows through l2h_kv_write, several attention
     tiles deep, no GQA, neox RoPE."""
     from llama2_jl_amd import synth
@@ -85,7 +113,7 @@ def test_kv_prefill_and_long_context(pkg, orc, rng):
     kw = dict(kw, seq_len=512, n_layers=2)
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
-    dev = lm.device()
+    dev = lm.device(path=path)
     om = orc.model_from_language_model(lm, nthreads=8)
     dev.reset()
     om.reset()
