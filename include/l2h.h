@@ -87,7 +87,7 @@ int l2h_model_set_tensor(l2h_model *m, int role, int layer, int ggml_type, const
 /* Reads a k-quant tensor back from the device layout into GGUF block order (the repack
  * is exactly invertible); host must hold ne1 * ne0/256 blocks.  For checks. */
 int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t host_bytes);
-/* How transformer! is launched (before finalize): 0 = automatic, 1 = one kernel per phase
+/* How transformer! is launched (before finalize): 0 = automatic (currently 1), 1 = one kernel per phase
  * (recorded once, replayed per token), 2 = the persistent one-launch-per-token kernel, an error
  * at finalize if the model's tensor types have no such kernel.  Both run the same device code
  * and give the same results.  No counterpart in the reference.  l2h_model_path reports the

@@ -555,7 +555,8 @@ static int mega_setup(l2h_model *m) {
     l2h_ctx *ctx = m->ctx;
     const l2h_config &c = m->c;
     m->mega = false;
-    if (m->path_request == 1 || getenv("L2H_NO_MEGA")) return L2H_OK;
+    // automatic choice: the per-phase recording, which is the faster of the two at present
+    if (m->path_request != 2) return L2H_OK;
     const char *why = nullptr;
     const int t_qkv = m->L(0, L2H_WQ).type, t_wo = m->L(0, L2H_WO).type, t_w13 = m->L(0, L2H_W1).type,
               t_w2 = m->L(0, L2H_W2).type, t_out = m->glob[L2H_OUTPUT].type;
@@ -638,8 +639,12 @@ static hipError_t enqueue_token(l2h_model *m) {
         float *kc = m->kc + (int64_t)l * m->cache_layer_elems;
         float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
         CK(launch_qkv(m, l));
-        CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->ctl, m->hs, c.n_heads, c.n_kv_heads,
-                       c.seq_len));  // :263-278 -> xb
+        // attention (:263-278) -> xb: one launch while the sequence fits one workgroup's LDS, else split over time
+        if (c.seq_len <= 1024)
+            CK(k_attention_fused(s, m->q, m->xb, kc, vc, m->ctl, m->hs, c.n_heads, c.n_kv_heads, c.seq_len));
+        else
+            CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->ctl, m->hs, c.n_heads, c.n_kv_heads,
+                           c.seq_len));
         CK(launch_wo(m, l));
         CK(launch_w13(m, l));
         CK(launch_w2(m, l));

@@ -6,7 +6,7 @@
 // launch sequence serves every position.
 // K cache layout per layer: [n_kv_heads][hs/4][seq_len][4] (a lane per timestep reads
 // contiguous 16-byte pieces); V cache: [n_kv_heads][seq_len][hs] (a lane per feature).
-#include "dev_common.h"
+#include "matvec_dev.h"
 
 // One wavefront: 64 consecutive timesteps of GH query heads that share one KV head.
 template <int GH>
@@ -101,6 +101,26 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(const double *part, fl
     double acc = 0.0;
     for (int s = 0; s < nsplit; s++) acc += part[(int64_t)s * dim + e];
     out[e] = (float)acc;
+}
+
+// Short sequences: one workgroup per head does scores, softmax and values in one launch.
+__global__ __launch_bounds__(1024) void attn_fused_kernel(const float *q, float *xb, const float *kc, const float *vc,
+                                                          const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
+                                                          int seq_len) {
+    extern __shared__ uint4 smem[];
+    __shared__ double redd[16];
+    __shared__ float redf[16];
+    attention_head<false>(q, xb, kc, vc, hs, n_heads, n_kv_heads, seq_len, blockIdx.x, ctl->pos, smem, redd, redf);
+}
+
+hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const float *kc, const float *vc,
+                             const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads, int seq_len) {
+    const size_t lds = (size_t)head_size * 8 + (size_t)seq_len * 8 + (size_t)(1024 / head_size) * head_size * 8 +
+                       (size_t)seq_len * 4;
+    if (lds > 64 * 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_heads), dim3(1024), lds, s, q, xb, kc, vc, ctl, head_size, n_heads,
+                       n_kv_heads, seq_len);
+    return hipGetLastError();
 }
 
 template <int GH>

@@ -61,68 +61,6 @@ __device__ __forceinline__ bool grid_barrier(GridBar *b, unsigned long long gen,
     return *s_abort == 0;
 }
 
-// ------------------------------------------------------------------------------------------
-// attention of one head by one workgroup (reference src/inference.jl:263-278):
-//   att[t] = fp32(sum_fp64 q[i] K[t][i]) / sqrt(hs); softmax (exp in fp64, fp64 sum); out[i] =
-//   fp32(sum_fp64 p[t] V[t][i]).  Same arithmetic as the stand-alone attention kernels.
-// LDS: q as fp64 [hs], att fp32 [np], p fp64 [np], partial sums [blockDim/hs][hs].
-// ------------------------------------------------------------------------------------------
-__device__ __forceinline__ void attention_head(const MegaArgs &g, int layer, int h, int pos, uint4 *smem,
-                                               double *redd, float *redf) {
-    const int hs = g.hs, seq_len = g.seq_len, np = pos + 1;
-    const int kvh = h / (g.n_heads / g.n_kv_heads);
-    const float *kc = g.kc + (int64_t)layer * g.cache_layer_elems;
-    const float *vc = g.vc + (int64_t)layer * g.cache_layer_elems;
-    double *s_q = (double *)smem;
-    double *s_p = s_q + hs;
-    double *s_red = s_p + seq_len;
-    float *s_att = (float *)(s_red + (blockDim.x / hs) * hs);
-    const int tid = threadIdx.x;
-    for (int i = tid; i < hs; i += blockDim.x) s_q[i] = (double)ld_f32<true>(g.q + (int64_t)h * hs + i);
-    __syncthreads();
-    const float scale = sqrtf((float)hs);
-    float mx = -INFINITY;
-    for (int t = tid; t < np; t += blockDim.x) {
-        const float *kp = kc + ((int64_t)kvh * (hs >> 2) * seq_len + t) * 4;
-        double acc = 0.0;
-        for (int i4 = 0; i4 < (hs >> 2); i4++) {
-            const float4 kv = ld_f32x4<true>(kp + (int64_t)i4 * seq_len * 4);
-            acc = fma(s_q[4 * i4 + 0], (double)kv.x, acc);
-            acc = fma(s_q[4 * i4 + 1], (double)kv.y, acc);
-            acc = fma(s_q[4 * i4 + 2], (double)kv.z, acc);
-            acc = fma(s_q[4 * i4 + 3], (double)kv.w, acc);
-        }
-        const float a = (float)acc / scale;
-        s_att[t] = a;
-        mx = fmaxf(mx, a);
-    }
-    mx = block_max_f32(mx, redf);
-    double sum = 0.0;
-    for (int t = tid; t < np; t += blockDim.x) {
-        const float e = (float)exp((double)(s_att[t] - mx));
-        s_att[t] = e;
-        sum += (double)e;
-    }
-    const float sf = (float)block_sum_f64(sum, redd);
-    for (int t = tid; t < np; t += blockDim.x) s_p[t] = (double)(s_att[t] / sf);
-    __syncthreads();
-    const int ngrp = blockDim.x / hs;
-    const int i = tid % hs, grp = tid / hs;
-    if (grp < ngrp) {
-        const float *vp = vc + (int64_t)kvh * seq_len * hs + i;
-        double acc = 0.0;
-        for (int t = grp; t < np; t += ngrp) acc = fma(s_p[t], (double)ld_f32<true>(vp + (int64_t)t * hs), acc);
-        s_red[grp * hs + i] = acc;
-    }
-    __syncthreads();
-    if (tid < hs) {
-        double acc = 0.0;
-        for (int k = 0; k < ngrp; k++) acc += s_red[k * hs + tid];
-        st_f32<true>(g.xb + (int64_t)h * hs + tid, (float)acc);
-    }
-    __syncthreads();
-}
-
 // first-maximum key of (value, index): larger value wins, then lower index (Julia's argmax)
 __device__ __forceinline__ unsigned long long mega_argmax_key(float v, uint32_t idx) {
     uint32_t b = __float_as_uint(v);
@@ -213,7 +151,8 @@ __global__ __launch_bounds__(1024) void decode_token_kernel(MegaArgs g) {
         BARRIER();
         MTL();
         // attention: one head per workgroup
-        for (int h = wg; h < g.n_heads; h += nwg) attention_head(g, l, h, pos, smem, red, redf);
+        for (int h = wg; h < g.n_heads; h += nwg) attention_head<true>(g.q, g.xb, g.kc + (int64_t)l * g.cache_layer_elems, g.vc + (int64_t)l * g.cache_layer_elems, g.hs,
+                                                                   g.n_heads, g.n_kv_heads, g.seq_len, h, pos, smem, red, redf);
         MTL();
         BARRIER();
         MTL();

@@ -150,6 +150,9 @@ hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int 
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
                        double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads,
                        int seq_len);
+// one launch for scores + softmax + values; needs head_size*8 + seq_len*12 + 8 KiB of LDS <= 64 KiB
+hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const float *kc, const float *vc,
+                             const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads, int seq_len);
 hipError_t k_softmax(hipStream_t s, float *x, int64_t n);
 hipError_t k_argmax(hipStream_t s, const float *x, int64_t n, int64_t *partial, DecodeCtl *ctl, int32_t *out_tokens,
                     int max_out);

@@ -739,3 +739,88 @@ __device__ __forceinline__ const float *matvec_phase_vals(const PhaseArgs &a, in
     n_local = L_hi > L_lo ? (int)(L_hi - L_lo) : 0;
     return (const float *)(s_part + (int64_t)a.rows_per_wg * a.ntpr);
 }
+
+// ------------------------------------------------------------------------------------------
+// attention of one head by one workgroup (reference src/inference.jl:263-278):
+//   att[t] = fp32(sum_fp64 q[i] K[t][i]) / sqrt(hs); softmax (exp in fp64, fp64 sum); out[i] =
+//   fp32(sum_fp64 p[t] V[t][i]).  Same arithmetic as the stand-alone attention kernels.
+// LDS: q as fp64 [hs], att fp32 [np], p fp64 [np], partial sums [blockDim/hs][hs].
+// ------------------------------------------------------------------------------------------
+template <bool COH>
+__device__ __forceinline__ void attention_head(const float *q, float *xb, const float *kc, const float *vc, int hs,
+                                               int n_heads, int n_kv_heads, int seq_len, int h, int pos, uint4 *smem,
+                                               double *redd, float *redf) {
+    const int np = pos + 1;
+    const int kvh = h / (n_heads / n_kv_heads);
+    double *s_q = (double *)smem;
+    double *s_p = s_q + hs;
+    double *s_red = s_p + seq_len;
+    float *s_att = (float *)(s_red + (blockDim.x / hs) * hs);
+    const int tid = threadIdx.x;
+    for (int i = tid; i < hs; i += blockDim.x) s_q[i] = (double)ld_f32<COH>(q + (int64_t)h * hs + i);
+    __syncthreads();
+    const float scale = sqrtf((float)hs);
+    float mx = -INFINITY;
+    for (int t = tid; t < np; t += blockDim.x) {
+        const float *kp = kc + ((int64_t)kvh * (hs >> 2) * seq_len + t) * 4;
+        double acc = 0.0;
+        // four independent 16-byte loads in flight per step (hs is a multiple of 16 for 64/96/128)
+        int i4 = 0;
+        for (; i4 + 4 <= (hs >> 2); i4 += 4) {
+            float4 kv[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) kv[u] = ld_f32x4<COH>(kp + (int64_t)(i4 + u) * seq_len * 4);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                acc = fma(s_q[4 * (i4 + u) + 0], (double)kv[u].x, acc);
+                acc = fma(s_q[4 * (i4 + u) + 1], (double)kv[u].y, acc);
+                acc = fma(s_q[4 * (i4 + u) + 2], (double)kv[u].z, acc);
+                acc = fma(s_q[4 * (i4 + u) + 3], (double)kv[u].w, acc);
+            }
+        }
+        for (; i4 < (hs >> 2); i4++) {
+            const float4 kv = ld_f32x4<COH>(kp + (int64_t)i4 * seq_len * 4);
+            acc = fma(s_q[4 * i4 + 0], (double)kv.x, acc);
+            acc = fma(s_q[4 * i4 + 1], (double)kv.y, acc);
+            acc = fma(s_q[4 * i4 + 2], (double)kv.z, acc);
+            acc = fma(s_q[4 * i4 + 3], (double)kv.w, acc);
+        }
+        const float a = (float)acc / scale;
+        s_att[t] = a;
+        mx = fmaxf(mx, a);
+    }
+    mx = block_max_f32(mx, redf);
+    double sum = 0.0;
+    for (int t = tid; t < np; t += blockDim.x) {
+        const float e = (float)exp((double)(s_att[t] - mx));
+        s_att[t] = e;
+        sum += (double)e;
+    }
+    const float sf = (float)block_sum_f64(sum, redd);
+    for (int t = tid; t < np; t += blockDim.x) s_p[t] = (double)(s_att[t] / sf);
+    __syncthreads();
+    const int ngrp = blockDim.x / hs;
+    const int i = tid % hs, grp = tid / hs;
+    if (grp < ngrp) {
+        const float *vp = vc + (int64_t)kvh * seq_len * hs + i;
+        double acc = 0.0;
+        int t = grp;
+        for (; t + 3 * ngrp < np; t += 4 * ngrp) {  // four loads in flight
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = ld_f32<COH>(vp + (int64_t)(t + u * ngrp) * hs);
+#pragma unroll
+            for (int u = 0; u < 4; u++) acc = fma(s_p[t + u * ngrp], (double)v[u], acc);
+        }
+        for (; t < np; t += ngrp) acc = fma(s_p[t], (double)ld_f32<COH>(vp + (int64_t)t * hs), acc);
+        s_red[grp * hs + i] = acc;
+    }
+    __syncthreads();
+    if (tid < hs) {
+        double acc = 0.0;
+        for (int k = 0; k < ngrp; k++) acc += s_red[k * hs + tid];
+        st_f32<COH>(xb + (int64_t)h * hs + tid, (float)acc);
+    }
+    __syncthreads();
+}
+

