@@ -1,0 +1,233 @@
+"""Pins the CPU oracle (oracle/l2c.c).  The reference ships no tests or vectors, so the oracle is
+checked against (1) hand-built blocks with closed-form expected values (tests/golden), (2) an
+independent numpy restatement written from the same Julia text (tests/np_ref.py), (3) identities
+the reference implies (vecdot == dot(dequantize)), (4) float64 closed forms of every operator and
+of the whole transformer, (5) closed-form properties of the q8_K quantizer and brute force for
+the integer dot products.  No GPU needed.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import np_ref
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+Q4, Q5, Q6, F32 = 12, 13, 14, 0
+BB = {Q4: 144, Q5: 176, Q6: 210}
+
+
+def rand_blocks(rng, typ, n):
+    raw = rng.integers(0, 256, size=(n, BB[typ]), dtype=np.uint8)
+    d = rng.uniform(-0.02, 0.02, size=(n, 2)).astype(np.float16).view(np.uint8)
+    if typ == Q6:
+        raw[:, 208:210] = d[:, :2]
+    else:
+        raw[:, 0:4] = d
+    return raw.reshape(-1)
+
+
+def rel(a, b):
+    return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64))) / max(1e-30, np.max(np.abs(b))))
+
+
+def test_block_sizes(orc):
+    # src/kquants.jl:7-42
+    assert [orc.lib().l2c_block_bytes(t) for t in (F32, Q4, Q5, Q6)] == [4, 144, 176, 210]
+    assert orc.block_q8_K.itemsize == 292 and np_ref.q8_dtype.itemsize == 292
+    assert np_ref.q4_dtype.itemsize == 144 and np_ref.q5_dtype.itemsize == 176 and np_ref.q6_dtype.itemsize == 210
+
+
+def test_golden_vectors(orc):
+    vecs = json.load(open(os.path.join(HERE, "golden", "kquant_vectors.json")))
+    assert len(vecs) >= 7
+    for v in vecs:
+        raw = np.frombuffer(bytes.fromhex(v["raw"]), np.uint8)
+        want = np.array(v["expected"], np.float32)
+        got = orc.dequantize(v["type"], raw)
+        assert np.array_equal(got, want), v["name"]
+        assert np.array_equal(np_ref.DEQUANT[v["type"]](raw), want), v["name"] + " (numpy restatement)"
+
+
+def test_fp16_conversion_exhaustive(orc):
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([orc.lib().l2c_fp16_to_fp32(int(x)) for x in h], np.float32)
+    ok = np.isnan(want) | (got.view(np.uint32) == want.view(np.uint32))
+    assert ok.all()
+
+
+def test_scale_unpack_every_bit(orc, rng):
+    """Toggle each of the 96 bits of the packed scales alone: exactly one 6-bit field changes."""
+    import ctypes
+    base = np.zeros(12, np.uint8)
+    sc, m = np.zeros(8, np.uint8), np.zeros(8, np.uint8)
+    for bit in range(96):
+        p = base.copy()
+        p[bit // 8] = 1 << (bit % 8)
+        orc.lib().l2c_scale_min_k4(p.ctypes.data_as(ctypes.c_void_p), sc.ctypes.data_as(ctypes.c_void_p),
+                                   m.ctypes.data_as(ctypes.c_void_p))
+        rsc, rm = np_ref.scales_k4(p[None])
+        assert np.array_equal(sc, rsc[0]) and np.array_equal(m, rm[0])
+        assert np.count_nonzero(sc) + np.count_nonzero(m) == 1
+    for _ in range(200):
+        p = rng.integers(0, 256, 12, dtype=np.uint8)
+        orc.lib().l2c_scale_min_k4(p.ctypes.data_as(ctypes.c_void_p), sc.ctypes.data_as(ctypes.c_void_p),
+                                   m.ctypes.data_as(ctypes.c_void_p))
+        rsc, rm = np_ref.scales_k4(p[None])
+        assert np.array_equal(sc, rsc[0]) and np.array_equal(m, rm[0]) and sc.max() < 64 and m.max() < 64
+
+
+@pytest.mark.parametrize("typ", [Q4, Q5, Q6])
+def test_dequantize_matches_numpy_restatement(orc, rng, typ):
+    raw = rand_blocks(rng, typ, 4000)
+    assert np.array_equal(orc.dequantize(typ, raw).view(np.uint32), np_ref.DEQUANT[typ](raw).view(np.uint32))
+
+
+@pytest.mark.parametrize("typ", [Q4, Q5, Q6])
+def test_vecdot_is_dot_of_dequantized(orc, rng, typ):
+    """The reference states the weight expression twice, in dequantize! and in vecdot
+    (src/kquants.jl:93 vs :152 etc.): vecdot(x, y) == dot(dequantize(x), y)."""
+    nb = 16
+    raw = rand_blocks(rng, typ, nb)
+    y = rng.standard_normal(nb * 256).astype(np.float32)
+    w = orc.dequantize(typ, raw)
+    exact = float(np.dot(w.astype(np.float64), y.astype(np.float64)))
+    assert orc.vecdot_f32act(typ, raw, y, canon=1) == np.float32(exact)
+    seq = np.float32(0)
+    for a, b in zip(w, y):
+        seq = np.float32(seq + np.float32(b * a))
+    assert orc.vecdot_f32act(typ, raw, y, canon=0) == seq
+    assert abs(orc.vecdot_f32act(typ, raw, y, canon=0) - exact) <= 1e-4 * np.abs(w * y).sum()
+
+
+def test_q8k_properties(orc, rng):
+    x = (rng.standard_normal(256 * 50) * rng.uniform(0.01, 100, 50).repeat(256)).astype(np.float32)
+    x[256 * 3:256 * 4] = 0
+    i, j = 256 * 5 + 7, 256 * 5 + 100  # tie of the extreme inside block 5: the first (negative) one fixes the sign
+    x[256 * 5:256 * 6] = rng.uniform(-1, 1, 256)
+    x[i], x[j] = -3.0, 3.0
+    q = orc.quantize_q8_K(x)
+    assert q.tobytes() == np_ref.quantize_q8(x).tobytes()
+    for b in range(50):
+        blk = x[256 * b:256 * b + 256]
+        if not blk.any():
+            assert q[b]["d"] == 0 and not q[b]["qs"].any() and not q[b]["bsums"].any()
+            continue
+        k = int(np.argmax(np.abs(blk)))
+        assert q[b]["qs"][k] == -127  # iscale = -127/max maps the extreme to -127
+        assert np.all(np.abs(q[b]["qs"].astype(np.float64) * q[b]["d"] - blk) <= abs(q[b]["d"]) * 0.5000001)
+        assert np.array_equal(q[b]["bsums"], q[b]["qs"].astype(np.int32).reshape(16, 16).sum(1))
+        assert np.sign(q[b]["d"]) == -np.sign(blk[k])
+    assert q[5]["qs"][7] == -127 and q[5]["qs"][100] == 127 and q[5]["d"] > 0
+
+
+@pytest.mark.parametrize("typ", [Q4, Q5, Q6])
+def test_integer_dots_brute_force(orc, rng, typ):
+    nb = 24
+    raw = rand_blocks(rng, typ, nb)
+    x = rng.standard_normal(nb * 256).astype(np.float32)
+    q8 = orc.quantize_q8_K(x)
+    v, isc, imin = orc.vecdot_q8k(typ, raw, q8, canon=1)
+    w_isc, w_imin = np_ref.block_ints(typ, raw, q8)
+    assert np.array_equal(isc, w_isc) and np.array_equal(imin, w_imin)
+    assert np.float32(v) == np_ref.vecdot_q8(typ, raw, q8)
+    # the q8_K path approximates the float path to the quantization step of the activations
+    f = orc.vecdot_f32act(typ, raw, x, canon=1)
+    w = orc.dequantize(typ, raw)
+    assert abs(v - f) <= 0.02 * np.sqrt((w.astype(np.float64) ** 2).sum()) * np.abs(x).max() / 127 * 16
+
+
+def test_matmul_rows_and_threads(orc, rng):
+    ne0, ne1 = 512, 37
+    raw = rand_blocks(rng, Q4, ne1 * 2)
+    x = rng.standard_normal(ne0).astype(np.float32)
+    for mode in (0, 1, 2, 3):
+        y1 = orc.matmul(Q4, raw, ne0, ne1, x, mode, nthreads=1)
+        y8 = orc.matmul(Q4, raw, ne0, ne1, x, mode, nthreads=8)
+        assert np.array_equal(y1.view(np.uint32), y8.view(np.uint32))  # rows are independent (src/matmul.jl:18)
+    rb = 2 * 144
+    for i in (0, 17, 36):
+        assert orc.matmul(Q4, raw, ne0, ne1, x, 0)[i] == np.float32(orc.vecdot_f32act(Q4, raw[i * rb:(i + 1) * rb], x, 0))
+    A = rng.standard_normal((ne1, ne0)).astype(np.float32)
+    assert rel(orc.matmul(F32, A, ne0, ne1, x, 0), A.astype(np.float64) @ x) < 1e-5
+    assert np.array_equal(orc.matmul(F32, A, ne0, ne1, x, 2), (A.astype(np.float64) @ x.astype(np.float64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_operators_against_float64(orc, rng, mode):
+    x = (rng.standard_normal(1376) * 3).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 1376).astype(np.float32)
+    assert rel(orc.rmsnorm(x, w, mode), np_ref.rmsnorm(x, w)) < 2e-6
+    for hs, neox, base in ((64, 0, 1e4), (128, 0, 5e5), (96, 1, 1e4)):
+        v = rng.standard_normal(hs * 3).astype(np.float32)
+        for pos in (0, 1, 100, 4095):
+            # the reference advances theta by repeated fp32 multiplication (src/inference.jl:126), so at
+            # large positions the angle itself carries fp32 round-off: ~pos * 1e-7 absolute
+            tol = 2e-6 + 4e-7 * pos
+            assert rel(orc.rope(v, hs, 3, pos, base, neox, mode), np_ref.rope(v, hs, pos, base, neox)) < tol
+    s = (rng.standard_normal(333) * 5).astype(np.float32)
+    assert rel(orc.softmax(s, mode), np_ref.softmax(s)) < 2e-6
+    a, b = (rng.standard_normal(500) * 4).astype(np.float32), rng.standard_normal(500).astype(np.float32)
+    assert rel(orc.swiglu(a, b, mode), np_ref.swiglu(a, b)) < 2e-6
+    for hs, nh, nkv, pos in ((64, 8, 8, 0), (128, 8, 2, 37), (96, 6, 6, 130), (64, 6, 2, 5)):
+        q = rng.standard_normal(hs * nh).astype(np.float32)
+        kc = rng.standard_normal((pos + 1, hs * nkv)).astype(np.float32)
+        vc = rng.standard_normal((pos + 1, hs * nkv)).astype(np.float32)
+        out, att = orc.attention(q, kc, vc, hs, nh, nkv, pos, mode)
+        assert rel(out, np_ref.attention(q, kc, vc, hs, nh, nkv)) < 5e-6
+        assert np.allclose(att.sum(1), 1, atol=1e-5)
+
+
+def test_argmax_first_maximum(orc):
+    assert orc.argmax(np.array([1, 5, 5, 2], np.float32)) == 1
+    assert orc.argmax(np.array([-3, -1, -1], np.float32)) == 1
+    assert orc.argmax(np.array([7], np.float32)) == 0
+
+
+def _f32_model(rng, cfg):
+    L, dim, hid = cfg["n_layers"], cfg["dim"], cfg["hidden_dim"]
+    kv_dim = dim // cfg["n_heads"] * cfg["n_kv_heads"]
+    g = lambda *s: (rng.standard_normal(s) * 0.05).astype(np.float32)
+    W = dict(emb=g(cfg["vocab_size"], dim), output=g(cfg["vocab_size"], dim),
+             rms_final=rng.uniform(0.8, 1.2, dim).astype(np.float32),
+             rms_att=[rng.uniform(0.8, 1.2, dim).astype(np.float32) for _ in range(L)],
+             rms_ffn=[rng.uniform(0.8, 1.2, dim).astype(np.float32) for _ in range(L)],
+             wq=[g(dim, dim) for _ in range(L)], wk=[g(kv_dim, dim) for _ in range(L)],
+             wv=[g(kv_dim, dim) for _ in range(L)], wo=[g(dim, dim) for _ in range(L)],
+             w1=[g(hid, dim) for _ in range(L)], w2=[g(dim, hid) for _ in range(L)], w3=[g(hid, dim) for _ in range(L)])
+    return W
+
+
+@pytest.mark.parametrize("neox,n_kv", [(False, 4), (True, 2)])
+def test_transformer_against_float64(orc, rng, neox, n_kv):
+    """l2c_forward (layer order, residuals, KV cache, GQA head map, both RoPE styles) against a float64
+    numpy transformer written from src/inference.jl:222-315."""
+    cfg = dict(dim=64, hidden_dim=96, n_layers=3, n_heads=4, n_kv_heads=n_kv, vocab_size=50, seq_len=16,
+               rope_freq_base=10000.0, rope_is_neox=neox)
+    W = _f32_model(rng, cfg)
+    T = {}
+    def put(role, layer, a):
+        a = np.ascontiguousarray(a, np.float32)
+        T[(role, layer)] = (F32, a, a.shape[-1], 1 if a.ndim == 1 else a.shape[0])
+    put(orc.TOK_EMB, 0, W["emb"]); put(orc.RMS_FINAL, 0, W["rms_final"]); put(orc.OUTPUT, 0, W["output"])
+    for l in range(cfg["n_layers"]):
+        for role, name in ((orc.RMS_ATT, "rms_att"), (orc.RMS_FFN, "rms_ffn"), (orc.WQ, "wq"), (orc.WK, "wk"),
+                           (orc.WV, "wv"), (orc.WO, "wo"), (orc.W1, "w1"), (orc.W2, "w2"), (orc.W3, "w3")):
+            put(role, l, W[name][l])
+    m = orc.Model(cfg, T)
+    tokens = [3, 17, 42, 8, 8, 1]
+    want = np_ref.transformer_f32(cfg, W, tokens)
+    for mode in (0, 2):
+        m.reset()
+        for pos, tok in enumerate(tokens):
+            got = m.forward(tok, pos, mode)
+            assert rel(got, want[pos]) < 2e-5, (mode, pos)
+    # the greedy loop: prompt tokens are fed, then argmax (src/inference.jl:349-386)
+    m.reset()
+    ids, _ = m.generate_greedy(tokens[:3], 4, 2)
+    seq = tokens[:3]
+    for _ in range(4):
+        seq = seq + [int(np.argmax(np_ref.transformer_f32(cfg, W, seq)[-1]))]
+    assert ids.tolist() == seq[3:]
