@@ -23,6 +23,7 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"8b-q4ks": 31264000}  # 31.23 MB read + 0.04 MB written
 
 WORKLOADS = {
     # name: (plan, config kwargs, prompt length)
@@ -152,6 +153,10 @@ def main():
         log("cpu baseline:", cpu)
         om.close()
 
+    # HBM traffic of the dominant kernel per launch (FETCH_SIZE + WRITE_SIZE, scaled), measured with
+    # rocprofv3 --pmc on this workload: profiles/pmc_fetch_write_bench_8b-q4ks.md
+    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
+
     result = {
         "metric": "decode tok/s, Llama-3-8B-shape Q4_K_S, batch 1; % of HBM-BW roofline",
         "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": K, "warmup": W,
@@ -166,7 +171,7 @@ def main():
                    "tokens_head": tokens[:8]},
         "roofline": {"bound": "hbm", "kernel": "matvec_kq_kernel (k-quant x q8_K dequant-matvec)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "bytes_per_launch": int(tot_b / max(1, n_launch)), "launches_per_token": n_launch,
                      "avg_launch_us": round(tot_us / max(1, n_launch), 2), "per_launch": per_kernel,
                      "measured_stream_read_GBs": round(stream_gbs, 1)},

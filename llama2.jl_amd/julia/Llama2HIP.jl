@@ -1,0 +1,156 @@
+# Llama2HIP.jl -- Julia binding of libl2hip.so for Llama2.jl users.
+#
+# Keeps the package surface of Llama2.jl (load_gguf_model, load_karpathy_model, LanguageModel,
+# sample): the loaders and tokenizers are Llama2.jl's own; only the per-token forward pass and the
+# greedy loop run on the GPU through `ccall`.  Token ids and positions are 1-based on this side and
+# 0-based in the C ABI (include/l2h.h).
+#
+# NOT EXERCISED BY THE TEST SUITE: no Julia toolchain is available where this library is built and
+# tested; the Python binding (llama2.jl_amd/_lib.py) calls the same symbols and is the tested one.
+module Llama2HIP
+
+using Llama2
+using Llama2: LanguageModel, ModelConfig, TransformerWeights, TransformerLayerWeights,
+              block_q4_K, block_q5_K, block_q6_K, encode
+
+const lib = get(ENV, "L2H_LIB", joinpath(@__DIR__, "..", "libl2hip.so"))
+
+struct L2HConfig            # l2h_config
+    dim::Int32; hidden_dim::Int32; n_layers::Int32; n_heads::Int32; n_kv_heads::Int32
+    vocab_size::Int32; seq_len::Int32; rope_freq_base::Float32; rope_is_neox::Int32
+end
+
+# tensor roles and GGML types of include/l2h.h
+const TOK_EMB, RMS_FINAL, OUTPUT, RMS_ATT, RMS_FFN, WQ, WK, WV, WO, W1, W2, W3 = 0:11
+ggml_type(::AbstractArray{Float32}) = 0
+ggml_type(::AbstractArray{block_q4_K}) = 12
+ggml_type(::AbstractArray{block_q5_K}) = 13
+ggml_type(::AbstractArray{block_q6_K}) = 14
+
+mutable struct Context
+    handle::Ptr{Cvoid}
+end
+
+function check(ctx::Ptr{Cvoid}, rc::Cint)
+    rc == 0 && return
+    msg = unsafe_string(ccall((:l2h_last_error, lib), Cstring, (Ptr{Cvoid},), ctx))
+    error("l2h error $rc: $msg")
+end
+
+function Context(device::Integer = 0)
+    h = Ref{Ptr{Cvoid}}(C_NULL)
+    rc = ccall((:l2h_ctx_create, lib), Cint, (Cint, Ref{Ptr{Cvoid}}), device, h)
+    check(Ptr{Cvoid}(C_NULL), rc)
+    ctx = Context(h[])
+    finalizer(c -> ccall((:l2h_ctx_destroy, lib), Cvoid, (Ptr{Cvoid},), c.handle), ctx)
+    return ctx
+end
+
+mutable struct DeviceModel
+    ctx::Context
+    handle::Ptr{Cvoid}
+    config::ModelConfig
+end
+
+# (in_features, out_rows) of a weight as matmul! sees it; k-quant arrays hold in/256 blocks per row
+in_out(A::AbstractMatrix{Float32}) = size(A)
+in_out(A::AbstractMatrix) = (size(A, 1) * 256, size(A, 2))
+in_out(v::AbstractVector{Float32}) = (length(v), 1)
+
+function set_tensor!(m::DeviceModel, role, layer, A)
+    host = A isa Array ? A : collect(A)          # views (Phi-3 fused tensors) and mmaps become dense
+    ne0, ne1 = in_out(host)
+    GC.@preserve host begin
+        rc = ccall((:l2h_model_set_tensor, lib), Cint,
+                   (Ptr{Cvoid}, Cint, Cint, Cint, Ptr{Cvoid}, Int64, Int64),
+                   m.handle, role, layer, ggml_type(host), pointer(host), ne0, ne1)
+    end
+    check(m.ctx.handle, rc)
+end
+
+"Upload the weights of a Llama2.jl `LanguageModel` once; the copy stays resident in HBM."
+function DeviceModel(model::LanguageModel; ctx::Context = Context(), seq_len::Integer = model.config.seq_len)
+    c = model.config
+    cfg = L2HConfig(c.dim, c.hidden_dim, c.n_layers, c.n_heads, c.n_kv_heads, c.vocab_size, seq_len,
+                    c.rope_freq_base, c.rope_is_neox ? 1 : 0)
+    h = Ref{Ptr{Cvoid}}(C_NULL)
+    check(ctx.handle, ccall((:l2h_model_create, lib), Cint, (Ptr{Cvoid}, Ref{L2HConfig}, Ref{Ptr{Cvoid}}),
+                            ctx.handle, cfg, h))
+    m = DeviceModel(ctx, h[], c)
+    finalizer(x -> ccall((:l2h_model_destroy, lib), Cvoid, (Ptr{Cvoid},), x.handle), m)
+    w = model.weights
+    set_tensor!(m, TOK_EMB, 0, w.token_embedding_table)
+    set_tensor!(m, RMS_FINAL, 0, w.rms_final_weight)
+    set_tensor!(m, OUTPUT, 0, w.output_weight)
+    for (l, lw) in enumerate(w.layers)
+        for (role, A) in ((RMS_ATT, lw.rms_att_weight), (RMS_FFN, lw.rms_ffn_weight), (WQ, lw.wq), (WK, lw.wk),
+                          (WV, lw.wv), (WO, lw.wo), (W1, lw.w1), (W2, lw.w2), (W3, lw.w3))
+            set_tensor!(m, role, l - 1, A)
+        end
+    end
+    check(ctx.handle, ccall((:l2h_model_finalize, lib), Cint, (Ptr{Cvoid},), m.handle))
+    return m
+end
+
+reset!(m::DeviceModel) = check(m.ctx.handle, ccall((:l2h_state_reset, lib), Cint, (Ptr{Cvoid},), m.handle))
+
+"transformer!(token, pos, ...) of Llama2.jl (src/inference.jl:222): fills `logits`, returns argmax (1-based)."
+function transformer!(logits::Vector{Float32}, m::DeviceModel, token::Int, pos::Int)
+    am = Ref{Int32}(0)
+    check(m.ctx.handle, ccall((:l2h_forward, lib), Cint, (Ptr{Cvoid}, Cint, Cint, Ptr{Float32}, Ref{Int32}),
+                              m.handle, token - 1, pos - 1, logits, am))
+    return Int(am[]) + 1
+end
+
+"Greedy continuation of 1-based token ids entirely on the device (the loop of sample() at temperature 0)."
+function generate(m::DeviceModel, prompt::Vector{Int}, n_new::Int; pos::Int = 1)
+    p = Int32.(prompt .- 1)
+    out = Vector{Int32}(undef, n_new)
+    check(m.ctx.handle, ccall((:l2h_generate_greedy, lib), Cint,
+                              (Ptr{Cvoid}, Ptr{Int32}, Cint, Cint, Cint, Ptr{Int32}, Ptr{Float32}),
+                              m.handle, p, length(p), pos - 1, n_new, out, C_NULL))
+    return Int.(out) .+ 1
+end
+
+"""
+    sample(m::DeviceModel, model::LanguageModel, prompt=""; temperature=0.9f0, stop_on_special_token=true,
+           max_seq_len=typemax(Int), bos_token=true)
+
+Same behaviour and output as `Llama2.sample` (src/inference.jl:317-395).
+"""
+function sample(m::DeviceModel, model::LanguageModel, prompt::String = ""; temperature::Float32 = 0.9f0,
+                stop_on_special_token = true, max_seq_len = typemax(Int), bos_token = true)
+    !bos_token && isempty(prompt) && error("Prompt cannot be empty if bos_token = false")
+    config, tokenizer = model.config, model.tokenizer
+    prompt_tokens = encode(prompt, tokenizer)
+    reset!(m)
+    logits = Vector{Float32}(undef, config.vocab_size)
+    time_start = time_ns()
+    bos_token && pushfirst!(prompt_tokens, tokenizer.bos_token_id)
+    !bos_token && print(tokenizer.id_to_token[prompt_tokens[1]])
+    token = prompt_tokens[1]
+    generated_seq_len = 0
+    for pos in 1:min(config.seq_len, max_seq_len)
+        am = transformer!(logits, m, token, pos)
+        generated_seq_len += 1
+        if pos + 1 <= length(prompt_tokens)
+            next = prompt_tokens[pos + 1]
+        elseif temperature == 0f0
+            next = am
+        else
+            logits ./= temperature
+            Llama2.softmax!(logits)
+            next = Llama2.wsample(1:config.vocab_size, logits)
+        end
+        if stop_on_special_token && (next == tokenizer.bos_token_id || next == tokenizer.eos_token_id)
+            break
+        end
+        print(tokenizer.id_to_token[next])
+        token = next
+    end
+    println()
+    println("-------\nachieved tok/s: ", round(generated_seq_len / (time_ns() - time_start) * 1e9; digits = 2))
+    return nothing
+end
+
+end # module
