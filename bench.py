@@ -33,6 +33,9 @@ WORKLOADS = {
                                     vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
     "llama2c-f32": ("PLAN_F32", dict(dim=512, hidden_dim=1376, n_layers=8, n_heads=8, n_kv_heads=8, vocab_size=32000,
                                      seq_len=1024, rope_freq_base=10000.0, rope_is_neox=False), 16),
+    # Phi-3-mini shape, no GQA, neox RoPE, 4096-long cache pre-filled with 3840 seeded rows: attention-dominated
+    "phi3-4k": ("PLAN_Q4_K", dict(dim=3072, hidden_dim=8192, n_layers=32, n_heads=32, n_kv_heads=32, vocab_size=32064,
+                                  seq_len=4096, rope_freq_base=10000.0, rope_is_neox=True), 3841),
     # small shape for a quick functional run of this script
     "tiny-q4ks": ("PLAN_Q4_K_S", dict(dim=512, hidden_dim=1024, n_layers=4, n_heads=8, n_kv_heads=2, vocab_size=2048,
                                       seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
@@ -81,14 +84,24 @@ def main():
 
     w_bytes = synth.weight_bytes_per_token(lm)
     kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads
-    prompt = synth.seeded_prompt(99, n_prompt, cfg.vocab_size)
+    # a prompt longer than 256 stands for a pre-filled cache: all but its last position are written
+    # as seeded random K/V rows, and a single prompt token is fed at the next position
+    n_pre = n_prompt - 1 if n_prompt > 256 else 0
+    prompt = synth.seeded_prompt(99, n_prompt - n_pre, cfg.vocab_size)
+    if n_pre:
+        rng = np.random.default_rng(7)
+        for layer in range(cfg.n_layers):
+            kv = rng.standard_normal((2, n_pre, kv_dim), dtype=np.float32)
+            dev.kv_write(layer, 0, kv[0], kv[1])
+        log("cache pre-filled with %d positions" % n_pre)
 
     # ---- timed region: K decode tokens after the prompt and W warm-up tokens --------------------
     times, tokens = [], None
     for rep in range(args.repeats):
-        dev.reset()
+        if not n_pre:
+            dev.reset()
         # prompt + warm-up tokens, untimed
-        warm = dev.generate_greedy(prompt, W) if W > 0 else np.zeros(0, np.int32)
+        warm = dev.generate_greedy(prompt, W, pos0=n_pre) if W > 0 else np.zeros(0, np.int32)
         # next step: position pos0, fed with the last warm-up token (or the last prompt token)
         pos0 = n_prompt - 1 + W
         first = int(warm[-1]) if W > 0 else int(prompt[-1])
@@ -143,7 +156,7 @@ def main():
         n_tok, t_cpu = 0, 0.0
         t_begin = time.perf_counter()
         while n_tok < 16 and (n_tok < 2 or t_cpu < args.cpu_seconds):
-            om.forward(int(prompt[n_tok % n_prompt]), n_tok, orc.REFERENCE)
+            om.forward(int(prompt[n_tok % len(prompt)]), n_tok, orc.REFERENCE)
             n_tok += 1
             t_cpu = time.perf_counter() - t_begin
         cpu = {"value": round(n_tok / t_cpu, 3), "unit": "tok/s", "cores": cores, "kind": "port",

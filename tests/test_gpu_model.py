@@ -82,6 +82,23 @@ def test_forward_and_greedy(pkg, orc, case, path):
     assert err <= 1e-3, case
 
 
+def test_headline_shape_128_greedy_tokens(pkg, orc):
+    """The headline bar at the headline widths (dim 4096, hidden 14336, 32/8 heads of 128, q4_K layers,
+    q6_K output), two layers deep so that the CPU side finishes in seconds: 128 greedy tokens from a
+    32-token prompt identical to the oracle's, final logits within 1e-3."""
+    from llama2_jl_amd import synth
+    kw = dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=32000, seq_len=192,
+              rope_freq_base=500000.0, rope_is_neox=False)
+    lm = _model(pkg, "PLAN_Q4_K_S", **kw)
+    prompt = synth.seeded_prompt(99, 32, kw["vocab_size"])
+    dev = lm.device()
+    om = orc.model_from_language_model(lm, nthreads=16)
+    ids, logits = dev.generate_greedy(prompt, 128, want_logits=True)
+    ref_ids, ref_logits = om.generate_greedy(prompt, 128, orc.GPU_SPEC)
+    assert ids.tolist() == ref_ids.tolist()
+    assert _rel(logits, ref_logits) <= 1e-3
+
+
 def test_paths_agree_bit_for_bit(pkg):
     """Both launch paths run the same device functions: identical logits and tokens."""
     from llama2_jl_amd import synth
