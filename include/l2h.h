@@ -118,6 +118,16 @@ int l2h_generate_greedy(l2h_model *m, const int32_t *prompt, int n_prompt, int p
  * measured with HIP events on the context's stream. */
 int l2h_generate_greedy_timed(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new,
                               int32_t *out, float *decode_ms);
+/* Batched prompt pass: positions pos0..pos0+n-1 of tokens[0..n) in one go.  The reference has no
+ * batched path; the result is defined as what calling transformer! (src/inference.jl:222-315) for
+ * these positions in turn leaves behind: the K/V cache rows pos0..pos0+n-1 of every layer, the
+ * logits of the last position (last_logits, may be NULL) and their argmax (next_token, may be
+ * NULL).  Matrix products run as bf16 x bf16 -> fp32 on the matrix cores (weights dequantized with
+ * the reference's fp32 expressions, then rounded to bf16; float activations, no q8_K step), so the
+ * result matches the per-token path to bf16 accuracy, not bit for bit.  Positions before pos0 must
+ * already be in the cache.  Decoding continues with l2h_generate_greedy(&next, 1, pos0+n, ...).
+ * Needs head size 32/64/96/128, dim and hidden_dim multiples of 8, w1 and w3 of one type. */
+int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0, float *last_logits, int32_t *next_token);
 /* Copies an activation of the last forward call: which = 0 x, 1 xb, 2 q (rotated), 5 hb,
  * 6 logits (RunState fields, src/inference.jl:72-86; k and v go straight into the cache). */
 int l2h_state_read(l2h_model *m, int which, float *host, int64_t n);

@@ -229,6 +229,11 @@ struct l2h_model {
 #ifdef L2H_TIMELINE
     long long *timeline = nullptr, *timeline2 = nullptr;
 #endif
+    // batched prompt pass: buffers for pf_cap positions, allocated at the first l2h_prefill
+    int pf_cap = 0;
+    float *pf_x = nullptr, *pf_raw = nullptr, *pf_cs = nullptr;
+    uint16_t *pf_xn = nullptr, *pf_q = nullptr, *pf_att = nullptr, *pf_hb = nullptr;
+    int32_t *pf_tok = nullptr;
     std::vector<void *> allocs;
 
     DevTensor &L(int layer_idx, int role) { return layer[(size_t)layer_idx * L2H_N_ROLES + role]; }
@@ -276,6 +281,7 @@ static void model_free_state(l2h_model *m) {
     m->graph = nullptr;
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
+    m->pf_cap = 0;
     m->finalized = false;
 }
 
@@ -838,6 +844,119 @@ static int generate_impl(l2h_model *m, const int32_t *prompt, int n_prompt, int 
                                    ctx->stream));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     return mega_check(m);
+}
+
+// ---- batched prompt pass --------------------------------------------------------------------
+#define L2H_PREFILL_CHUNK 2048
+
+static int prefill_buffers(l2h_model *m, int cap) {
+    if (m->pf_cap >= cap) return L2H_OK;
+    const l2h_config &c = m->c;
+    int rc;
+    // earlier, smaller buffers stay in the allocation list and are released with the model
+#define DA(p, n)                            \
+    if ((rc = dalloc(m, &(p), (n), false))) \
+        return rc;
+    DA(m->pf_x, (int64_t)cap * c.dim);
+    DA(m->pf_raw, (int64_t)cap * (c.dim + 2 * m->kv_dim));
+    DA(m->pf_cs, (int64_t)cap * m->hs);
+    DA(m->pf_xn, (int64_t)cap * c.dim);
+    DA(m->pf_q, (int64_t)cap * c.dim);
+    DA(m->pf_att, (int64_t)cap * c.dim);
+    DA(m->pf_hb, (int64_t)cap * c.hidden_dim);
+    DA(m->pf_tok, cap);
+#undef DA
+    m->pf_cap = cap;
+    return L2H_OK;
+}
+
+static hipError_t prefill_chunk(l2h_model *m, int M, int pos0) {
+    hipStream_t s = m->ctx->stream;
+    const l2h_config &c = m->c;
+    const int dim = c.dim, kvd = m->kv_dim;
+    hipError_t e;
+#define CK(call)                       \
+    do {                               \
+        e = (call);                    \
+        if (e != hipSuccess) return e; \
+    } while (0)
+    CK(k_pf_embed(s, m->glob[L2H_TOK_EMB], m->pf_tok, m->pf_x, M));
+    CK(k_pf_rope_table(s, m->pf_cs, pos0, M, m->hs / 2, m->theta_scale));
+    for (int l = 0; l < c.n_layers; l++) {
+        float *kc = m->kc + (int64_t)l * m->cache_layer_elems;
+        float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
+        CK(k_pf_rmsnorm(s, m->pf_x, m->L(l, L2H_RMS_ATT).f32, m->pf_xn, M, dim));
+        // q | k | v columns of pf_raw; consecutive tensors of one type share a launch
+        const DevTensor w[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
+        const int64_t col[3] = {0, dim, dim + kvd};
+        for (int i = 0; i < 3;) {
+            int j = i + 1;
+            while (j < 3 && w[j].type == w[i].type) j++;
+            CK(k_pf_gemm(s, w + i, j - i, 0, m->pf_xn, M, dim, PF_STORE, m->pf_raw, dim + 2 * kvd, col[i], nullptr, 0));
+            i = j;
+        }
+        CK(k_pf_rope_scatter(s, m->pf_raw, m->pf_cs, m->pf_q, kc, vc, M, pos0, dim, kvd, m->hs, c.seq_len,
+                             c.rope_is_neox));
+        CK(k_pf_attention(s, m->pf_q, m->pf_att, kc, vc, M, pos0, m->hs, c.n_heads, c.n_kv_heads, c.seq_len, dim));
+        const DevTensor wo = m->L(l, L2H_WO);
+        CK(k_pf_gemm(s, &wo, 1, 0, m->pf_att, M, dim, PF_RESID, m->pf_x, dim, 0, nullptr, 0));
+        CK(k_pf_rmsnorm(s, m->pf_x, m->L(l, L2H_RMS_FFN).f32, m->pf_xn, M, dim));
+        const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
+        CK(k_pf_gemm(s, w13, 2, 1, m->pf_xn, M, dim, PF_SWIGLU, nullptr, 0, 0, m->pf_hb, c.hidden_dim));
+        const DevTensor w2 = m->L(l, L2H_W2);
+        CK(k_pf_gemm(s, &w2, 1, 0, m->pf_hb, M, c.hidden_dim, PF_RESID, m->pf_x, dim, 0, nullptr, 0));
+    }
+#undef CK
+    return hipSuccess;
+}
+
+extern "C" int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0, float *last_logits,
+                           int32_t *next_token) {
+    if (!m) return L2H_EINVAL;
+    l2h_ctx *ctx = m->ctx;
+    if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
+    if (!tokens || n < 1) return set_err(ctx, L2H_EINVAL, "prompt cannot be empty");
+    if (pos0 < 0 || pos0 + n > m->c.seq_len)
+        return set_err(ctx, L2H_EINVAL, "positions %d..%d outside the cache of %d", pos0, pos0 + n - 1, m->c.seq_len);
+    for (int i = 0; i < n; i++)
+        if (tokens[i] < 0 || tokens[i] >= m->c.vocab_size)
+            return set_err(ctx, L2H_EINVAL, "tokens[%d] = %d outside vocabulary", i, tokens[i]);
+    if (!k_pf_attention_supported(m->hs))
+        return set_err(ctx, L2H_EINVAL, "batched prompt pass needs a head size of 32, 64, 96 or 128 (have %d)", m->hs);
+    if (m->c.dim % 8 != 0 || m->c.hidden_dim % 8 != 0)
+        return set_err(ctx, L2H_EINVAL, "batched prompt pass needs dim and hidden_dim to be multiples of 8");
+    for (int l = 0; l < m->c.n_layers; l++)
+        if (m->L(l, L2H_W1).type != m->L(l, L2H_W3).type)
+            return set_err(ctx, L2H_EINVAL, "batched prompt pass needs w1 and w3 of one type (layer %d)", l);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    int rc;
+    if ((rc = prefill_buffers(m, std::min(n, L2H_PREFILL_CHUNK)))) return rc;
+    int M = 0;
+    for (int c0 = 0; c0 < n; c0 += M) {
+        M = std::min(m->pf_cap, n - c0);
+        HIPCHK(ctx, hipMemcpyAsync(m->pf_tok, tokens + c0, (size_t)M * 4, hipMemcpyHostToDevice, ctx->stream));
+        hipError_t e = prefill_chunk(m, M, pos0 + c0);
+        if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "prompt pass launch failed: %s", hipGetErrorString(e));
+    }
+    // last position: its hidden state becomes the decode state; classifier and argmax as in a decode step
+    HIPCHK(ctx, hipMemcpyAsync(m->x, m->pf_x + (int64_t)(M - 1) * m->c.dim, (size_t)m->c.dim * 4,
+                               hipMemcpyDeviceToDevice, ctx->stream));
+    DecodeCtl h{};
+    h.token = tokens[n - 1];
+    h.pos = pos0 + n - 1;
+    h.n_prompt = 1;
+    HIPCHK(ctx, hipMemcpyAsync(m->ctl, &h, sizeof h, hipMemcpyHostToDevice, ctx->stream));
+    hipError_t e = launch_output(m);
+    if (e == hipSuccess)
+        e = k_argmax(ctx->stream, m->logits, m->c.vocab_size, m->argmax_partial, m->ctl, m->out_tokens, m->max_out);
+    if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "classifier launch failed: %s", hipGetErrorString(e));
+    if (next_token)
+        HIPCHK(ctx, hipMemcpyAsync(next_token, m->out_tokens, 4, hipMemcpyDeviceToHost, ctx->stream));
+    if (last_logits)
+        HIPCHK(ctx, hipMemcpyAsync(last_logits, m->logits, (size_t)m->c.vocab_size * 4, hipMemcpyDeviceToHost,
+                                   ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return L2H_OK;
 }
 
 extern "C" int l2h_generate_greedy(l2h_model *m, const int32_t *prompt, int n_prompt, int pos0, int n_new,

@@ -1,0 +1,604 @@
+// Batched prompt pass ("prefill"): the same layer sequence as transformer! (reference
+// src/inference.jl:222-315) applied to M positions at once, where the matrix products are dense
+// contractions and run on the matrix cores: weights are dequantized tile by tile into LDS as bf16
+// (the reference's fp32 dequantization expressions, src/kquants.jl:83-98,213-217,333-343, then one
+// rounding to bf16), activations are bf16, accumulation is fp32 (v_mfma_f32_32x32x16_bf16).
+// The reference has no batched path; the result is defined as what its per-token loop would leave
+// in the KV cache and the last position's logits, to bf16 accuracy.
+#include "matvec_dev.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    bf16x2 v;
+    v.x = (__bf16)a;
+    v.y = (__bf16)b;
+    return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ bf16x8 as_bf16x8(uint4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// ------------------------------------------------------------------------------------------
+// small per-position kernels
+// ------------------------------------------------------------------------------------------
+// X[m][:] = dequantized embedding row of tokens[m]  (src/inference.jl:236)
+__global__ __launch_bounds__(256) void pf_embed_kernel(DevTensor emb, const int32_t *tokens, float *X, int M) {
+    const int m = blockIdx.y;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (m >= M || i >= emb.ne0) return;
+    X[(int64_t)m * emb.ne0 + i] = dequant_elem(emb, tokens[m], i);
+}
+
+// cos/sin of the RoPE angles of positions pos0..pos0+M-1: theta_i = fp32(pos) advanced by i fp32
+// multiplications (src/inference.jl:122-127), cos/sin in fp64, rounded.  cs[m][i][2].
+__global__ __launch_bounds__(64) void pf_rope_table_kernel(float *cs, int pos0, int M, int half, float theta_scale) {
+    const int m = blockIdx.x, i = threadIdx.x;
+    if (m >= M) return;
+    for (int p = i; p < half; p += blockDim.x) {
+        float theta = 1.0f * (float)(pos0 + m);
+        for (int k = 0; k < p; k++) theta *= theta_scale;
+        cs[((int64_t)m * half + p) * 2] = (float)cos((double)theta);
+        cs[((int64_t)m * half + p) * 2 + 1] = (float)sin((double)theta);
+    }
+}
+
+// rmsnorm! of every row (src/inference.jl:102-110), fp64 sum of squares, output rounded to bf16
+__global__ __launch_bounds__(256) void pf_rmsnorm_kernel(const float *X, const float *w, uint16_t *out, int64_t K) {
+    __shared__ double red[16];
+    const float *x = X + (int64_t)blockIdx.x * K;
+    double acc = 0.0;
+    for (int64_t i = threadIdx.x; i < K; i += blockDim.x) acc = fma((double)x[i], (double)x[i], acc);
+    float ss = (float)block_sum_f64(acc, red);
+    ss /= (float)K;
+    ss += 1e-5f;
+    ss = 1.0f / sqrtf(ss);
+    __bf16 *o = (__bf16 *)out + (int64_t)blockIdx.x * K;
+    for (int64_t i = threadIdx.x; i < K; i += blockDim.x) o[i] = (__bf16)(w[i] * (ss * x[i]));
+}
+
+// rope! of q and k (src/inference.jl:112-157), cache append (:259-260): raw[m] = (q | k | v) fp32 ->
+// Qb bf16 [M][dim], K cache [n_kv][hs/4][seq_len][4], V cache [n_kv][seq_len][hs]
+__global__ __launch_bounds__(256) void pf_rope_scatter_kernel(const float *raw, const float *cs, uint16_t *Qb,
+                                                              float *kc, float *vc, int M, int pos0, int dim,
+                                                              int kv_dim, int hs, int seq_len, int neox) {
+    const int m = blockIdx.x;
+    if (m >= M) return;
+    const float *r = raw + (int64_t)m * (dim + 2 * kv_dim);
+    const int half = hs >> 1, pos = pos0 + m;
+    const int npairs = (dim + kv_dim) >> 1;
+    for (int p = threadIdx.x; p < npairs; p += blockDim.x) {
+        const bool is_q = p < (dim >> 1);
+        const int pp = is_q ? p : p - (dim >> 1);
+        const int h = pp / half, i = pp % half;
+        const int e0 = neox ? i : 2 * i, e1 = neox ? i + half : 2 * i + 1;
+        const float *src = r + (is_q ? 0 : dim) + h * hs;
+        const float re = src[e0], im = src[e1];
+        const float c = cs[((int64_t)m * half + i) * 2], s = cs[((int64_t)m * half + i) * 2 + 1];
+        const float o0 = (re * c) - (im * s), o1 = (re * s) + (im * c);
+        if (is_q) {
+            __bf16 *q = (__bf16 *)Qb + (int64_t)m * dim + h * hs;
+            q[e0] = (__bf16)o0;
+            q[e1] = (__bf16)o1;
+        } else {
+            kc[(((int64_t)h * (hs >> 2) + (e0 >> 2)) * seq_len + pos) * 4 + (e0 & 3)] = o0;
+            kc[(((int64_t)h * (hs >> 2) + (e1 >> 2)) * seq_len + pos) * 4 + (e1 & 3)] = o1;
+        }
+    }
+    for (int e = threadIdx.x; e < kv_dim; e += blockDim.x) {
+        const int h = e / hs, d = e % hs;
+        vc[((int64_t)h * seq_len + pos) * hs + d] = r[dim + kv_dim + e];
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// dense product  C[m][L] = sum_k act[m][k] * W[L][k]   over logical weight rows L
+// ------------------------------------------------------------------------------------------
+struct PfGemmArgs {
+    DevTensor w[3];
+    int nseg;
+    int interleave;  // logical row L = (segment L & 1, row L >> 1): w1/w3 pairs for SwiGLU
+    int64_t n_rows;  // logical rows
+    int64_t K;
+    const uint16_t *act;  // bf16 [M][K]
+    int M;
+    float *out;  // STORE: fp32 [M][ldo] at column out_col0 + L; RESID: out[m][L] += C
+    int64_t ldo, out_col0;
+    uint16_t *out_bf;  // SWIGLU: bf16 [M][ldb], column L/2
+    int64_t ldb;
+};
+
+struct PfRow {
+    bool valid;
+    int seg;
+    int64_t row;
+};
+__device__ __forceinline__ PfRow pf_row(const PfGemmArgs &a, int64_t L) {
+    PfRow r{false, 0, 0};
+    if (L >= a.n_rows) return r;
+    r.valid = true;
+    if (a.interleave) {
+        r.seg = (int)(L & 1);
+        r.row = L >> 1;
+        return r;
+    }
+    const int64_t n0 = a.w[0].ne1, n1 = a.nseg > 1 ? a.w[1].ne1 : 0;
+    if (L < n0) {
+        r.seg = 0;
+        r.row = L;
+    } else if (L < n0 + n1) {
+        r.seg = 1;
+        r.row = L - n0;
+    } else {
+        r.seg = 2;
+        r.row = L - n0 - n1;
+    }
+    return r;
+}
+
+// raw bytes of 32 consecutive weights of one row (k0 a multiple of 32), and their conversion to bf16
+struct PfRaw {
+    uint4 hdr, qa, qb, ha, hb;
+    uint32_t sc[2];
+    uint32_t d;
+};
+
+struct PfRowPtr {  // stream pointers of the row a thread dequantizes
+    const uint4 *hdr;
+    const uint8_t *qs, *qh;
+    const uint32_t *sc6;
+    const uint16_t *d6;
+    const float *f32;
+    int64_t nb, ne0;
+    bool valid;
+};
+
+template <int TYPE>
+__device__ __forceinline__ void pf_load_raw(PfRaw &r, const PfRowPtr &p, int64_t row, int64_t k0, int64_t K) {
+    if (!p.valid) return;
+    const int64_t blk = row * p.nb + (k0 >> 8);
+    const int rr = (int)(k0 & 255);
+    if (TYPE == L2H_TYPE_Q4_K || TYPE == L2H_TYPE_Q5_K) {
+        const int j = rr >> 6;
+        r.hdr = p.hdr[blk];
+        const uint4 *q = (const uint4 *)(p.qs + blk * 128 + 32 * j);
+        r.qa = q[0];
+        r.qb = q[1];
+        if (TYPE == L2H_TYPE_Q5_K) {
+            const uint4 *h = (const uint4 *)(p.qh + blk * 32);
+            r.ha = h[0];
+            r.hb = h[1];
+        }
+    } else if (TYPE == L2H_TYPE_Q6_K) {
+        const int n = rr >> 7, g = (rr & 127) >> 5;
+        const uint4 *q = (const uint4 *)(p.qs + blk * 128 + 64 * n + 32 * (g & 1));
+        r.qa = q[0];
+        r.qb = q[1];
+        const uint4 *h = (const uint4 *)(p.qh + blk * 64 + 32 * n);
+        r.ha = h[0];
+        r.hb = h[1];
+        r.sc[0] = p.sc6[blk * 4 + 2 * n];
+        r.sc[1] = p.sc6[blk * 4 + 2 * n + 1];
+        r.d = p.d6[blk];
+    } else {  // F32: 32 floats kept in the five uint4 + ... (loaded in convert; nothing to stage here)
+    }
+}
+
+__device__ __forceinline__ uint32_t u4_word(const uint4 &a, const uint4 &b, int w) {  // word w (0..7) of a|b
+    switch (w) {
+    case 0: return a.x;
+    case 1: return a.y;
+    case 2: return a.z;
+    case 3: return a.w;
+    case 4: return b.x;
+    case 5: return b.y;
+    case 6: return b.z;
+    default: return b.w;
+    }
+}
+
+// out[4] = the 32 weights as bf16 (8 per uint4), in element order
+template <int TYPE>
+__device__ __forceinline__ void pf_convert(const PfRaw &r, const PfRowPtr &p, int64_t row, int64_t k0, int64_t K,
+                                           uint4 out[4]) {
+    uint32_t pk[16];
+    if (!p.valid) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) pk[i] = 0;
+    } else if (TYPE == L2H_TYPE_Q4_K || TYPE == L2H_TYPE_Q5_K) {
+        const int rr = (int)(k0 & 255), s = rr >> 5, hi = s & 1;
+        int sc, mn;
+        kq_scale_min(r.hdr, s, sc, mn);
+        const float d = half_bits_to_float((uint16_t)(r.hdr.x & 0xFFFF));
+        const float dmin = half_bits_to_float((uint16_t)(r.hdr.x >> 16));
+        const float d1 = d * (float)sc, m1 = dmin * (float)mn;
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            uint32_t qw = u4_word(r.qa, r.qb, w);
+            qw = hi ? (qw >> 4) & 0x0F0F0F0Fu : qw & 0x0F0F0F0Fu;
+            if (TYPE == L2H_TYPE_Q5_K) {
+                const uint32_t hw = u4_word(r.ha, r.hb, w);
+                qw |= ((hw >> s) & 0x01010101u) << 4;
+            }
+            const float v0 = d1 * (float)(qw & 0xFF) - m1, v1 = d1 * (float)((qw >> 8) & 0xFF) - m1;
+            const float v2 = d1 * (float)((qw >> 16) & 0xFF) - m1, v3 = d1 * (float)(qw >> 24) - m1;
+            pk[2 * w] = pack_bf16(v0, v1);
+            pk[2 * w + 1] = pack_bf16(v2, v3);
+        }
+    } else if (TYPE == L2H_TYPE_Q6_K) {
+        const int rr = (int)(k0 & 255), g = (rr & 127) >> 5;
+        const float d = half_bits_to_float((uint16_t)r.d);
+#pragma unroll
+        for (int w = 0; w < 8; w++) {
+            uint32_t qw = u4_word(r.qa, r.qb, w);
+            qw = (g & 2) ? (qw >> 4) & 0x0F0F0F0Fu : qw & 0x0F0F0F0Fu;
+            const uint32_t hw = u4_word(r.ha, r.hb, w);
+            qw |= ((hw >> (2 * g)) & 0x03030303u) << 4;
+            const uint32_t scw = r.sc[w >> 2];  // elements 0..15 -> first scale dword, 16..31 -> second
+            const int sc = (int)(int8_t)((scw >> (8 * g)) & 0xFF);
+            const float v0 = d * (float)(sc * ((int)(qw & 0xFF) - 32)), v1 = d * (float)(sc * ((int)((qw >> 8) & 0xFF) - 32));
+            const float v2 = d * (float)(sc * ((int)((qw >> 16) & 0xFF) - 32)), v3 = d * (float)(sc * ((int)(qw >> 24) - 32));
+            pk[2 * w] = pack_bf16(v0, v1);
+            pk[2 * w + 1] = pack_bf16(v2, v3);
+        }
+    } else {
+        const float *src = p.f32 + row * p.ne0 + k0;
+#pragma unroll
+        for (int i = 0; i < 16; i++) {
+            const float v0 = (k0 + 2 * i) < K ? src[2 * i] : 0.0f;
+            const float v1 = (k0 + 2 * i + 1) < K ? src[2 * i + 1] : 0.0f;
+            pk[i] = pack_bf16(v0, v1);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++) out[c] = make_uint4(pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]);
+}
+
+// Workgroup tile: 128 weight rows x 128 positions, K in steps of 64; 4 wavefronts, each 64 x 64 as
+// 2 x 2 tiles of 32 x 32.  Weights are the A operand (rows), positions the B operand (columns), so
+// a lane ends up holding one position and groups of 4 consecutive weight rows: neighbours such as a
+// w1/w3 pair sit in one lane.  LDS rows are 64 bf16 = 8 chunks of 16 bytes, chunk c of row r kept at
+// c ^ (r & 7) so that the 8 lanes of a 128-byte access phase hit distinct banks.
+template <int TYPE, int EPI>
+__global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
+    __shared__ uint4 s_w[128 * 8];
+    __shared__ uint4 s_x[128 * 8];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wn = wave & 1, wm = wave >> 1;
+    const int64_t n0 = (int64_t)blockIdx.y * 128;
+    const int m0 = blockIdx.x * 128;
+    const int64_t K = a.K;
+
+    // the weight row this thread dequantizes: row t/2 of the tile, elements 32*(t&1).. of each K step
+    const int wr = t >> 1, whh = t & 1;
+    const PfRow lr = pf_row(a, n0 + wr);
+    PfRowPtr rp;
+    {
+        const int sg = lr.seg;
+#define PICK(F) (sg == 0 ? a.w[0].F : (sg == 1 ? a.w[1].F : a.w[2].F))
+        rp.hdr = PICK(hdr);
+        rp.qs = PICK(qs);
+        rp.qh = PICK(qh);
+        rp.sc6 = PICK(sc6);
+        rp.d6 = PICK(d6);
+        rp.f32 = PICK(f32);
+        rp.nb = PICK(nb);
+        rp.ne0 = PICK(ne0);
+#undef PICK
+        rp.valid = lr.valid;
+    }
+    // activations: 4 chunks of 16 bytes per thread and K step: position (t>>3) + 32*i, chunk t&7
+    const int xc = t & 7;
+    const uint16_t *xrow[4];
+    bool xvalid[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int m = m0 + (t >> 3) + 32 * i;
+        xvalid[i] = m < a.M;
+        xrow[i] = a.act + (int64_t)(xvalid[i] ? m : 0) * K + 8 * xc;
+    }
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    PfRaw raw;
+    uint4 xreg[4];
+    auto gload = [&](int64_t k0) {
+        if (k0 + 32 * whh < K) pf_load_raw<TYPE>(raw, rp, lr.row, k0 + 32 * whh, K);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            xreg[i] = make_uint4(0, 0, 0, 0);
+            if (xvalid[i] && k0 + 8 * xc < K) xreg[i] = *(const uint4 *)(xrow[i] + k0);
+        }
+    };
+    gload(0);
+    for (int64_t k0 = 0; k0 < K; k0 += 64) {
+        // registers -> LDS
+        {
+            uint4 wv[4];
+            PfRowPtr q = rp;
+            q.valid = rp.valid && (k0 + 32 * whh < K);
+            pf_convert<TYPE>(raw, q, lr.row, k0 + 32 * whh, K, wv);
+#pragma unroll
+            for (int c = 0; c < 4; c++) s_w[wr * 8 + ((4 * whh + c) ^ (wr & 7))] = wv[c];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int r = (t >> 3) + 32 * i;
+                s_x[r * 8 + (xc ^ (r & 7))] = xreg[i];
+            }
+        }
+        __syncthreads();
+        if (k0 + 64 < K) gload(k0 + 64);  // in flight during the products
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) {
+            const int c = 2 * kk + (lane >> 5);
+            bf16x8 A[2], B[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int ra = 64 * wn + 32 * i + (lane & 31);
+                A[i] = as_bf16x8(s_w[ra * 8 + (c ^ (ra & 7))]);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int rb = 64 * wm + 32 * j + (lane & 31);
+                B[j] = as_bf16x8(s_x[rb * 8 + (c ^ (rb & 7))]);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[i], B[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // lane: position m0 + 64 wm + 32 j + lane%32; register r of tile i: logical weight row
+    // n0 + 64 wn + 32 i + 8 (r/4) + 4 (lane/32) + r%4
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int m = m0 + 64 * wm + 32 * j + (lane & 31);
+        if (m >= a.M) continue;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                const int64_t L = n0 + 64 * wn + 32 * i + 8 * rq + 4 * (lane >> 5);
+                if (L >= a.n_rows) continue;
+                const float v0 = acc[i][j][4 * rq], v1 = acc[i][j][4 * rq + 1], v2 = acc[i][j][4 * rq + 2],
+                            v3 = acc[i][j][4 * rq + 3];
+                if (EPI == PF_SWIGLU) {  // (w1 row u, w3 row u) = logical rows (2u, 2u+1), src/inference.jl:295-299
+                    const float h0 = swiglu_val(v0, v1), h1 = swiglu_val(v2, v3);
+                    uint16_t *o = a.out_bf + (int64_t)m * a.ldb + (L >> 1);
+                    if (L + 3 < a.n_rows)
+                        *(uint32_t *)o = pack_bf16(h0, h1);  // L/2 is even and ldb is even: aligned
+                    else
+                        ((__bf16 *)o)[0] = (__bf16)h0;
+                } else {
+                    float *o = a.out + (int64_t)m * a.ldo + a.out_col0 + L;
+                    const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (L + e >= a.n_rows) break;
+                        if (EPI == PF_RESID)
+                            o[e] += v[e];  // x .+= ... (src/inference.jl:284,305)
+                        else
+                            o[e] = v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// causal attention over a block of positions (src/inference.jl:263-278 for each of them):
+// one workgroup = one head x 128 query positions (32 per wavefront), keys in tiles of 32.
+//   S^T = K_tile Q^T          A = K rows (keys), B = Q columns (queries)
+//   running max / sum per query (a lane holds one query: 16 of the 32 keys, the lane 32 further the rest)
+//   O^T += V_tile^T P^T       A = V^T rows (head dims), B = P^T columns (queries)
+// The k index of the second product is a permutation of the keys chosen so that the lane's own
+// probabilities are its B operand without any exchange; V^T is staged in LDS in that key order.
+// ------------------------------------------------------------------------------------------
+template <int HS>
+__global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const float *kc,
+                                                      const float *vc, int M, int qpos0, int n_heads, int n_kv,
+                                                      int seq_len, int dim) {
+    constexpr int KSTEPS = HS / 16, DT = HS / 32;
+    constexpr int KROW = HS * 2 + 16;  // bytes per key row: +16 spreads the rows over the banks
+    constexpr int VROW = 80;           // bytes per head-dim row of V^T: 32 keys + 16 bytes of padding
+    __shared__ __align__(16) unsigned char s_k[32 * KROW];
+    __shared__ __align__(16) unsigned char s_v[HS * VROW];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, g = lane >> 5, ql = lane & 31;
+    const int h = blockIdx.y, kvh = h / (n_heads / n_kv);
+    const int q0 = blockIdx.x * 128;
+    const int myq = q0 + 32 * wave + ql;
+    const bool qvalid = myq < M;
+    bf16x8 qf[KSTEPS];
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; kk++) {
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (qvalid) v = *(const uint4 *)(Qb + (int64_t)myq * dim + h * HS + 16 * kk + 8 * g);
+        qf[kk] = as_bf16x8(v);
+    }
+    f32x16 o[DT];
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[d][r] = 0.0f;
+    float mrun = -INFINITY, lrun = 0.0f;
+    const int wave_qmax = min(M - 1, q0 + 32 * wave + 31), wg_qmax = min(M - 1, q0 + 127);
+    const int nkt = (qpos0 + wg_qmax) / 32 + 1;
+    const float scale = sqrtf((float)HS);
+    for (int kt = 0; kt < nkt; kt++) {
+        const int key0 = 32 * kt;
+        __syncthreads();
+        for (int idx = t; idx < 32 * (HS / 4); idx += 256) {  // K tile -> bf16 rows
+            const int key = idx & 31, i4 = idx >> 5;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (key0 + key < seq_len) v = *(const float4 *)(kc + (((int64_t)kvh * (HS / 4) + i4) * seq_len + key0 + key) * 4);
+            uint2 w;
+            w.x = pack_bf16(v.x, v.y);
+            w.y = pack_bf16(v.z, v.w);
+            *(uint2 *)(s_k + key * KROW + i4 * 8) = w;
+        }
+        for (int idx = t; idx < 32 * (HS / 4); idx += 256) {  // V tile -> bf16, transposed, keys permuted
+            const int d4 = idx % (HS / 4), key = idx / (HS / 4);
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (key0 + key < seq_len) v = *(const float4 *)(vc + ((int64_t)kvh * seq_len + key0 + key) * HS + 4 * d4);
+            // key = 16 s + 8 a + 4 g + b  ->  slot 16 s + 8 g + 4 a + b
+            const int rem = key & 15;
+            const int slot = (key & 16) + 8 * ((rem >> 2) & 1) + 4 * (rem >> 3) + (rem & 3);
+            __bf16 *dst = (__bf16 *)(s_v + (4 * d4) * VROW) + slot;
+            dst[0] = (__bf16)v.x;
+            dst[VROW / 2] = (__bf16)v.y;
+            dst[VROW] = (__bf16)v.z;
+            dst[3 * VROW / 2] = (__bf16)v.w;
+        }
+        __syncthreads();
+        if (key0 > qpos0 + wave_qmax) continue;  // every key of the tile lies in this wavefront's future
+        f32x16 s;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS; kk++) {
+            const bf16x8 A = as_bf16x8(*(const uint4 *)(s_k + ql * KROW + (16 * kk + 8 * g) * 2));
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, qf[kk], s, 0, 0, 0);
+        }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int key = key0 + 8 * (r >> 2) + 4 * g + (r & 3);
+            float v = s[r] / scale;  // att ./= sqrt(hs) (src/inference.jl:268)
+            if (!qvalid || key > qpos0 + myq) v = -INFINITY;
+            s[r] = v;
+            tmax = fmaxf(tmax, v);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+        const float mnew = fmaxf(mrun, tmax);
+        const float alpha = (mnew == -INFINITY) ? 1.0f : expf(mrun - mnew);
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const float pv = (s[r] == -INFINITY) ? 0.0f : expf(s[r] - mnew);
+            s[r] = pv;
+            psum += pv;
+        }
+        psum += __shfl_xor(psum, 32, WAVE);
+        lrun = lrun * alpha + psum;
+        mrun = mnew;
+#pragma unroll
+        for (int d = 0; d < DT; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+#pragma unroll
+        for (int st = 0; st < 2; st++) {
+            const uint4 pb = make_uint4(pack_bf16(s[8 * st], s[8 * st + 1]), pack_bf16(s[8 * st + 2], s[8 * st + 3]),
+                                        pack_bf16(s[8 * st + 4], s[8 * st + 5]), pack_bf16(s[8 * st + 6], s[8 * st + 7]));
+            const bf16x8 B = as_bf16x8(pb);
+#pragma unroll
+            for (int d = 0; d < DT; d++) {
+                const bf16x8 A = as_bf16x8(*(const uint4 *)(s_v + (32 * d + ql) * VROW + (16 * st + 8 * g) * 2));
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, o[d], 0, 0, 0);
+            }
+        }
+    }
+    if (!qvalid) return;
+    const float inv = 1.0f / lrun;
+#pragma unroll
+    for (int d = 0; d < DT; d++)
+#pragma unroll
+        for (int rq = 0; rq < 4; rq++) {
+            const int e = 32 * d + 8 * rq + 4 * g;
+            uint2 w;
+            w.x = pack_bf16(o[d][4 * rq] * inv, o[d][4 * rq + 1] * inv);
+            w.y = pack_bf16(o[d][4 * rq + 2] * inv, o[d][4 * rq + 3] * inv);
+            *(uint2 *)(Att + (int64_t)myq * dim + h * HS + e) = w;
+        }
+}
+
+// ------------------------------------------------------------------------------------------
+// launchers
+// ------------------------------------------------------------------------------------------
+hipError_t k_pf_embed(hipStream_t s, const DevTensor &emb, const int32_t *tokens, float *X, int M) {
+    hipLaunchKernelGGL(pf_embed_kernel, dim3((unsigned)((emb.ne0 + 255) / 256), (unsigned)M), dim3(256), 0, s, emb,
+                       tokens, X, M);
+    return hipGetLastError();
+}
+hipError_t k_pf_rope_table(hipStream_t s, float *cs, int pos0, int M, int half, float theta_scale) {
+    hipLaunchKernelGGL(pf_rope_table_kernel, dim3((unsigned)M), dim3(64), 0, s, cs, pos0, M, half, theta_scale);
+    return hipGetLastError();
+}
+hipError_t k_pf_rmsnorm(hipStream_t s, const float *X, const float *w, uint16_t *out, int M, int64_t K) {
+    hipLaunchKernelGGL(pf_rmsnorm_kernel, dim3((unsigned)M), dim3(256), 0, s, X, w, out, K);
+    return hipGetLastError();
+}
+hipError_t k_pf_rope_scatter(hipStream_t s, const float *raw, const float *cs, uint16_t *Qb, float *kc, float *vc, int M,
+                             int pos0, int dim, int kv_dim, int hs, int seq_len, int neox) {
+    hipLaunchKernelGGL(pf_rope_scatter_kernel, dim3((unsigned)M), dim3(256), 0, s, raw, cs, Qb, kc, vc, M, pos0, dim,
+                       kv_dim, hs, seq_len, neox);
+    return hipGetLastError();
+}
+
+template <int TYPE>
+static hipError_t pf_gemm_type(hipStream_t s, const PfGemmArgs &a, int epi, dim3 grid) {
+    switch (epi) {
+    case PF_STORE: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_STORE>), grid, dim3(256), 0, s, a); break;
+    case PF_RESID: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_RESID>), grid, dim3(256), 0, s, a); break;
+    case PF_SWIGLU: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_SWIGLU>), grid, dim3(256), 0, s, a); break;
+    default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// w: nseg tensors of one type sharing the input; see PfGemmArgs for the outputs
+hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *act, int M, int64_t K,
+                     int epi, float *out, int64_t ldo, int64_t out_col0, uint16_t *out_bf, int64_t ldb) {
+    PfGemmArgs a{};
+    int64_t rows = 0;
+    for (int i = 0; i < nseg; i++) {
+        if (w[i].type != w[0].type || w[i].ne0 != K) return hipErrorInvalidValue;
+        a.w[i] = w[i];
+        rows += w[i].ne1;
+    }
+    if (interleave && (nseg != 2 || w[0].ne1 != w[1].ne1)) return hipErrorInvalidValue;
+    if (K % 8 != 0 || M < 1) return hipErrorInvalidValue;
+    a.nseg = nseg;
+    a.interleave = interleave;
+    a.n_rows = rows;
+    a.K = K;
+    a.act = act;
+    a.M = M;
+    a.out = out;
+    a.ldo = ldo;
+    a.out_col0 = out_col0;
+    a.out_bf = out_bf;
+    a.ldb = ldb;
+    const dim3 grid((unsigned)((M + 127) / 128), (unsigned)((rows + 127) / 128));
+    switch (w[0].type) {
+    case L2H_TYPE_Q4_K: return pf_gemm_type<L2H_TYPE_Q4_K>(s, a, epi, grid);
+    case L2H_TYPE_Q5_K: return pf_gemm_type<L2H_TYPE_Q5_K>(s, a, epi, grid);
+    case L2H_TYPE_Q6_K: return pf_gemm_type<L2H_TYPE_Q6_K>(s, a, epi, grid);
+    case L2H_TYPE_F32: return pf_gemm_type<L2H_TYPE_F32>(s, a, epi, grid);
+    }
+    return hipErrorInvalidValue;
+}
+
+bool k_pf_attention_supported(int hs) { return hs == 32 || hs == 64 || hs == 96 || hs == 128; }
+
+hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const float *kc, const float *vc, int M,
+                          int qpos0, int hs, int n_heads, int n_kv, int seq_len, int dim) {
+    const dim3 grid((unsigned)((M + 127) / 128), (unsigned)n_heads);
+#define GO(HS) hipLaunchKernelGGL((pf_attn_kernel<HS>), grid, dim3(256), 0, s, Qb, Att, kc, vc, M, qpos0, n_heads, n_kv, seq_len, dim)
+    switch (hs) {
+    case 32: GO(32); break;
+    case 64: GO(64); break;
+    case 96: GO(96); break;
+    case 128: GO(128); break;
+    default: return hipErrorInvalidValue;
+    }
+#undef GO
+    return hipGetLastError();
+}

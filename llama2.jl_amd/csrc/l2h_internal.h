@@ -161,6 +161,19 @@ hipError_t k_kv_layout(hipStream_t s, float *kc, float *vc, float *k_lin, float 
 hipError_t k_stream_read(hipStream_t s, const uint4 *p, int64_t n16, uint32_t *sink);
 hipError_t k_f32_to_f64(hipStream_t s, const float *x, double *y, int64_t n);
 
+// batched prompt pass (k_prefill.hip); activations travel as bf16 bit patterns
+enum { PF_STORE = 0, PF_RESID = 1, PF_SWIGLU = 2 };
+hipError_t k_pf_embed(hipStream_t s, const DevTensor &emb, const int32_t *tokens, float *X, int M);
+hipError_t k_pf_rope_table(hipStream_t s, float *cs, int pos0, int M, int half, float theta_scale);
+hipError_t k_pf_rmsnorm(hipStream_t s, const float *X, const float *w, uint16_t *out, int M, int64_t K);
+hipError_t k_pf_rope_scatter(hipStream_t s, const float *raw, const float *cs, uint16_t *Qb, float *kc, float *vc, int M,
+                             int pos0, int dim, int kv_dim, int hs, int seq_len, int neox);
+hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *act, int M, int64_t K,
+                     int epi, float *out, int64_t ldo, int64_t out_col0, uint16_t *out_bf, int64_t ldb);
+bool k_pf_attention_supported(int hs);
+hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const float *kc, const float *vc, int M,
+                          int qpos0, int hs, int n_heads, int n_kv, int seq_len, int dim);
+
 static inline int64_t l2h_gguf_block_bytes(int type) {
     switch (type) {
     case L2H_TYPE_F32: return 4;

@@ -131,6 +131,17 @@ class DeviceModel:
                                                       _lib.ptr(out), _lib.ptr(logits)))
         return (out[:n_new], logits) if want_logits else out[:n_new]
 
+    def prefill(self, tokens, pos0=0, want_logits=True):
+        """Batched prompt pass over positions pos0..pos0+len(tokens)-1: fills the K/V cache and returns
+        (logits of the last position, their argmax) like calling forward() for each position in turn
+        (src/inference.jl:222-315), with the matrix products in bf16 on the matrix cores."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.int32)
+        logits = np.empty(self.config.vocab_size, np.float32) if want_logits else None
+        nxt = C.c_int32()
+        self.ctx.check(_lib.lib().l2h_prefill(self.handle, _lib.ptr(tokens), tokens.size, int(pos0), _lib.ptr(logits),
+                                              C.byref(nxt)))
+        return logits, nxt.value
+
     def kv_write(self, layer, pos0, k, v):
         k = np.ascontiguousarray(k, dtype=np.float32)
         v = np.ascontiguousarray(v, dtype=np.float32)
