@@ -44,7 +44,7 @@ __global__ __launch_bounds__(256) void attn_scores_kernel(const double *qd, cons
 
 // One workgroup per head: softmax over att[h][0..pos]; probabilities written as fp32 (att)
 // and widened to fp64 (pd) for the value pass.
-__global__ __launch_bounds__(256) void attn_softmax_kernel(float *att, double *pd, const DecodeCtl *ctl, int seq_len) {
+__global__ __launch_bounds__(1024) void attn_softmax_kernel(float *att, double *pd, const DecodeCtl *ctl, int seq_len) {
     __shared__ double redd[16];
     __shared__ float redf[16];
     const int n = ctl->pos + 1;
@@ -103,6 +103,147 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(const double *part, fl
     out[e] = (float)acc;
 }
 
+// ---- long caches: three launches sized to fill the chip --------------------------------------
+// Scores: a workgroup = 64 timesteps of GH heads that share a KV head; wavefront w takes quarter w
+// of the head dimension (all of its 16-byte loads in flight at once), the quarters are added in
+// fixed order through LDS.
+template <int GH>
+__global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, const float *kc, float *att,
+                                                           const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
+                                                           int seq_len) {
+    __shared__ double s_q[GH * 128];
+    __shared__ double s_part[4][GH][64];
+    const int pos = ctl->pos;
+    const int t0 = blockIdx.x * 64;
+    if (t0 > pos) return;
+    const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
+    const int h0 = blockIdx.y * GH, kvh = h0 / (n_heads / n_kv_heads);
+    for (int i = threadIdx.x; i < GH * hs; i += 256) s_q[(i / hs) * 128 + i % hs] = qd[(int64_t)h0 * hs + i];
+    const int per = hs >> 4;  // 16-byte groups per quarter (hs <= 128: at most 8)
+    const int t = min(t0 + lane, pos);
+    const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
+    float4 kv[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++)
+        if (u < per) kv[u] = ldg_nt_f4(kp + (int64_t)u * seq_len);
+    __syncthreads();
+    double acc[GH];
+#pragma unroll
+    for (int g = 0; g < GH; g++) acc[g] = 0.0;
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        if (u < per) {
+            const double k0 = (double)kv[u].x, k1 = (double)kv[u].y, k2 = (double)kv[u].z, k3 = (double)kv[u].w;
+#pragma unroll
+            for (int g = 0; g < GH; g++) {
+                const double *qq = s_q + g * 128 + 4 * (part * per + u);
+                acc[g] = fma(qq[0], k0, acc[g]);
+                acc[g] = fma(qq[1], k1, acc[g]);
+                acc[g] = fma(qq[2], k2, acc[g]);
+                acc[g] = fma(qq[3], k3, acc[g]);
+            }
+        }
+    }
+#pragma unroll
+    for (int g = 0; g < GH; g++) s_part[part][g][lane] = acc[g];
+    __syncthreads();
+    const float scale = sqrtf((float)hs);
+    for (int i = threadIdx.x; i < GH * 64; i += 256) {
+        const int g = i >> 6, l = i & 63;
+        if (t0 + l > pos) continue;
+        const double v = ((s_part[0][g][l] + s_part[1][g][l]) + s_part[2][g][l]) + s_part[3][g][l];
+        att[(int64_t)(h0 + g) * seq_len + t0 + l] = (float)v / scale;
+    }
+}
+
+// Values: a workgroup = `chunk` (a multiple of 64) timesteps of GH heads sharing a KV head; thread =
+// (16-byte group of the head dimension, timestep group), eight loads in flight per round; fp64
+// partial sums per workgroup go to `part`, which attn_reduce4_kernel adds in block order.
+template <int GH>
+__global__ __launch_bounds__(256) void attn_av4_kernel(const double *pd, const float *vc, double *part,
+                                                       const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
+                                                       int seq_len, int chunk) {
+    __shared__ double s_p[GH][64];
+    __shared__ double s_red[8][GH][128];
+    const int pos = ctl->pos;
+    const int split = blockIdx.x, c0 = split * chunk;
+    if (c0 > pos) return;
+    const int h0 = blockIdx.y * GH, kvh = h0 / (n_heads / n_kv_heads);
+    const int n4 = hs >> 2, ngrp = min(8, 256 / n4);  // hs <= 128
+    const int i4 = threadIdx.x % n4, tg = threadIdx.x / n4;
+    const bool active = tg < ngrp;
+    double acc[GH][4];
+#pragma unroll
+    for (int g = 0; g < GH; g++) acc[g][0] = acc[g][1] = acc[g][2] = acc[g][3] = 0.0;
+    for (int t0 = c0; t0 < c0 + chunk && t0 <= pos; t0 += 64) {
+        const int nt = min(64, pos + 1 - t0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < GH * 64; i += 256) {
+            const int g = i >> 6, l = i & 63;
+            s_p[g][l] = l < nt ? pd[(int64_t)(h0 + g) * seq_len + t0 + l] : 0.0;
+        }
+        float4 v[8];
+        if (active) {
+            const float4 *vp = (const float4 *)(vc + ((int64_t)kvh * seq_len + t0) * hs) + i4;
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int l = tg + ngrp * u;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (l < nt) v[u] = ldg_nt_f4(vp + (int64_t)l * n4);
+            }
+        }
+        __syncthreads();
+        if (active) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const int l = tg + ngrp * u;
+                if (l < 64) {
+#pragma unroll
+                    for (int g = 0; g < GH; g++) {
+                        const double p = s_p[g][l];
+                        acc[g][0] = fma(p, (double)v[u].x, acc[g][0]);
+                        acc[g][1] = fma(p, (double)v[u].y, acc[g][1]);
+                        acc[g][2] = fma(p, (double)v[u].z, acc[g][2]);
+                        acc[g][3] = fma(p, (double)v[u].w, acc[g][3]);
+                    }
+                }
+            }
+        }
+    }
+    if (active) {
+#pragma unroll
+        for (int g = 0; g < GH; g++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) s_red[tg][g][4 * i4 + c] = acc[g][c];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < GH * hs; i += 256) {
+        const int g = i / hs, e = i % hs;
+        double a = 0.0;
+        for (int k = 0; k < ngrp; k++) a += s_red[k][g][e];
+        part[((int64_t)split * n_heads + h0 + g) * hs + e] = a;
+    }
+}
+
+// out[e] = fp32(sum of the partial sums of the timestep blocks, in block order): 64 elements per
+// workgroup, four threads per element each adding a quarter of the blocks, quarters added in order
+__global__ __launch_bounds__(256) void attn_reduce4_kernel(const double *part, float *out, const DecodeCtl *ctl,
+                                                           int dim, int chunk) {
+    __shared__ double s_q[4][64];
+    const int e = blockIdx.x * 64 + (threadIdx.x & 63), qtr = threadIdx.x >> 6;
+    const int nsplit = ctl->pos / chunk + 1;
+    const int per = (nsplit + 3) >> 2;
+    double acc = 0.0;
+    if (e < dim) {
+        const int s1 = min(nsplit, (qtr + 1) * per);
+#pragma unroll 8
+        for (int s = qtr * per; s < s1; s++) acc += part[(int64_t)s * dim + e];
+    }
+    s_q[qtr][threadIdx.x & 63] = acc;
+    __syncthreads();
+    if (qtr == 0 && e < dim) out[e] = (float)(((s_q[0][threadIdx.x] + s_q[1][threadIdx.x]) + s_q[2][threadIdx.x]) + s_q[3][threadIdx.x]);
+}
+
 // Short sequences: one workgroup per head does scores, softmax and values in one launch.
 __global__ __launch_bounds__(1024) void attn_fused_kernel(const float *q, float *xb, const float *kc, const float *vc,
                                                           const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
@@ -125,9 +266,28 @@ hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const flo
 
 template <int GH>
 static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att,
-                              double *pd, double *part, float *out, const DecodeCtl *ctl, int hs, int n_heads,
-                              int n_kv_heads, int seq_len) {
+                              double *pd, double *part, float *out, unsigned int *counter, const DecodeCtl *ctl, int hs,
+                              int n_heads, int n_kv_heads, int seq_len) {
     const int ntiles = (seq_len + L2H_ATT_TILE - 1) / L2H_ATT_TILE;
+    if (hs <= 128 && hs % 16 == 0 && L2H_ATT_TILE == 64) {
+        hipLaunchKernelGGL((attn_scores4_kernel<GH>), dim3(ntiles, n_heads / GH), dim3(256), 0, s, qd, kc, att, ctl, hs,
+                           n_heads, n_kv_heads, seq_len);
+        hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(attn_softmax_kernel, dim3(n_heads), dim3(1024), 0, s, att, pd, ctl, seq_len);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        // timesteps per value workgroup: as large as still leaves about 512 workgroups over a full cache
+        int chunk = 64;
+        while (chunk < 512 && (int64_t)(seq_len / (2 * chunk)) * (n_heads / GH) >= 512) chunk *= 2;
+        hipLaunchKernelGGL((attn_av4_kernel<GH>), dim3((seq_len + chunk - 1) / chunk, n_heads / GH), dim3(256), 0, s, pd,
+                           vc, part, ctl, hs, n_heads, n_kv_heads, seq_len, chunk);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        const int dim = hs * n_heads;
+        hipLaunchKernelGGL(attn_reduce4_kernel, dim3((dim + 63) / 64), dim3(256), 0, s, part, out, ctl, dim, chunk);
+        return hipGetLastError();
+    }
     hipLaunchKernelGGL((attn_scores_kernel<GH>), dim3((ntiles + 3) / 4, n_heads / GH), dim3(256), 0, s, qd, kc, att,
                        ctl, hs, n_heads, n_kv_heads, seq_len);
     hipError_t e = hipGetLastError();
@@ -145,10 +305,10 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
 }
 
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
-                       double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads,
-                       int seq_len) {
+                       double *part, float *out, unsigned int *counter, const DecodeCtl *ctl, int head_size, int n_heads,
+                       int n_kv_heads, int seq_len) {
     const int G = n_heads / n_kv_heads;
-    if (G % 4 == 0) return launch_attn<4>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    if (G % 2 == 0) return launch_attn<2>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    return launch_attn<1>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    if (G % 4 == 0) return launch_attn<4>(s, qd, kc, vc, att, pd, part, out, counter, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    if (G % 2 == 0) return launch_attn<2>(s, qd, kc, vc, att, pd, part, out, counter, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    return launch_attn<1>(s, qd, kc, vc, att, pd, part, out, counter, ctl, head_size, n_heads, n_kv_heads, seq_len);
 }

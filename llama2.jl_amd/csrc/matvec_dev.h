@@ -10,6 +10,12 @@ __device__ __forceinline__ uint4 ldg_nt(const uint4 *p) {
     return make_uint4(t.x, t.y, t.z, t.w);
 }
 
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ldg_nt_f4(const float4 *p) {
+    const f32x4v t = __builtin_nontemporal_load((const f32x4v *)p);
+    return make_float4(t.x, t.y, t.z, t.w);
+}
+
 // ------------------------------------------------------------------------------------------
 // Activations exchanged between workgroups INSIDE one kernel (the persistent decode kernel) are
 // written and read with device-scope relaxed atomics: such stores go through to memory and such
