@@ -15,7 +15,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libl2hip.so")
 
-SOURCES = ["api.cpp", "synth.cpp", "k_misc.hip", "k_matvec.hip", "k_attn.hip", "k_mega.hip", "k_prefill.hip"]
+SOURCES = ["api.cpp", "synth.cpp", "k_misc.hip", "k_matvec.hip", "k_attn.hip", "k_mega.hip", "k_prefill.hip", "k_flow.hip"]
 
 COMMON = [
     "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function",

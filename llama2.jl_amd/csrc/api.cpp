@@ -195,6 +195,7 @@ extern "C" int l2h_device_info(l2h_ctx *ctx, char *name, int name_cap, int32_t *
 // ------------------------------------------------------------------------------------------
 struct l2h_model;
 static l2h_model *g_bound_model = nullptr;  // whose phase arguments the persistent kernel's constant memory holds
+static l2h_model *g_flow_bound = nullptr;   // whose arguments the streaming kernel's constant memory holds
 
 struct l2h_model {
     l2h_ctx *ctx = nullptr;
@@ -230,6 +231,11 @@ struct l2h_model {
 #ifdef L2H_TIMELINE
     long long *timeline = nullptr, *timeline2 = nullptr;
 #endif
+    // streaming decode kernel
+    bool flow = false;
+    FlowArgs flow_args{};
+    int flow_grid = 0, flow_cls_type = 0;
+    unsigned int flow_gen = 1;  // epoch of the next launch's input; 0 is what cleared memory holds
     // batched prompt pass: buffers for pf_cap positions, allocated at the first l2h_prefill
     int pf_cap = 0;
     float *pf_x = nullptr, *pf_raw = nullptr, *pf_cs = nullptr;
@@ -289,6 +295,7 @@ static void model_free_state(l2h_model *m) {
 extern "C" void l2h_model_destroy(l2h_model *m) {
     if (!m) return;
     if (g_bound_model == m) g_bound_model = nullptr;
+    if (g_flow_bound == m) g_flow_bound = nullptr;
     (void)hipStreamSynchronize(m->ctx->stream);
     model_free_state(m);
     for (auto &t : m->glob) dev_tensor_free(&t);
@@ -347,12 +354,12 @@ extern "C" int l2h_model_set_tensor(l2h_model *m, int role, int layer, int type,
 extern "C" int l2h_model_set_path(l2h_model *m, int path) {
     if (!m) return L2H_EINVAL;
     if (m->finalized) return set_err(m->ctx, L2H_ESTATE, "model already finalized");
-    if (path < 0 || path > 2) return set_err(m->ctx, L2H_EINVAL, "path must be 0, 1 or 2");
+    if (path < 0 || path > 3) return set_err(m->ctx, L2H_EINVAL, "path must be 0, 1, 2 or 3");
     m->path_request = path;
     return L2H_OK;
 }
 
-extern "C" int l2h_model_path(l2h_model *m) { return (m && m->finalized) ? (m->mega ? 2 : 1) : 0; }
+extern "C" int l2h_model_path(l2h_model *m) { return (m && m->finalized) ? (m->flow ? 3 : (m->mega ? 2 : 1)) : 0; }
 
 extern "C" int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t host_bytes) {
     if (!m || !host) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "l2h_model_get_tensor: NULL argument");
@@ -618,6 +625,102 @@ static int mega_setup(l2h_model *m) {
     return L2H_OK;
 }
 
+// Builds the per-wavefront weight streams and the tagged activation buffers of the streaming kernel.
+static int flow_setup(l2h_model *m) {
+    l2h_ctx *ctx = m->ctx;
+    const l2h_config &c = m->c;
+    m->flow = false;
+    if (m->path_request != 3) return L2H_OK;
+    FlowArgs a{};
+    a.dim = c.dim;
+    a.hidden = c.hidden_dim;
+    a.hs = m->hs;
+    a.n_heads = c.n_heads;
+    a.n_kv_heads = c.n_kv_heads;
+    a.kv_dim = m->kv_dim;
+    a.seq_len = c.seq_len;
+    a.n_layers = c.n_layers;
+    a.vocab = c.vocab_size;
+    a.neox = c.rope_is_neox;
+    a.theta_scale = m->theta_scale;
+    std::vector<int> types;
+    for (int l = 0; l < c.n_layers; l++)
+        for (int r : {L2H_WQ, L2H_WK, L2H_WV, L2H_WO, L2H_W1, L2H_W2, L2H_W3}) types.push_back(m->L(l, r).type);
+    const int grid = ctx->prop.multiProcessorCount;
+    const int cls_type = m->glob[L2H_OUTPUT].type;
+    std::string why;
+    if (!k_flow_plan(a, types.data(), (int)types.size(), cls_type, grid, &why))
+        return set_err(ctx, L2H_EINVAL, "streaming kernel not available: %s", why.c_str());
+    if (m->L(0, L2H_RMS_ATT).layer_stride != m->L(0, L2H_RMS_FFN).layer_stride)
+        return set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ");
+    std::vector<int64_t> off;
+    const int64_t total = k_flow_offsets(a, cls_type, grid, off);
+    unsigned char *stream = nullptr;
+    int64_t *off_dev = nullptr;
+    int rc;
+    if ((rc = dalloc(m, &stream, total, false))) return rc;
+    if ((rc = dalloc(m, &off_dev, (int64_t)off.size(), false))) return rc;
+    HIPCHK(ctx, hipMemcpy(off_dev, off.data(), off.size() * 8, hipMemcpyHostToDevice));
+    for (int l = 0; l < c.n_layers; l++) {
+        const DevTensor qkv[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
+        const DevTensor wo[1] = {m->L(l, L2H_WO)};
+        const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
+        const DevTensor w2[1] = {m->L(l, L2H_W2)};
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 0, l, qkv, 3, grid));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 1, l, wo, 1, grid));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 2, l, w13, 2, grid));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 3, l, w2, 1, grid));
+    }
+    HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    a.stream = stream;
+    a.wave_off = off_dev;
+#define TA(p, n)                           \
+    if ((rc = dalloc(m, &(p), (n), true))) \
+        return rc;
+    TA(a.x_a, c.dim);
+    TA(a.x_b, c.dim);
+    TA(a.xb, c.dim);
+    TA(a.q, c.dim);
+    TA(a.kcur, m->kv_dim);
+    TA(a.vcur, m->kv_dim);
+    TA(a.hb, c.hidden_dim);
+    TA(a.amax, 2 * grid);
+    TA(a.abort_flag, 1);
+#undef TA
+    a.kc = m->kc;
+    a.vc = m->vc;
+    a.logits = m->logits;
+    a.rms_att = m->L(0, L2H_RMS_ATT).f32;
+    a.rms_ffn = m->L(0, L2H_RMS_FFN).f32;
+    a.rms_final = m->glob[L2H_RMS_FINAL].f32;
+    a.norm_stride = m->L(0, L2H_RMS_ATT).layer_stride / 4;
+    a.cache_layer_elems = m->cache_layer_elems;
+    a.emb = m->glob[L2H_TOK_EMB];
+    a.ctl = m->ctl;
+    a.prompt = m->prompt_dev;
+    a.out_tokens = m->out_tokens;
+    a.max_out = m->max_out;
+    a.spin_limit = 1u << 20;
+    m->flow_args = a;
+    m->flow_grid = grid;
+    m->flow_cls_type = cls_type;
+    m->flow_gen = 1;
+    m->flow = true;
+    return L2H_OK;
+}
+
+static hipError_t flow_launch_token(l2h_model *m) {
+    if (g_flow_bound != m) {
+        hipError_t eb = k_flow_bind(m->ctx->stream, m->flow_args);
+        if (eb != hipSuccess) return eb;
+        g_flow_bound = m;
+    }
+    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, m->flow_cls_type, m->flow_grid);
+    if (e == hipSuccess) m->flow_gen += 5u * (unsigned)m->c.n_layers + 2u;
+    return e;
+}
+
 static hipError_t mega_launch_token(l2h_model *m) {
     if (g_bound_model != m) {
         hipError_t e = k_mega_bind(m->ctx->stream, m->mega_ph);
@@ -705,10 +808,11 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
 #undef DA
     HIPCHK(ctx, hipDeviceSynchronize());
     if ((rc = mega_setup(m))) return rc;
+    if ((rc = flow_setup(m))) return rc;
 
     // Record the launch sequence of one token; positions and tokens are read from the
     // control block on the device, so the recording is replayed unchanged for every step.
-    if (!m->mega && !getenv("L2H_NO_GRAPH")) {
+    if (!m->mega && !m->flow && !getenv("L2H_NO_GRAPH")) {
         HIPCHK(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeGlobal));
         hipError_t e = enqueue_token(m);
         hipGraph_t g = nullptr;
@@ -728,7 +832,10 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
 static int run_steps(l2h_model *m, int n) {
     l2h_ctx *ctx = m->ctx;
     for (int i = 0; i < n; i++) {
-        if (m->mega) {
+        if (m->flow) {
+            hipError_t e = flow_launch_token(m);
+            if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "decode kernel launch failed: %s", hipGetErrorString(e));
+        } else if (m->mega) {
             hipError_t e = mega_launch_token(m);
             if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "decode kernel launch failed: %s", hipGetErrorString(e));
         } else if (m->exec) {
@@ -743,6 +850,13 @@ static int run_steps(l2h_model *m, int n) {
 
 // after the stream has drained: did a workgroup of the persistent kernel give up at a barrier?
 static int mega_check(l2h_model *m) {
+    if (m->flow) {
+        unsigned int ab = 0;
+        HIPCHK(m->ctx, hipMemcpy(&ab, m->flow_args.abort_flag, 4, hipMemcpyDeviceToHost));
+        if (!ab) return L2H_OK;
+        HIPCHK(m->ctx, hipMemset(m->flow_args.abort_flag, 0, 4));
+        return set_err(m->ctx, L2H_EHIP, "streaming decode kernel: a wait for activations timed out");
+    }
     if (!m->mega) return L2H_OK;
     unsigned int ab = 0;
     HIPCHK(m->ctx, hipMemcpy(&ab, &m->bar->abort, 4, hipMemcpyDeviceToHost));

@@ -128,6 +128,41 @@ struct MegaArgs {
 #endif
 };
 
+// Streaming decode kernel (k_flow.hip): geometry of one matvec phase, and the kernel's arguments.
+struct FlowGeom {
+    int n_rows;  // logical rows
+    int rpw;     // rows per workgroup (even)
+    int ppr;     // pieces per row
+    int K;       // input length
+};
+struct FlowArgs {
+    const unsigned char *stream;  // per-wavefront weight streams
+    const int64_t *wave_off;      // [grid * 16] byte offset of each wavefront's stream
+    // activations as {fp32 value, epoch} words
+    unsigned long long *x_a, *x_b, *xb, *q, *kcur, *vcur, *hb, *amax;
+    float *kc, *vc, *logits;
+    const float *rms_att, *rms_ffn, *rms_final;
+    int64_t norm_stride;  // floats between the norm weights of consecutive layers
+    int64_t cache_layer_elems;
+    DevTensor emb;
+    DecodeCtl *ctl;
+    const int32_t *prompt;
+    int32_t *out_tokens;
+    int max_out;
+    unsigned int gen0, spin_limit;
+    unsigned int *abort_flag;
+    int dim, hidden, hs, n_heads, n_kv_heads, kv_dim, seq_len, n_layers, vocab, neox;
+    float theta_scale;
+    FlowGeom qkv, wo, w13, w2, cls;
+};
+bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls_type, int grid, std::string *why);
+int64_t k_flow_offsets(const FlowArgs &a, int cls_type, int grid, std::vector<int64_t> &off);
+// kind 0 q|k|v, 1 wo, 2 w1|w3, 3 w2 (of `layer`), 4 classifier; w: the phase's tensors
+hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream, const int64_t *wave_off_dev, int kind,
+                         int layer, const DevTensor *w, int nw, int grid);
+hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a);
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid);
+
 // ---- launchers (kernel files) ----------------------------------------------------------------
 // Each returns hipGetLastError() of its launch.
 hipError_t k_repack(hipStream_t s, const DevTensor &t, const void *raw_dev, bool inverse, void *raw_out);

@@ -99,6 +99,64 @@ def test_headline_shape_128_greedy_tokens(pkg, orc):
     assert _rel(logits, ref_logits) <= 1e-3
 
 
+# the streaming kernel (path 3) needs input lengths that are multiples of 2048 (4096 for a q6_K classifier)
+FLOW_CASES = {
+    "all_q4": ("PLAN_Q4_K", dict(dim=2048, hidden_dim=4096, n_layers=3, n_heads=16, n_kv_heads=4, vocab_size=1000,
+                                 seq_len=160, rope_freq_base=500000.0, rope_is_neox=False)),
+    "all_q4_neox": ("PLAN_Q4_K", dict(dim=2048, hidden_dim=2048, n_layers=2, n_heads=32, n_kv_heads=32, vocab_size=777,
+                                      seq_len=96, rope_freq_base=10000.0, rope_is_neox=True)),
+    "q4ks_headline_widths": ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8,
+                                                 vocab_size=32000, seq_len=192, rope_freq_base=500000.0,
+                                                 rope_is_neox=False)),
+}
+
+
+@pytest.mark.parametrize("case", sorted(FLOW_CASES))
+def test_streaming_kernel(pkg, orc, case):
+    """Path 3: one launch per token, weights streamed through per-wavefront LDS rings, activations
+    exchanged as tagged words.  Same bar as the other paths, and the per-phase path's logits are
+    reproduced bit for bit (same arithmetic; only the grouping of the fp64 partial sums differs,
+    which is reported if it ever shows)."""
+    from llama2_jl_amd import synth
+    plan, kw = FLOW_CASES[case]
+    lm = _model(pkg, plan, **kw)
+    cfg = lm.config
+    prompt = synth.seeded_prompt(5, 9, cfg.vocab_size)
+    n_new = 128 if case == "q4ks_headline_widths" else 40
+    n_new = min(n_new, cfg.seq_len - len(prompt))
+    dev = lm.device(path=3)
+    assert dev.path == 3
+    om = orc.model_from_language_model(lm, nthreads=16)
+    dev.reset()
+    for pos in range(3):
+        logits, am = dev.forward(int(prompt[pos]), pos)
+        ref = om.forward(int(prompt[pos]), pos, orc.GPU_SPEC)
+        assert _rel(logits, ref) <= 1e-3, (case, pos)
+        assert am == orc.argmax(ref)
+    for layer in range(cfg.n_layers):
+        k, v = dev.kv_read(layer, 0, 3)
+        rk, rv = om.kv_read(layer, 0, 3)
+        assert _rel(k, rk) <= 1e-5 and _rel(v, rv) <= 1e-5
+    dev.reset()
+    om.reset()
+    ids, logits = dev.generate_greedy(prompt, n_new, want_logits=True)
+    ref_ids, ref_logits = om.generate_greedy(prompt, n_new, orc.GPU_SPEC)
+    assert ids.tolist() == ref_ids.tolist(), case
+    assert _rel(logits, ref_logits) <= 1e-3, case
+    lm2 = _model(pkg, plan, **kw)
+    ids1, logits1 = lm2.device(path=1).generate_greedy(prompt, n_new, want_logits=True)
+    same = np.array_equal(logits1.view(np.uint32), logits.view(np.uint32))
+    print("\n[%s] streaming kernel: logits rel err vs oracle %.3g; bit-identical to the per-phase path: %s"
+          % (case, _rel(logits, ref_logits), same))
+    assert ids1.tolist() == ids.tolist()
+
+
+def test_streaming_kernel_refuses_other_shapes(pkg):
+    plan, kw = CASES["q4ks_gqa"]  # dim 512: rows do not split into whole pieces
+    with pytest.raises(pkg.L2HError):
+        _model(pkg, plan, **kw).device(path=3)
+
+
 def test_paths_agree_bit_for_bit(pkg):
     """Both launch paths run the same device functions: identical logits and tokens."""
     from llama2_jl_amd import synth
