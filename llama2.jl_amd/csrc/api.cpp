@@ -702,6 +702,10 @@ static int flow_setup(l2h_model *m) {
     a.out_tokens = m->out_tokens;
     a.max_out = m->max_out;
     a.spin_limit = 1u << 20;
+#ifdef L2H_TIMELINE
+    if ((rc = dalloc(m, &m->timeline, (int64_t)grid * 64 + 1024, true))) return rc;
+    a.timeline = m->timeline;
+#endif
     m->flow_args = a;
     m->flow_grid = grid;
     m->flow_cls_type = cls_type;
@@ -1466,8 +1470,8 @@ extern "C" int l2h_profile_stream_read(l2h_ctx *ctx, int64_t n_bytes, int iters,
 #ifdef L2H_TIMELINE
 // profiling build only: wall-clock stamps (100 MHz) of the last persistent-kernel launch
 extern "C" int l2h_debug_timeline(l2h_model *m, long long *out, int n_wg) {
-    if (!m || !m->mega || !m->timeline) return L2H_ESTATE;
-    HIPCHK(m->ctx, hipMemcpy(out, m->timeline, (size_t)n_wg * 64 * 8, hipMemcpyDeviceToHost));
+    if (!m || !(m->mega || m->flow) || !m->timeline) return L2H_ESTATE;
+    HIPCHK(m->ctx, hipMemcpy(out, m->timeline, ((size_t)n_wg * 64 + (m->flow ? 1024 : 0)) * 8, hipMemcpyDeviceToHost));
     return L2H_OK;
 }
 extern "C" int l2h_debug_timeline2(l2h_model *m, long long *out, int n_wg) {

@@ -26,7 +26,7 @@
 #define FLOW_SLOT 1152      // one q4_K piece: 8 headers (128 B) + 8 x 128 B of quants
 #define FLOW_Q6_PIECE 3360  // 16 q6_K super-blocks: ql 2048, qh 1024, scales 256, d 32
 #define FLOW_NW 16
-#define FLOW_ACT_BYTES 20480
+#define FLOW_ACT_BYTES 28672
 #define FLOW_MAX_PIECES 1024  // per workgroup and phase
 #define FLOW_MAX_ROWS 512     // per workgroup and phase
 
@@ -63,18 +63,25 @@ __host__ __device__ inline int flow_n_local(const FlowGeom &g, int wg) {
     const int hi = lo + g.rpw < g.n_rows ? lo + g.rpw : g.n_rows;
     return hi > lo ? hi - lo : 0;
 }
-// pieces of workgroup wg that wavefront `wave` takes: local piece numbers wave, wave+16, ...
+// pieces of workgroup wg that wavefront `wave` takes: a contiguous run of the workgroup's pieces
+// (consecutive pieces of a row stay in one wavefront where possible), the first np % 16 wavefronts
+// one piece longer than the rest
 __host__ __device__ inline int flow_wave_pieces(const FlowGeom &g, int wg, int wave) {
     const int np = flow_n_local(g, wg) * g.ppr;
-    return np > wave ? (np - wave + FLOW_NW - 1) / FLOW_NW : 0;
+    return np / FLOW_NW + (wave < np % FLOW_NW ? 1 : 0);
+}
+__host__ __device__ inline int flow_wave_start(const FlowGeom &g, int wg, int wave) {
+    const int np = flow_n_local(g, wg) * g.ppr;
+    const int base = np / FLOW_NW, rem = np % FLOW_NW;
+    return wave * base + (wave < rem ? wave : rem);
 }
 
 // logical row L of a phase -> (tensor of the phase, row in it).  Logical rows put the two rows an
 // epilogue combines next to each other: (w1 row u, w3 row u) and the two halves of a RoPE pair.
-__host__ __device__ inline void flow_row_src(int kind, int64_t L, int dim, int kv_dim, int hs, int neox, int &seg,
-                                             int64_t &row) {
+__host__ __device__ inline void flow_row_src(int kind, int L, int dim, int kv_dim, int hs, int neox, int &seg,
+                                             int &row) {
     if (kind == 2) {  // w1 | w3
-        seg = (int)(L & 1);
+        seg = L & 1;
         row = L >> 1;
         return;
     }
@@ -86,8 +93,7 @@ __host__ __device__ inline void flow_row_src(int kind, int64_t L, int dim, int k
     seg = L < dim ? 0 : (L < dim + kv_dim ? 1 : 2);
     row = L - (seg == 0 ? 0 : (seg == 1 ? dim : dim + kv_dim));
     if (neox && seg != 2) {  // neox pairs element i with i + hs/2 (reference src/inference.jl:146)
-        const int64_t h = row / hs;
-        const int e = (int)(row % hs);
+        const int h = row / hs, e = row % hs;
         row = h * hs + (e >> 1) + ((e & 1) ? (hs >> 1) : 0);
     }
 }
@@ -104,6 +110,35 @@ struct Ring {
     int drain_mark;             // pieces known to have landed (issued before the last full wait)
     int iss_layer, iss_kind, iss_left;
 };
+
+// Headers inside the streams carry the twelve 6-bit scale bytes of a q4_K super-block (reference
+// src/kquants.jl:80-109) regrouped so that a lane finds the four values of its sub-block pair j in
+// one 24-bit field f_j = sc(2j) | sc(2j+1) << 6 | m(2j) << 12 | m(2j+1) << 18:
+//   word 0 = d | dmin << 16;  word 1+k (k = 0..2) = f_k | byte k of f_3 << 24.
+__host__ __device__ inline uint32_t flow_pair_field(int sc_a, int sc_b, int m_a, int m_b) {
+    return (uint32_t)sc_a | (uint32_t)sc_b << 6 | (uint32_t)m_a << 12 | (uint32_t)m_b << 18;
+}
+__device__ __forceinline__ uint4 flow_encode_hdr(const uint4 hdr) {
+    uint32_t f[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        int sa, sb, ma, mb;
+        kq_scales_pair(hdr, j, sa, sb, ma, mb);
+        f[j] = flow_pair_field(sa, sb, ma, mb);
+    }
+    return make_uint4(hdr.x, f[0] | (f[3] & 0xFF) << 24, f[1] | ((f[3] >> 8) & 0xFF) << 24, f[2] | (f[3] >> 16) << 24);
+}
+// this lane's field (j = 0..3 is fixed per lane: the selects use lane-constant conditions)
+__device__ __forceinline__ void flow_decode_pair(const uint4 hdr, int j, int &sc_a, int &sc_b, int &m_a, int &m_b) {
+    const uint32_t fw = j == 0 ? hdr.y : (j == 1 ? hdr.z : hdr.w);
+    const uint32_t t = __builtin_amdgcn_perm(hdr.z, hdr.y, 0x0c0c0703u);  // byte 3 of word 1, byte 3 of word 2
+    const uint32_t g = __builtin_amdgcn_perm(hdr.w, t, 0x0c070100u);      // ... and byte 3 of word 3
+    const uint32_t f = j == 3 ? g : fw;
+    sc_a = (int)(f & 63);
+    sc_b = (int)((f >> 6) & 63);
+    m_a = (int)((f >> 12) & 63);
+    m_b = (int)((f >> 18) & 63);
+}
 
 // geometry of layer phase `kind`, field by field (scalar selects of scalar loads)
 __device__ __forceinline__ FlowGeom flow_geom(const FlowArgs &a, int kind) {
@@ -137,8 +172,11 @@ __device__ __forceinline__ void ring_uniform(Ring &r) {
 // fetch the next q4_K piece of this wavefront's stream, if the layer phases have one left
 __device__ __forceinline__ void flow_issue_q4(Ring &r, const FlowArgs &a, unsigned char *ring_base, int wg, int wave,
                                               int lane) {
-    ring_uniform(r);
-    while (r.iss_left == 0) {
+    // (the bookkeeping is the same on every lane; saying so where it steers a branch keeps the
+    // branches on the scalar unit)
+    while (uni(r.iss_left) == 0) {
+        r.iss_layer = uni(r.iss_layer);
+        r.iss_kind = uni(r.iss_kind);
         if (r.iss_layer >= a.n_layers) return;
         if (++r.iss_kind == 4) {
             r.iss_kind = 0;
@@ -146,7 +184,7 @@ __device__ __forceinline__ void flow_issue_q4(Ring &r, const FlowArgs &a, unsign
         }
         r.iss_left = uni(flow_wave_pieces(flow_geom(a, r.iss_kind), wg, wave));
     }
-    unsigned char *slot = ring_base + (r.issued % FLOW_D) * FLOW_SLOT;
+    unsigned char *slot = ring_base + (uni(r.issued) % FLOW_D) * FLOW_SLOT;
     const unsigned char *g = r.gptr;
     if (lane < 8) __builtin_amdgcn_global_load_lds((const AS1 void *)(g + lane * 16), (AS3 void *)slot, 16, 0, 2);
     __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 128 + lane * 16), (AS3 void *)(slot + 128), 16, 0, 2);
@@ -166,6 +204,11 @@ template <int OPS>
 __device__ __forceinline__ void flow_wait_piece(const Ring &r) {
     if (uni(r.consumed) < uni(r.drain_mark)) return;
     const int younger = uni(r.issued - 1 - r.consumed);
+    constexpr int DEPTH = OPS == 2 ? FLOW_D : 2;
+    if (younger >= DEPTH - 1) {  // the steady state: a full ring
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * (DEPTH - 1)) : "memory");
+        return;
+    }
     switch (younger) {
     case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
     case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * 1) : "memory"); break;
@@ -309,14 +352,15 @@ __device__ __forceinline__ XLds flow_x() {
 
 __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ppr = g.ppr;
-    const int np = uni(flow_n_local(g, wg) * ppr);
+    const int ppr = uni(g.ppr);
+    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     const XLds x = flow_x();
     flow_drain(r);
-    for (int j = wave; j < np; j += FLOW_NW) {
-        ring_uniform(r);
+    int part = uni(start % ppr);
+    double acc = 0.0;
+    for (int k = 0; k < cnt; k++) {
         flow_wait_piece<2>(r);
-        const unsigned slot = r.lds + (unsigned)(r.consumed % FLOW_D) * FLOW_SLOT;
+        const unsigned slot = r.lds + (unsigned)(uni(r.consumed) % FLOW_D) * FLOW_SLOT;
         Chunk<L2H_TYPE_Q4_K> ch;
         asm volatile("ds_read_b128 %0, %2 offset:128\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
                      : "=&v"(ch.w), "=&v"(ch.hdr)
@@ -324,10 +368,22 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
                      : "memory");
         r.consumed++;
         flow_issue_q4(r, c_flow, ring_base, wg, wave, lane);  // the slot is free again
-        const int part = j % ppr;
-        const double t = chunk_term<false>(ch, part * 64 + lane, x, nullptr, nullptr, 0);
-        const double v = wave_sum_f64_dpp(t);
-        if (lane == 0) s_part[j] = v;
+        {
+            int sc_a, sc_b, m_a, m_b, i_sc, i_min;
+            flow_decode_pair(ch.hdr, (lane & 7) >> 1, sc_a, sc_b, m_a, m_b);
+            acc += q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, part * 64 + lane, x, i_sc, i_min);
+        }
+        // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot
+        // in s_part, the run's total goes to its last piece and zero to the others
+        const bool last = k == cnt - 1 || uni(part) == ppr - 1;
+        if (last) {
+            const double v = wave_sum_f64_dpp(acc);
+            if (lane == 0) s_part[start + k] = v;
+            acc = 0.0;
+        } else if (lane == 0) {
+            s_part[start + k] = 0.0;
+        }
+        part = part == ppr - 1 ? 0 : part + 1;
     }
 }
 
@@ -335,9 +391,8 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
 // holds two pieces
 #define FLOW_Q6_D 2
 __device__ __forceinline__ void flow_issue_q6(Ring &r, unsigned char *ring_base, int lane) {
-    ring_uniform(r);
-    if (r.iss_left == 0) return;
-    unsigned char *slot = ring_base + (r.issued % FLOW_Q6_D) * FLOW_Q6_PIECE;
+    if (uni(r.iss_left) == 0) return;
+    unsigned char *slot = ring_base + (uni(r.issued) % FLOW_Q6_D) * FLOW_Q6_PIECE;
     const unsigned char *g = r.gptr;
     __builtin_amdgcn_global_load_lds((const AS1 void *)(g + lane * 16), (AS3 void *)slot, 16, 0, 2);
     __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 1024 + lane * 16), (AS3 void *)(slot + 1024), 16, 0, 2);
@@ -353,15 +408,16 @@ __device__ __forceinline__ void flow_issue_q6(Ring &r, unsigned char *ring_base,
 
 __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ppr = g.ppr;
-    const int np = flow_n_local(g, wg) * ppr;
+    const int ppr = uni(g.ppr);
+    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     const int b = lane >> 2, c = lane & 3, n = c >> 1, h = c & 1;
     const XLds x = flow_x();
     flow_drain(r);
-    for (int j = wave; j < np; j += FLOW_NW) {
-        ring_uniform(r);
+    int part = uni(start % ppr);
+    double acc = 0.0;
+    for (int k = 0; k < cnt; k++) {
         flow_wait_piece<5>(r);
-        const unsigned slot = r.lds + (unsigned)(r.consumed % FLOW_Q6_D) * FLOW_Q6_PIECE;
+        const unsigned slot = r.lds + (unsigned)(uni(r.consumed) % FLOW_Q6_D) * FLOW_Q6_PIECE;
         Chunk<L2H_TYPE_Q6_K> ch;
         uint32_t d16;
         asm volatile("ds_read_b128 %0, %5\n\tds_read_b128 %1, %5 offset:32\n\tds_read_b128 %2, %6 offset:2048\n\t"
@@ -373,10 +429,16 @@ __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigne
         ch.d = d16;
         r.consumed++;
         flow_issue_q6(r, ring_base, lane);
-        const int part = j % ppr;
-        const double t = chunk_term<false>(ch, part * 64 + lane, x, nullptr, nullptr, 0);
-        const double v = wave_sum_f64_dpp(t);
-        if (lane == 0) s_part[j] = v;
+        acc += chunk_term<false>(ch, part * 64 + lane, x, nullptr, nullptr, 0);
+        const bool last = k == cnt - 1 || uni(part) == ppr - 1;
+        if (last) {
+            const double v = wave_sum_f64_dpp(acc);
+            if (lane == 0) s_part[start + k] = v;
+            acc = 0.0;
+        } else if (lane == 0) {
+            s_part[start + k] = 0.0;
+        }
+        part = part == ppr - 1 ? 0 : part + 1;
     }
 }
 
@@ -398,12 +460,11 @@ __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_
     const int n_local = flow_n_local(a.qkv, wg), tid = threadIdx.x;
     flow_row_values(n_local, a.qkv.ppr);
     if (tid >= n_local) return;
-    const int64_t L = (int64_t)wg * a.qkv.rpw + tid;
-    int seg;
-    int64_t row;
+    const int L = wg * a.qkv.rpw + tid;
+    int seg, row;
     flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
     const float val = s_val[tid], other = s_val[tid ^ 1];
-    const int hh = (int)(row / a.hs), e = (int)(row % a.hs);
+    const int hh = row / a.hs, e = row % a.hs;
     if (seg == 2) {
         (a.vc + (int64_t)l * a.cache_layer_elems)[((int64_t)hh * a.seq_len + pos) * a.hs + e] = val;
         tag_store(a.vcur + row, val, e_q);
@@ -424,8 +485,9 @@ __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_
     }
 }
 
-// dst = src + result (x .+= ..., :284,305); which = 1 after wo (x_a -> x_b), 3 after w2 (x_b -> x_a)
-__device__ __noinline__ void flow_finish_resid(int which, int wg, unsigned e_src, unsigned e_dst) {
+// dst = old + result (x .+= ..., :284,305); which = 1 after wo (-> x_b), 3 after w2 (-> x_a); `old` is
+// this thread's row of the other buffer, fetched before the loop
+__device__ __noinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsigned e_src, unsigned e_dst) {
     const FlowArgs &a = c_flow;
     const FlowGeom &g = which == 1 ? a.wo : a.w2;
     const u64 *src = which == 1 ? a.x_a : a.x_b;
@@ -433,8 +495,9 @@ __device__ __noinline__ void flow_finish_resid(int which, int wg, unsigned e_src
     const int n_local = flow_n_local(g, wg), tid = threadIdx.x;
     flow_row_values(n_local, g.ppr);
     if (tid >= n_local) return;
-    const int64_t row = (int64_t)wg * g.rpw + tid;
-    tag_store(dst + row, flow_read(src + row, e_src) + s_val[tid], e_dst);
+    const int row = wg * g.rpw + tid;
+    const float old = tag_is(oldw, e_src) ? tag_val(oldw) : flow_read(src + row, e_src);
+    tag_store(dst + row, old + s_val[tid], e_dst);
 }
 
 // SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u
@@ -544,11 +607,21 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
     double *s_q = (double *)s_act;
     double *s_p = s_q + hs;
     double *s_r = s_p + seq_len;
-    float *s_att = (float *)(s_r + (blockDim.x / hs) * hs);
-    float *s_kcur = s_att + seq_len;
+    float *s_att = (float *)(s_r + (FLOW_NW * hs > 1024 ? FLOW_NW * hs : 1024));
+    float *s_kcur = s_att + ((seq_len + 3) & ~3);
     float *s_vcur = s_kcur + hs;
     const int tid = threadIdx.x;
     bool ok = true;
+#ifdef L2H_TIMELINE
+    int atl = 0;
+#define ATL()                                                                                                    \
+    do {                                                                                                         \
+        if (a.timeline && tid == 0 && layer == 2 && atl < 16) a.timeline[256 * 64 + h * 16 + atl++] = wall_clock64(); \
+    } while (0)
+#else
+#define ATL()
+#endif
+    ATL();
     __syncthreads();  // the activation area is free
     if (tid < 3 * hs) {
         const int which = tid / hs, i = tid % hs;
@@ -578,39 +651,49 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
         if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return false;
     }
+    ATL();
     const float scale = sqrtf((float)hs);
     float mx = -INFINITY;
-    for (int t = tid; t < np; t += blockDim.x) {
-        double acc = 0.0;
-        if (t == pos) {
-            for (int i = 0; i < hs; i++) acc = fma(s_q[i], (double)s_kcur[i], acc);
-        } else {
-            const float *kp = kc + ((int64_t)kvh * (hs >> 2) * seq_len + t) * 4;
-            int i4 = 0;
-            for (; i4 + 4 <= (hs >> 2); i4 += 4) {
-                float4 kv[4];
+    // scores: thread = (timestep tl of a block of 256, quarter of the head dimension); the quarter's
+    // 16-byte loads are all in flight at once; quarters are added in order (fp64)
+    {
+        const int tl = tid & 255, part = tid >> 8, per = hs >> 4;  // hs is a multiple of 16, at most 128
+        double *s_sp = s_r;                                        // [4][256]
+        for (int t0 = 0; t0 < np; t0 += 256) {
+            const int t = t0 + tl;
+            double acc = 0.0;
+            if (t < np) {
+                if (t == pos) {
+                    for (int i = 4 * part * per; i < 4 * (part + 1) * per; i++) acc = fma(s_q[i], (double)s_kcur[i], acc);
+                } else {
+                    const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
+                    float4 kv[8];
 #pragma unroll
-                for (int u = 0; u < 4; u++) kv[u] = *(const float4 *)(kp + (int64_t)(i4 + u) * seq_len * 4);
+                    for (int u = 0; u < 8; u++)
+                        if (u < per) kv[u] = kp[(int64_t)u * seq_len];
 #pragma unroll
-                for (int u = 0; u < 4; u++) {
-                    acc = fma(s_q[4 * (i4 + u) + 0], (double)kv[u].x, acc);
-                    acc = fma(s_q[4 * (i4 + u) + 1], (double)kv[u].y, acc);
-                    acc = fma(s_q[4 * (i4 + u) + 2], (double)kv[u].z, acc);
-                    acc = fma(s_q[4 * (i4 + u) + 3], (double)kv[u].w, acc);
+                    for (int u = 0; u < 8; u++)
+                        if (u < per) {
+                            const double *qq = s_q + 4 * (part * per + u);
+                            acc = fma(qq[0], (double)kv[u].x, acc);
+                            acc = fma(qq[1], (double)kv[u].y, acc);
+                            acc = fma(qq[2], (double)kv[u].z, acc);
+                            acc = fma(qq[3], (double)kv[u].w, acc);
+                        }
                 }
             }
-            for (; i4 < (hs >> 2); i4++) {
-                const float4 kv = *(const float4 *)(kp + (int64_t)i4 * seq_len * 4);
-                acc = fma(s_q[4 * i4 + 0], (double)kv.x, acc);
-                acc = fma(s_q[4 * i4 + 1], (double)kv.y, acc);
-                acc = fma(s_q[4 * i4 + 2], (double)kv.z, acc);
-                acc = fma(s_q[4 * i4 + 3], (double)kv.w, acc);
+            s_sp[part * 256 + tl] = acc;
+            __syncthreads();
+            if (part == 0 && t < np) {
+                const double v = ((s_sp[tl] + s_sp[256 + tl]) + s_sp[512 + tl]) + s_sp[768 + tl];
+                const float sc = (float)v / scale;
+                s_att[t] = sc;
+                mx = fmaxf(mx, sc);
             }
+            __syncthreads();
         }
-        const float sc = (float)acc / scale;
-        s_att[t] = sc;
-        mx = fmaxf(mx, sc);
     }
+    ATL();
     mx = block_max_f32(mx, s_redf);
     double sum = 0.0;
     for (int t = tid; t < np; t += blockDim.x) {
@@ -621,26 +704,50 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
     const float sf = (float)block_sum_f64(sum, s_red);
     for (int t = tid; t < np; t += blockDim.x) s_p[t] = (double)(s_att[t] / sf);
     __syncthreads();
-    const int ngrp = blockDim.x / hs;
-    const int i = tid % hs, grp = tid / hs;
-    if (grp < ngrp) {
-        const float *vp = vc + (int64_t)kvh * seq_len * hs + i;
-        double acc = 0.0;
-        int t = grp;
-        for (; t + 3 * ngrp < pos; t += 4 * ngrp) {  // four loads in flight; the cache holds positions < pos
-            float v[4];
+    ATL();
+    // values: thread = (16-byte group i4 of the head dimension, timestep group), up to eight loads in
+    // flight; the groups of one wavefront are folded with lane exchanges, the rest through LDS
+    const int n4 = hs >> 2;         // a power of two (hs 32, 64, 128)
+    const int ngrp = blockDim.x / n4;
+    {
+        const int i4 = tid & (n4 - 1), grp = tid / n4;
+        const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
+        double acc[4] = {0.0, 0.0, 0.0, 0.0};
+        for (int t0 = grp; t0 < np; t0 += 8 * ngrp) {
+            float4 v[8];
 #pragma unroll
-            for (int u = 0; u < 4; u++) v[u] = vp[(int64_t)(t + u * ngrp) * hs];
+            for (int u = 0; u < 8; u++) {
+                const int t = t0 + u * ngrp;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (t < pos) v[u] = vp[(int64_t)t * n4];
+                else if (t == pos) v[u] = *(const float4 *)(s_vcur + 4 * i4);
+            }
 #pragma unroll
-            for (int u = 0; u < 4; u++) acc = fma(s_p[t + u * ngrp], (double)v[u], acc);
+            for (int u = 0; u < 8; u++) {
+                const int t = t0 + u * ngrp;
+                if (t < np) {
+                    const double p = s_p[t];
+                    acc[0] = fma(p, (double)v[u].x, acc[0]);
+                    acc[1] = fma(p, (double)v[u].y, acc[1]);
+                    acc[2] = fma(p, (double)v[u].z, acc[2]);
+                    acc[3] = fma(p, (double)v[u].w, acc[3]);
+                }
+            }
         }
-        for (; t < np; t += ngrp) acc = fma(s_p[t], (double)(t == pos ? s_vcur[i] : vp[(int64_t)t * hs]), acc);
-        s_r[grp * hs + i] = acc;
+        for (int off = n4; off < 64; off <<= 1)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[c] += __shfl_xor(acc[c], off, WAVE);
+        if ((tid & 63) < n4) {
+            const int wv = tid >> 6;
+#pragma unroll
+            for (int c = 0; c < 4; c++) s_r[wv * hs + 4 * i4 + c] = acc[c];
+        }
     }
     __syncthreads();
+    ATL();
     if (tid < hs) {
         double acc = 0.0;
-        for (int k = 0; k < ngrp; k++) acc += s_r[k * hs + tid];
+        for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
         tag_store(a.xb + (int64_t)h * hs + tid, (float)acc, e_out);
     }
     __syncthreads();
@@ -664,8 +771,25 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     r.iss_layer = 0;
     r.iss_kind = 0;
     r.iss_left = flow_wave_pieces(a.qkv, wg, wave);
+    ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
     for (int k = 0; k < FLOW_D; k++) flow_issue_q4(r, a, ring_base, wg, wave, lane);
 
+#ifdef L2H_TIMELINE
+    int tl_n = 0;
+#define FTL()                                                                                   \
+    do {                                                                                        \
+        if (a.timeline && tid == 0 && tl_n < 64) a.timeline[wg * 64 + tl_n++] = wall_clock64(); \
+    } while (0)
+#define FTLS()          \
+    do {                \
+        __syncthreads(); \
+        FTL();          \
+    } while (0)
+#else
+#define FTL()
+#define FTLS()
+#endif
+    FTL();
 #define LEAVE()        \
     do {               \
         flow_drain(r); \
@@ -694,31 +818,54 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         // ---- rmsnorm (:244), q, k, v (:247-249), rope (:255-256), cache append (:259-260) ----
         {
             const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
-            const bool ok = l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok)
-                                   : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok);
+            const bool ok = uni(l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok)
+                                       : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok));
             if (!ok) LEAVE();
+            FTL();
             flow_loop_q4(a.qkv, r, ring_base, wg);
+            FTL();
+            FTLS();
             flow_finish_qkv(l, wg, pos, e_q);
+            FTL();
         }
         // ---- attention (:263-278): head h on workgroup h*stride + h%stride ----
         {
             const int stride = nwg / a.n_heads;
             const int h = wg / stride;
             if (h < a.n_heads && wg % stride == h % stride)
-                if (!flow_attention(l, h, pos, e_q, e_att)) LEAVE();
+                if (!uni(flow_attention(l, h, pos, e_q, e_att))) LEAVE();
+            FTL();
         }
         // ---- x += wo * xb (:281-284) ----
-        if (!flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok)) LEAVE();
-        flow_loop_q4(a.wo, r, ring_base, wg);
-        flow_finish_resid(1, wg, e_x, e_wo);
+        if (!uni(flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok))) LEAVE();
+        FTL();
+        {
+            const u64 oldw = tid < flow_n_local(a.wo, wg) ? tag_load(a.x_a + wg * a.wo.rpw + tid) : 0;
+            flow_loop_q4(a.wo, r, ring_base, wg);
+            FTL();
+            FTLS();
+            flow_finish_resid(1, wg, oldw, e_x, e_wo);
+        }
+        FTL();
         // ---- rmsnorm (:287), w1, w3 (:291-292), SwiGLU (:295-299) ----
-        if (!flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok)) LEAVE();
+        if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok))) LEAVE();
+        FTL();
         flow_loop_q4(a.w13, r, ring_base, wg);
+        FTL();
+        FTLS();
         flow_finish_w13(wg, e_w13);
+        FTL();
         // ---- x += w2 * hb (:302-305) ----
-        if (!flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok)) LEAVE();
-        flow_loop_q4(a.w2, r, ring_base, wg);
-        flow_finish_resid(3, wg, e_wo, e_w2);
+        if (!uni(flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok))) LEAVE();
+        FTL();
+        {
+            const u64 oldw = tid < flow_n_local(a.w2, wg) ? tag_load(a.x_b + wg * a.w2.rpw + tid) : 0;
+            flow_loop_q4(a.w2, r, ring_base, wg);
+            FTL();
+            FTLS();
+            flow_finish_resid(3, wg, oldw, e_wo, e_w2);
+        }
+        FTL();
     }
 
     // ---- final rmsnorm (:309) + classifier (:312); the ring restarts on the classifier's pieces ----
@@ -727,12 +874,13 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     r.issued = r.consumed = r.drain_mark = 0;
     r.iss_layer = a.n_layers;  // the layer phases are over: flow_issue_q4 fetches while iss_left lasts
     r.iss_left = flow_wave_pieces(a.cls, wg, wave);
+    ring_uniform(r);
     if (T_CLS == L2H_TYPE_Q6_K) {
         for (int k = 0; k < FLOW_Q6_D; k++) flow_issue_q6(r, ring_base, lane);
     } else {
         for (int k = 0; k < FLOW_D; k++) flow_issue_q4(r, a, ring_base, wg, wave, lane);
     }
-    if (!flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok)) LEAVE();
+    if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok))) LEAVE();
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
     else
@@ -770,12 +918,14 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
     const int per_wg = g.rpw * g.ppr;
     const int wg = blockIdx.x / per_wg, j = blockIdx.x % per_wg;
     if (j >= flow_n_local(g, wg) * g.ppr) return;
-    const int wave = j % FLOW_NW, idx = j / FLOW_NW;
-    const int64_t L = (int64_t)wg * g.rpw + j / g.ppr;
+    const int np = flow_n_local(g, wg) * g.ppr, base = np / FLOW_NW, rem = np % FLOW_NW;
+    const int wave = j < rem * (base + 1) ? j / (base + 1) : rem + (j - rem * (base + 1)) / base;
+    const int idx = j - flow_wave_start(g, wg, wave);
+    const int L = wg * g.rpw + j / g.ppr;
     const int part = j % g.ppr;
-    int seg;
-    int64_t row;
-    flow_row_src(p.kind == 4 ? 1 : p.kind, L, p.dim, p.kv_dim, p.hs, p.neox, seg, row);
+    int seg, row32;
+    flow_row_src(p.kind == 4 ? 1 : p.kind, L, p.dim, p.kv_dim, p.hs, p.neox, seg, row32);
+    const int64_t row = row32;
     const DevTensor &t = seg == 0 ? p.w[0] : (seg == 1 ? p.w[1] : p.w[2]);
     const int64_t layer_b = flow_layer_bytes(p.g4, wg, wave, 4);
     const int lane = threadIdx.x;
@@ -784,7 +934,7 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
                                         : (int64_t)p.layer * layer_b + flow_layer_bytes(p.g4, wg, wave, p.kind);
         uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + off + (int64_t)idx * FLOW_SLOT);
         const int64_t blk0 = row * t.nb + part * 8;
-        if (lane < 8) dst[lane] = t.hdr[blk0 + lane];
+        if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
         dst[8 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
     } else {  // q6_K classifier
         const int64_t off = (int64_t)p.n_layers * layer_b;
@@ -827,9 +977,9 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     if (a.dim % 2048 != 0 || a.hidden % 2048 != 0) return no("dim and hidden_dim must be multiples of 2048");
     if (cls_type == L2H_TYPE_Q6_K && a.dim % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
     if (a.hidden > 14336 || a.dim > 14336) return no("input vectors longer than 14336");
-    if (a.n_heads > grid || a.hs > 128 || 3 * a.hs > 1024) return no("head layout");
-    const size_t att = (size_t)a.hs * 8 + (size_t)a.seq_len * 8 + (size_t)(1024 / a.hs) * a.hs * 8 + (size_t)a.seq_len * 4 +
-                       (size_t)a.hs * 8;
+    if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 128)) return no("head size must be 32, 64 or 128");
+    const size_t att = (size_t)a.hs * 8 + (size_t)a.seq_len * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 +
+                       (size_t)((a.seq_len + 3) & ~3) * 4 + (size_t)a.hs * 8;
     if (att > FLOW_ACT_BYTES) return no("sequence too long for the attention area");
     a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim, L2H_TYPE_Q4_K, grid);
     a.wo = make_geom(a.dim, a.dim, L2H_TYPE_Q4_K, grid);

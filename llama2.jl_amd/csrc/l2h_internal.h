@@ -154,6 +154,9 @@ struct FlowArgs {
     int dim, hidden, hs, n_heads, n_kv_heads, kv_dim, seq_len, n_layers, vocab, neox;
     float theta_scale;
     FlowGeom qkv, wo, w13, w2, cls;
+#ifdef L2H_TIMELINE
+    long long *timeline;  // profiling build only: [workgroup][64] wall-clock stamps of the first phases
+#endif
 };
 bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls_type, int grid, std::string *why);
 int64_t k_flow_offsets(const FlowArgs &a, int cls_type, int grid, std::vector<int64_t> &off);

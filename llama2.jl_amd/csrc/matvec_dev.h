@@ -54,6 +54,9 @@ __device__ __forceinline__ void st_f64(double *p, double v) {
         *p = v;
 }
 
+// a*b + c on the 24-bit multiplier (v_mad_i32_i24): a and b must fit 24 bits
+__device__ __forceinline__ int mad24(int a, int b, int c) { return __mul24(a, b) + c; }
+
 __device__ __forceinline__ int sdot4(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }
@@ -168,16 +171,13 @@ __device__ __forceinline__ void load_chunk<L2H_TYPE_Q6_K>(Chunk<L2H_TYPE_Q6_K> &
 }
 
 // ---- this lane's fp64 share of one chunk; DEBUG also stores the per-block integer sums ----------
-template <bool DEBUG>
-__device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q4_K> &ch, int g, const XLds &x, int32_t *dbg_isc,
-                                             int32_t *dbg_imin, int64_t dbg_base) {
+// q4_K chunk given its unpacked scales: this lane's integer sums and their fp64 term
+__device__ __forceinline__ double q4_term(const uint4 w, uint32_t d_dmin, int sc_a, int sc_b, int m_a, int m_b, int g,
+                                          const XLds &x, int &i_sc, int &i_min) {
     const int b = g >> 3, c = g & 7, j = c >> 1, h = c & 1;
-    int sc_a, sc_b, m_a, m_b;
-    kq_scales_pair(ch.hdr, j, sc_a, sc_b, m_a, m_b);
     const int8_t *xb = x.qs + b * 256 + 64 * j + 16 * h;
     const uint4 xlo = *(const uint4 *)xb;
     const uint4 xhi = *(const uint4 *)(xb + 32);
-    const uint4 w = ch.w;
     int dot_a = 0, dot_b = 0;
     dot_a = sdot4(w.x & 0x0F0F0F0Fu, xlo.x, dot_a);
     dot_a = sdot4(w.y & 0x0F0F0F0Fu, xlo.y, dot_a);
@@ -188,13 +188,25 @@ __device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q4_K> &ch, int
     dot_b = sdot4((w.z >> 4) & 0x0F0F0F0Fu, xhi.z, dot_b);
     dot_b = sdot4((w.w >> 4) & 0x0F0F0F0Fu, xhi.w, dot_b);
     const int16_t *bs = x.bsums + b * 16 + 4 * j + h;
-    int i_sc = sc_a * dot_a + sc_b * dot_b;
-    int i_min = m_a * (int)bs[0] + m_b * (int)bs[2];
+    // every factor fits 24 bits (scales < 64, |dot| <= 16*15*127, |bsum| <= 16*127): full-rate multiplies
+    i_sc = mad24(sc_a, dot_a, __mul24(sc_b, dot_b));
+    i_min = mad24(m_a, (int)bs[0], __mul24(m_b, (int)bs[2]));
     const float yd = x.d[b];
-    const float dy = half_bits_to_float((uint16_t)(ch.hdr.x & 0xFFFF)) * yd;
-    const float my = half_bits_to_float((uint16_t)(ch.hdr.x >> 16)) * yd;
+    const float dy = half_bits_to_float((uint16_t)(d_dmin & 0xFFFF)) * yd;
+    const float my = half_bits_to_float((uint16_t)(d_dmin >> 16)) * yd;
     double t = (double)dy * (double)i_sc;
     t = fma(-(double)my, (double)i_min, t);
+    return t;
+}
+
+template <bool DEBUG>
+__device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q4_K> &ch, int g, const XLds &x, int32_t *dbg_isc,
+                                             int32_t *dbg_imin, int64_t dbg_base) {
+    const int b = g >> 3, c = g & 7, j = c >> 1;
+    int sc_a, sc_b, m_a, m_b;
+    kq_scales_pair(ch.hdr, j, sc_a, sc_b, m_a, m_b);
+    int i_sc, i_min;
+    const double t = q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, g, x, i_sc, i_min);
     if (DEBUG) {
         i_sc += __shfl_xor(i_sc, 1, WAVE);
         i_min += __shfl_xor(i_min, 1, WAVE);
@@ -235,8 +247,8 @@ __device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q5_K> &ch, int
 #undef Q5LO
 #undef Q5HI
     const int16_t *bs = x.bsums + b * 16 + 4 * j + h;
-    int i_sc = sc_a * dot_a + sc_b * dot_b;
-    int i_min = m_a * (int)bs[0] + m_b * (int)bs[2];
+    int i_sc = mad24(sc_a, dot_a, __mul24(sc_b, dot_b));
+    int i_min = mad24(m_a, (int)bs[0], __mul24(m_b, (int)bs[2]));
     const float yd = x.d[b];
     const float dy = half_bits_to_float((uint16_t)(ch.hdr.x & 0xFFFF)) * yd;
     const float my = half_bits_to_float((uint16_t)(ch.hdr.x >> 16)) * yd;
@@ -281,8 +293,9 @@ __device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q6_K> &ch, int
     const uint32_t scw = ch.sc;
     const int s0 = (int)(int8_t)(scw & 0xFF), s1 = (int)(int8_t)((scw >> 8) & 0xFF),
               s2 = (int)(int8_t)((scw >> 16) & 0xFF), s3 = (int)(int8_t)(scw >> 24);
-    int i_sc = s0 * (d0 - 32 * (int)bs[0]) + s1 * (d1 - 32 * (int)bs[2]) + s2 * (d2 - 32 * (int)bs[4]) +
-               s3 * (d3 - 32 * (int)bs[6]);
+    // |d - 32 bsum| < 2^18 and |scale| < 2^7: 24-bit (full-rate) multiplies are exact
+    int i_sc = mad24(s0, d0 - 32 * (int)bs[0],
+                       mad24(s1, d1 - 32 * (int)bs[2], mad24(s2, d2 - 32 * (int)bs[4], __mul24(s3, d3 - 32 * (int)bs[6]))));
     const float dy = half_bits_to_float((uint16_t)ch.d) * x.d[b];
     const double t = (double)dy * (double)i_sc;
     if (DEBUG) {
@@ -301,13 +314,15 @@ __device__ __forceinline__ double chunk_term(const Chunk<L2H_TYPE_Q6_K> &ch, int
 // ------------------------------------------------------------------------------------------
 template <int CTRL>
 __device__ __forceinline__ double dpp_f64(double v) {
-    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(v), CTRL, 0xF, 0xF, false);
-    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(v), CTRL, 0xF, 0xF, false);
+    // (quad_perm / row mirrors read a valid lane everywhere, so the "old" operand is never used)
+    const int l = __double2loint(v), h = __double2hiint(v);
+    const int lo = __builtin_amdgcn_update_dpp(l, l, CTRL, 0xF, 0xF, true);
+    const int hi = __builtin_amdgcn_update_dpp(h, h, CTRL, 0xF, 0xF, true);
     return __hiloint2double(hi, lo);
 }
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, false));
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, true));
 }
 __device__ __forceinline__ double readlane_f64(double v, int lane) {
     const int lo = __builtin_amdgcn_readlane(__double2loint(v), lane);
@@ -340,8 +355,8 @@ __device__ __forceinline__ float wave_max_f32_dpp(float v) {
 }
 // sum within aligned groups of 4 lanes
 __device__ __forceinline__ int quad_sum_i32(int v) {
-    v += __builtin_amdgcn_update_dpp(0, v, DPP_QUAD_SWAP1, 0xF, 0xF, false);
-    v += __builtin_amdgcn_update_dpp(0, v, DPP_QUAD_SWAP2, 0xF, 0xF, false);
+    v += __builtin_amdgcn_update_dpp(v, v, DPP_QUAD_SWAP1, 0xF, 0xF, true);
+    v += __builtin_amdgcn_update_dpp(v, v, DPP_QUAD_SWAP2, 0xF, 0xF, true);
     return v;
 }
 
