@@ -23,7 +23,8 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"8b-q4ks": 31264000}  # 31.23 MB read + 0.04 MB written
+# (workload, launch path) -> bytes; path 1: per matvec launch, 31.23 MB read + 0.04 MB written
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000}
 
 WORKLOADS = {
     # name: (plan, config kwargs, prompt length)
@@ -70,7 +71,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--workload", default="8b-q4ks", choices=sorted(WORKLOADS))
     ap.add_argument("--repeats", type=int, default=3, help="timed regions; the median is reported")
-    ap.add_argument("--path", type=int, default=0, help="0 auto, 1 kernel per phase, 2 persistent kernel")
+    ap.add_argument("--path", type=int, default=0, help="0 auto, 1 kernel per phase, 2 persistent kernel, 3 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -97,7 +98,7 @@ def main():
     t0 = time.time()
     dev = lm.device(path=args.path)
     ctx.sync()
-    log("uploaded in %.1f s; launch path %d (1 = kernel per phase, 2 = persistent kernel)" % (time.time() - t0, dev.path))
+    log("uploaded in %.1f s; launch path %d (1 = kernel per phase, 2 = persistent kernel, 3 = streaming kernel)" % (time.time() - t0, dev.path))
 
     w_bytes = synth.weight_bytes_per_token(lm)
     kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads
@@ -182,6 +183,16 @@ def main():
             n_launch += mult
     log("per-launch matvec timings:", json.dumps(per_kernel))
     achieved = tot_b / tot_us / 1e3  # GB/s over the launches of the dominant kernel within one token
+    kernel_name = "matvec_kq_kernel (k-quant x q8_K dequant-matvec)"
+    bytes_per_launch, launches, avg_launch_us = int(tot_b / max(1, n_launch)), n_launch, tot_us / max(1, n_launch)
+    if dev.path == 3:
+        # the streaming kernel: one launch per token does everything; its duration comes from HIP events
+        # around the K launches on the library's stream, its algorithmic bytes are the token's
+        _, ev_ms = dev.generate_greedy([first], K, pos0=pos0, timed=True)
+        kernel_name = "flow_token_kernel (whole token: q4_K/q6_K x q8_K matvecs, attention, argmax)"
+        bytes_per_launch, launches, avg_launch_us = int(bytes_per_token), 1, ev_ms * 1e3 / K
+        achieved = bytes_per_launch / avg_launch_us / 1e3
+        log("streaming kernel: %.1f us per launch (HIP events), %.0f GB/s of algorithmic bytes" % (avg_launch_us, achieved))
     stream_us = pkg.lib().l2h_profile_stream_read
     import ctypes
     us = ctypes.c_float()
@@ -211,7 +222,7 @@ def main():
 
     # HBM traffic of the dominant kernel per launch (FETCH_SIZE + WRITE_SIZE, scaled), measured with
     # rocprofv3 --pmc on this workload: profiles/pmc_fetch_write_bench_8b-q4ks.md
-    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(args.workload)
+    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dev.path))
 
     result = {
         "metric": "decode tok/s, Llama-3-8B-shape Q4_K_S, batch 1; % of HBM-BW roofline",
@@ -225,17 +236,20 @@ def main():
                    "roofline_tok_s_at_8TBs": round(roofline_tok_s, 1),
                    "frac_of_roofline": round(tok_s / roofline_tok_s, 4),
                    "tokens_head": tokens[:8]},
-        "roofline": {"bound": "hbm", "kernel": "matvec_kq_kernel (k-quant x q8_K dequant-matvec)",
+        "roofline": {"bound": "hbm", "kernel": kernel_name,
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "bytes_per_launch": int(tot_b / max(1, n_launch)), "launches_per_token": n_launch,
-                     "avg_launch_us": round(tot_us / max(1, n_launch), 2), "per_launch": per_kernel,
+                     "bytes_per_launch": bytes_per_launch, "launches_per_token": launches,
+                     "avg_launch_us": round(avg_launch_us, 2), "per_phase_kernels": per_kernel,
                      "measured_stream_read_GBs": round(stream_gbs, 1)},
         "cpu_baseline": cpu,
     }
     if prefill:
         result["prefill"] = prefill
     print(json.dumps(result), flush=True)
+    # release the device objects in order while the interpreter is still whole
+    dev.close()
+    ctx.sync()
 
 
 if __name__ == "__main__":

@@ -87,11 +87,14 @@ int l2h_model_set_tensor(l2h_model *m, int role, int layer, int ggml_type, const
 /* Reads a k-quant tensor back from the device layout into GGUF block order (the repack
  * is exactly invertible); host must hold ne1 * ne0/256 blocks.  For checks. */
 int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t host_bytes);
-/* How transformer! is launched (before finalize): 0 = automatic (currently 1), 1 = one kernel per phase
- * (recorded once, replayed per token), 2 = the persistent one-launch-per-token kernel, an error
- * at finalize if the model's tensor types have no such kernel.  Both run the same device code
- * and give the same results.  No counterpart in the reference.  l2h_model_path reports the
- * choice after finalize (1 or 2). */
+/* How transformer! is launched (before finalize): 0 = automatic (3 where the model fits it, else 1),
+ * 1 = one kernel per phase (recorded once, replayed per token), 2 = a persistent kernel per token
+ * with grid barriers between the phases, 3 = the streaming kernel per token (per-wavefront weight
+ * streams fetched ahead into LDS, activations exchanged as epoch-tagged words; needs q4_K layer
+ * matrices, a q4_K or q6_K classifier, dim and hidden_dim multiples of 2048, a short cache).
+ * 2 and 3 are an error at finalize if the model does not fit.  All paths compute the same
+ * arithmetic and give the same results.  No counterpart in the reference.  l2h_model_path reports
+ * the choice after finalize (1, 2 or 3). */
 int l2h_model_set_path(l2h_model *m, int path);
 int l2h_model_path(l2h_model *m);
 /* RunState(config) (src/inference.jl:88-100): checks every tensor is present, allocates

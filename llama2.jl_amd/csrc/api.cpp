@@ -220,7 +220,7 @@ struct l2h_model {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     // persistent decode kernel
-    int path_request = 0;  // 0 auto, 1 one kernel per phase, 2 persistent kernel required
+    int path_request = 0;  // 0 auto, 1 one kernel per phase, 2 persistent kernel, 3 streaming kernel (2, 3: required)
     bool mega = false;
     PhaseArgs mega_ph[5];  // q/k/v, wo, w1+w3, w2 of layer 0 and the classifier, planned for the persistent grid
     GridBar *bar = nullptr;
@@ -630,7 +630,9 @@ static int flow_setup(l2h_model *m) {
     l2h_ctx *ctx = m->ctx;
     const l2h_config &c = m->c;
     m->flow = false;
-    if (m->path_request != 3) return L2H_OK;
+    // automatic choice: this kernel where the model fits it (it is the fastest path), else one kernel per phase
+    if (m->path_request != 3 && m->path_request != 0) return L2H_OK;
+    const bool required = m->path_request == 3;
     FlowArgs a{};
     a.dim = c.dim;
     a.hidden = c.hidden_dim;
@@ -650,9 +652,9 @@ static int flow_setup(l2h_model *m) {
     const int cls_type = m->glob[L2H_OUTPUT].type;
     std::string why;
     if (!k_flow_plan(a, types.data(), (int)types.size(), cls_type, grid, &why))
-        return set_err(ctx, L2H_EINVAL, "streaming kernel not available: %s", why.c_str());
+        return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: %s", why.c_str()) : L2H_OK;
     if (m->L(0, L2H_RMS_ATT).layer_stride != m->L(0, L2H_RMS_FFN).layer_stride)
-        return set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ");
+        return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ") : L2H_OK;
     std::vector<int64_t> off;
     const int64_t total = k_flow_offsets(a, cls_type, grid, off);
     unsigned char *stream = nullptr;

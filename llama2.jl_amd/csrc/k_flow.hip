@@ -22,10 +22,16 @@
 
 #include <string.h>
 
-#define FLOW_D 6            // ring slots per wavefront
+#define FLOW_D 7            // ring slots per wavefront
 #define FLOW_SLOT 1152      // one q4_K piece: 8 headers (128 B) + 8 x 128 B of quants
 #define FLOW_Q6_PIECE 3360  // 16 q6_K super-blocks: ql 2048, qh 1024, scales 256, d 32
 #define FLOW_NW 16
+#ifndef FLOW_FILL
+#define FLOW_FILL 0         // pieces a wavefront may fetch per poll while it waits for activations
+#endif
+#ifndef FLOW_DEFER
+#define FLOW_DEFER 0        // 1: inside a phase's loop fetch only that phase's pieces
+#endif
 #define FLOW_ACT_BYTES 28672
 #define FLOW_MAX_PIECES 1024  // per workgroup and phase
 #define FLOW_MAX_ROWS 512     // per workgroup and phase
@@ -41,9 +47,11 @@ __constant__ __attribute__((aligned(16))) unsigned char c_flow_raw[(sizeof(FlowA
 // object: the compiler then knows that ordinary LDS reads of the other areas never touch memory
 // that an asynchronous fetch is still writing.
 __shared__ __attribute__((aligned(16))) unsigned char s_ring[FLOW_NW * FLOW_D * FLOW_SLOT];
+// activation area: q8_K input of the running phase in the first 16 KiB, then the per-piece partial sums
+// and the row values; attention (between two matvec phases) uses the whole area for itself
 __shared__ uint4 s_act[FLOW_ACT_BYTES / 16];
-__shared__ double s_part[FLOW_MAX_PIECES];
-__shared__ float s_val[FLOW_MAX_ROWS];
+#define s_part ((double *)((unsigned char *)s_act + 16384))
+#define s_val ((float *)((unsigned char *)s_act + 16384 + FLOW_MAX_PIECES * 8))
 __shared__ float s_rope[256];
 __shared__ double s_red[16];
 __shared__ float s_redf[16];
@@ -109,6 +117,7 @@ struct Ring {
     int issued, consumed;       // pieces fetched / used so far
     int drain_mark;             // pieces known to have landed (issued before the last full wait)
     int iss_layer, iss_kind, iss_left;
+    int iss_seq;                // phases the fetch cursor has passed: 4 * layer + kind of the phase it is in
 };
 
 // Headers inside the streams carry the twelve 6-bit scale bytes of a q4_K super-block (reference
@@ -164,6 +173,42 @@ __device__ __forceinline__ void ring_uniform(Ring &r) {
     r.iss_layer = uni(r.iss_layer);
     r.iss_kind = uni(r.iss_kind);
     r.iss_left = uni(r.iss_left);
+    r.iss_seq = uni(r.iss_seq);
+}
+
+// Between the phases the bookkeeping lives in LDS (one row per wavefront), so that the staging
+// function, which is a separate function, can keep fetching while it waits for activations.
+__shared__ int s_rs[FLOW_NW][12];
+__device__ __forceinline__ void ring_store(const Ring &r) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if ((threadIdx.x & 63) == 0) {
+        const unsigned long long p = (unsigned long long)r.gptr;
+        int *d = s_rs[wave];
+        d[0] = (int)(unsigned)p;
+        d[1] = (int)(unsigned)(p >> 32);
+        d[2] = (int)r.lds;
+        d[3] = r.issued;
+        d[4] = r.consumed;
+        d[5] = r.drain_mark;
+        d[6] = r.iss_layer;
+        d[7] = r.iss_kind;
+        d[8] = r.iss_left;
+        d[9] = r.iss_seq;
+    }
+}
+__device__ __forceinline__ void ring_load(Ring &r) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int *d = s_rs[wave];
+    const unsigned lo = (unsigned)uni(d[0]), hi = (unsigned)uni(d[1]);
+    r.gptr = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
+    r.lds = (unsigned)uni(d[2]);
+    r.issued = uni(d[3]);
+    r.consumed = uni(d[4]);
+    r.drain_mark = uni(d[5]);
+    r.iss_layer = uni(d[6]);
+    r.iss_kind = uni(d[7]);
+    r.iss_left = uni(d[8]);
+    r.iss_seq = uni(d[9]);
 }
 
 #define AS1 __attribute__((address_space(1)))
@@ -178,6 +223,7 @@ __device__ __forceinline__ void flow_issue_q4(Ring &r, const FlowArgs &a, unsign
         r.iss_layer = uni(r.iss_layer);
         r.iss_kind = uni(r.iss_kind);
         if (r.iss_layer >= a.n_layers) return;
+        r.iss_seq = uni(r.iss_seq) + 1;
         if (++r.iss_kind == 4) {
             r.iss_kind = 0;
             if (++r.iss_layer >= a.n_layers) return;
@@ -224,8 +270,11 @@ __device__ __forceinline__ void flow_wait_piece(const Ring &r) {
 // epoch `epoch`, or (EMB) the embedding row of `tok`.  Returns false if the wait gave up.
 // Separate functions (not inlined): the kernel stays small enough to keep its state in registers.
 // ------------------------------------------------------------------------------------------
+// While it polls, every wavefront keeps fetching pieces of its weight stream into free ring slots
+// (`fill` pieces per poll at most; 0 = not at all): the fetches are issued behind the poll's loads, so
+// the poll does not wait for them, and they use the time in which the arithmetic has nothing to do.
 template <int PRO, bool EMB>
-__device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, const float *normw, int tok) {
+__device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, const float *normw, int tok, int fill) {
     const FlowArgs &a = c_flow;
     int8_t *s_qs = (int8_t *)s_act;
     int16_t *s_bs = (int16_t *)(s_qs + 14336);
@@ -244,33 +293,57 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
         }
     } else {
         unsigned spins = 0;
+        Ring ring;
+        unsigned char *ring_base = s_ring + wave * (FLOW_D * FLOW_SLOT);
+        if (fill > 0) ring_load(ring);
+        // first pass: every word; later passes: only the words that did not carry the epoch yet, so
+        // that waiting for a slow producer costs next to no traffic
+        u64 w[STAGE_MAX_ROUNDS][4];
+#pragma unroll
+        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+            const int b = wave + r * FLOW_NW;
+            if (b < nb)
+#pragma unroll
+                for (int k = 0; k < 4; k++) w[r][k] = tag_load(src + 256 * b + 4 * lane + k);
+        }
         for (;;) {
+#pragma nounroll
+            for (int f = 0; f < fill; f++) {
+                if (uni(ring.issued) - uni(ring.consumed) >= FLOW_D) break;
+                flow_issue_q4(ring, a, ring_base, blockIdx.x, wave, lane);
+            }
             bool all = true;
-            u64 w[STAGE_MAX_ROUNDS][4];
 #pragma unroll
             for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
                 const int b = wave + r * FLOW_NW;
                 if (b < nb)
 #pragma unroll
-                    for (int k = 0; k < 4; k++) w[r][k] = tag_load(src + 256 * b + 4 * lane + k);
+                    for (int k = 0; k < 4; k++) all = all && tag_is(w[r][k], epoch);
             }
-#pragma unroll
-            for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-                const int b = wave + r * FLOW_NW;
-                if (b < nb)
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        all = all && tag_is(w[r][k], epoch);
-                        xv[r][k] = tag_val(w[r][k]);
-                    }
-            }
-            if (all) break;
+            // the wavefront leaves the loop as a whole: the fetches above need all of its lanes
+            if (__ballot(!all) == 0ull) break;
             if (++spins > a.spin_limit ||
                 ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
                 ok = false;
                 break;
             }
+#pragma unroll
+            for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+                const int b = wave + r * FLOW_NW;
+                if (b < nb)
+#pragma unroll
+                    for (int k = 0; k < 4; k++)
+                        if (!tag_is(w[r][k], epoch)) w[r][k] = tag_load(src + 256 * b + 4 * lane + k);
+            }
         }
+#pragma unroll
+        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+            const int b = wave + r * FLOW_NW;
+            if (b < nb)
+#pragma unroll
+                for (int k = 0; k < 4; k++) xv[r][k] = tag_val(w[r][k]);
+        }
+        if (fill > 0) ring_store(ring);
     }
     if (threadIdx.x == 0) s_flag = 0;
     __syncthreads();
@@ -350,12 +423,23 @@ __device__ __forceinline__ XLds flow_x() {
     return x;
 }
 
-__device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
+// Fetches are issued inside the loop only while pieces of THIS phase are still missing (an issue
+// blocks while the memory pipeline is full, and would hold up the arithmetic); the slots freed
+// beyond that are refilled by the staging function of the following phases while it waits.
+// cur_seq = 4 * layer + kind of the phase, or -1 for the classifier (which has nothing after it).
+__device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg, int cur_seq) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     const XLds x = flow_x();
     flow_drain(r);
+    // whatever the waits before this phase did not fetch of its pieces is requested now
+#pragma nounroll
+    for (int k = 0; k < FLOW_D; k++) {
+        if (uni(r.issued) - uni(r.consumed) >= FLOW_D) break;
+        if (FLOW_DEFER && !(cur_seq < 0 || uni(r.iss_seq) < cur_seq || (uni(r.iss_seq) == cur_seq && uni(r.iss_left) > 0))) break;
+        flow_issue_q4(r, c_flow, ring_base, wg, wave, lane);
+    }
     int part = uni(start % ppr);
     double acc = 0.0;
     for (int k = 0; k < cnt; k++) {
@@ -367,12 +451,17 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
                      : "v"(slot + lane * 16), "v"(slot + (lane >> 3) * 16)
                      : "memory");
         r.consumed++;
-        flow_issue_q4(r, c_flow, ring_base, wg, wave, lane);  // the slot is free again
+        if (!FLOW_DEFER || cur_seq < 0 || uni(r.iss_seq) < cur_seq || (uni(r.iss_seq) == cur_seq && uni(r.iss_left) > 0))
+            flow_issue_q4(r, c_flow, ring_base, wg, wave, lane);  // the slot is free again
+#ifdef FLOW_EXP_NOMATH
+        acc += (double)(ch.w.x ^ ch.hdr.y);
+#else
         {
             int sc_a, sc_b, m_a, m_b, i_sc, i_min;
             flow_decode_pair(ch.hdr, (lane & 7) >> 1, sc_a, sc_b, m_a, m_b);
             acc += q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, part * 64 + lane, x, i_sc, i_min);
         }
+#endif
         // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot
         // in s_part, the run's total goes to its last piece and zero to the others
         const bool last = k == cnt - 1 || uni(part) == ppr - 1;
@@ -770,8 +859,10 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     r.issued = r.consumed = r.drain_mark = 0;
     r.iss_layer = 0;
     r.iss_kind = 0;
+    r.iss_seq = 0;
     r.iss_left = flow_wave_pieces(a.qkv, wg, wave);
     ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
+#pragma nounroll
     for (int k = 0; k < FLOW_D; k++) flow_issue_q4(r, a, ring_base, wg, wave, lane);
 
 #ifdef L2H_TIMELINE
@@ -785,9 +876,15 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         __syncthreads(); \
         FTL();          \
     } while (0)
+#define FTLD()         \
+    do {               \
+        flow_drain(r); \
+        FTL();         \
+    } while (0)
 #else
 #define FTL()
 #define FTLS()
+#define FTLD()
 #endif
     FTL();
 #define LEAVE()        \
@@ -815,57 +912,53 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     for (int l = 0; l < a.n_layers; l++) {
         const unsigned e_x = E0 + 5u * (unsigned)l;  // x entering the layer
         const unsigned e_q = e_x + 1, e_att = e_x + 2, e_wo = e_x + 3, e_w13 = e_x + 4, e_w2 = e_x + 5;
-        // ---- rmsnorm (:244), q, k, v (:247-249), rope (:255-256), cache append (:259-260) ----
-        {
-            const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
-            const bool ok = uni(l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok)
-                                       : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok));
-            if (!ok) LEAVE();
+        // the four matvec phases of the layer share one copy of the streaming loop (the kernel must stay
+        // small enough for the instruction cache):
+        //   0  rmsnorm (:244), q, k, v (:247-249), rope (:255-256), cache append (:259-260)
+        //   1  attention (:263-278) on workgroup h*stride + h%stride, then x += wo * xb (:281-284)
+        //   2  rmsnorm (:287), w1, w3 (:291-292), SwiGLU (:295-299)
+        //   3  x += w2 * hb (:302-305)
+#pragma nounroll
+        for (int kind = 0; kind < 4; kind++) {
+            bool ok;
+            ring_store(r);
+            if (kind == 0) {
+                const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
+                ok = l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok, 0)
+                            : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok, FLOW_FILL);
+            } else if (kind == 1) {
+                const int stride = nwg / a.n_heads;
+                const int h = wg / stride;
+                if (h < a.n_heads && wg % stride == h % stride)
+                    if (!uni(flow_attention(l, h, pos, e_q, e_att))) LEAVE();
+                FTL();
+                ok = flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok, FLOW_FILL);
+            } else if (kind == 2) {
+                ok = flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok, FLOW_FILL);
+            } else {
+                ok = flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok, FLOW_FILL);
+            }
+            ring_load(r);
+            if (!uni(ok)) LEAVE();
             FTL();
-            flow_loop_q4(a.qkv, r, ring_base, wg);
-            FTL();
-            FTLS();
-            flow_finish_qkv(l, wg, pos, e_q);
-            FTL();
-        }
-        // ---- attention (:263-278): head h on workgroup h*stride + h%stride ----
-        {
-            const int stride = nwg / a.n_heads;
-            const int h = wg / stride;
-            if (h < a.n_heads && wg % stride == h % stride)
-                if (!uni(flow_attention(l, h, pos, e_q, e_att))) LEAVE();
-            FTL();
-        }
-        // ---- x += wo * xb (:281-284) ----
-        if (!uni(flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok))) LEAVE();
-        FTL();
-        {
-            const u64 oldw = tid < flow_n_local(a.wo, wg) ? tag_load(a.x_a + wg * a.wo.rpw + tid) : 0;
-            flow_loop_q4(a.wo, r, ring_base, wg);
-            FTL();
-            FTLS();
-            flow_finish_resid(1, wg, oldw, e_x, e_wo);
-        }
-        FTL();
-        // ---- rmsnorm (:287), w1, w3 (:291-292), SwiGLU (:295-299) ----
-        if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok))) LEAVE();
-        FTL();
-        flow_loop_q4(a.w13, r, ring_base, wg);
-        FTL();
-        FTLS();
-        flow_finish_w13(wg, e_w13);
-        FTL();
-        // ---- x += w2 * hb (:302-305) ----
-        if (!uni(flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok))) LEAVE();
-        FTL();
-        {
-            const u64 oldw = tid < flow_n_local(a.w2, wg) ? tag_load(a.x_b + wg * a.w2.rpw + tid) : 0;
-            flow_loop_q4(a.w2, r, ring_base, wg);
+            const FlowGeom g = flow_geom(a, kind);
+            // the row of x this thread adds to after wo / w2: fetched now, used after the loop
+            u64 oldw = 0;
+            if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = tag_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
+            FTLD();
+            flow_loop_q4(g, r, ring_base, wg, 4 * l + kind);
             FTL();
             FTLS();
-            flow_finish_resid(3, wg, oldw, e_wo, e_w2);
+            if (kind == 0)
+                flow_finish_qkv(l, wg, pos, e_q);
+            else if (kind == 1)
+                flow_finish_resid(1, wg, oldw, e_x, e_wo);
+            else if (kind == 2)
+                flow_finish_w13(wg, e_w13);
+            else
+                flow_finish_resid(3, wg, oldw, e_wo, e_w2);
+            FTL();
         }
-        FTL();
     }
 
     // ---- final rmsnorm (:309) + classifier (:312); the ring restarts on the classifier's pieces ----
@@ -880,11 +973,11 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     } else {
         for (int k = 0; k < FLOW_D; k++) flow_issue_q4(r, a, ring_base, wg, wave, lane);
     }
-    if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok))) LEAVE();
+    if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok, 0))) LEAVE();
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
     else
-        flow_loop_q4(a.cls, r, ring_base, wg);
+        flow_loop_q4(a.cls, r, ring_base, wg, -1);
     flow_finish_cls(wg, e_cls);
     flow_drain(r);
     if (wg == 0) flow_pick_token(nwg, e_cls);

@@ -173,8 +173,9 @@ def test_paths_agree_bit_for_bit(pkg):
 
 def test_automatic_path_choice(pkg):
     from llama2_jl_amd import synth
-    assert _model(pkg, *[CASES["q4ks_gqa"][0]], **CASES["q4ks_gqa"][1]).device().path in (1, 2)
-    assert _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device().path == 1  # no persistent kernel for F32
+    assert _model(pkg, *[CASES["q4ks_gqa"][0]], **CASES["q4ks_gqa"][1]).device().path == 1  # dim 512: no whole pieces
+    assert _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device().path == 1  # no single-launch kernel for F32
+    assert _model(pkg, *[FLOW_CASES["all_q4"][0]], **FLOW_CASES["all_q4"][1]).device().path == 3
     with pytest.raises(pkg.L2HError):
         _model(pkg, *[CASES["f32"][0]], **CASES["f32"][1]).device(path=2)
 
