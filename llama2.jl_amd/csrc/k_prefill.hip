@@ -259,13 +259,14 @@ __device__ __forceinline__ void pf_convert(const PfRaw &r, const PfRowPtr &p, in
 // a lane ends up holding one position and groups of 4 consecutive weight rows: neighbours such as a
 // w1/w3 pair sit in one lane.  LDS rows are 64 bf16 = 8 chunks of 16 bytes, chunk c of row r kept at
 // c ^ (r & 7) so that the 8 lanes of a 128-byte access phase hit distinct banks.
-template <int TYPE, int EPI>
+template <int TYPE, int EPI, int JT>
 __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
+    constexpr int MT = 64 * JT;  // positions per workgroup: 2 wavefront columns x JT tiles of 32
     __shared__ uint4 s_w[128 * 8];
-    __shared__ uint4 s_x[128 * 8];
+    __shared__ uint4 s_x[MT * 8];
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6, wn = wave & 1, wm = wave >> 1;
     const int64_t n0 = (int64_t)blockIdx.y * 128;
-    const int m0 = blockIdx.x * 128;
+    const int m0 = blockIdx.x * MT;
     const int64_t K = a.K;
 
     // the weight row this thread dequantizes: row t/2 of the tile, elements 32*(t&1).. of each K step
@@ -286,31 +287,32 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #undef PICK
         rp.valid = lr.valid;
     }
-    // activations: 4 chunks of 16 bytes per thread and K step: position (t>>3) + 32*i, chunk t&7
+    // activations: 2 JT chunks of 16 bytes per thread and K step: position (t>>3) + 32*i, chunk t&7
+    constexpr int XL = 2 * JT;
     const int xc = t & 7;
-    const uint16_t *xrow[4];
-    bool xvalid[4];
+    const uint16_t *xrow[XL];
+    bool xvalid[XL];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < XL; i++) {
         const int m = m0 + (t >> 3) + 32 * i;
         xvalid[i] = m < a.M;
         xrow[i] = a.act + (int64_t)(xvalid[i] ? m : 0) * K + 8 * xc;
     }
 
-    f32x16 acc[2][2];
+    f32x16 acc[2][JT];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < JT; j++)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     PfRaw raw;
-    uint4 xreg[4];
+    uint4 xreg[XL];
     auto gload = [&](int64_t k0) {
         if (k0 + 32 * whh < K) pf_load_raw<TYPE>(raw, rp, lr.row, k0 + 32 * whh, K);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < XL; i++) {
             xreg[i] = make_uint4(0, 0, 0, 0);
             if (xvalid[i] && k0 + 8 * xc < K) xreg[i] = *(const uint4 *)(xrow[i] + k0);
         }
@@ -326,7 +328,7 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #pragma unroll
             for (int c = 0; c < 4; c++) s_w[wr * 8 + ((4 * whh + c) ^ (wr & 7))] = wv[c];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < XL; i++) {
                 const int r = (t >> 3) + 32 * i;
                 s_x[r * 8 + (xc ^ (r & 7))] = xreg[i];
             }
@@ -336,30 +338,30 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #pragma unroll
         for (int kk = 0; kk < 4; kk++) {
             const int c = 2 * kk + (lane >> 5);
-            bf16x8 A[2], B[2];
+            bf16x8 A[2], B[JT];
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const int ra = 64 * wn + 32 * i + (lane & 31);
                 A[i] = as_bf16x8(s_w[ra * 8 + (c ^ (ra & 7))]);
             }
 #pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const int rb = 64 * wm + 32 * j + (lane & 31);
+            for (int j = 0; j < JT; j++) {
+                const int rb = 32 * JT * wm + 32 * j + (lane & 31);
                 B[j] = as_bf16x8(s_x[rb * 8 + (c ^ (rb & 7))]);
             }
 #pragma unroll
             for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[i], B[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < JT; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A[i], B[j], acc[i][j], 0, 0, 0);
         }
         __syncthreads();
     }
 
-    // lane: position m0 + 64 wm + 32 j + lane%32; register r of tile i: logical weight row
+    // lane: position m0 + 32 JT wm + 32 j + lane%32; register r of tile i: logical weight row
     // n0 + 64 wn + 32 i + 8 (r/4) + 4 (lane/32) + r%4
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        const int m = m0 + 64 * wm + 32 * j + (lane & 31);
+    for (int j = 0; j < JT; j++) {
+        const int m = m0 + 32 * JT * wm + 32 * j + (lane & 31);
         if (m >= a.M) continue;
 #pragma unroll
         for (int i = 0; i < 2; i++) {
@@ -542,12 +544,14 @@ hipError_t k_pf_rope_scatter(hipStream_t s, const float *raw, const float *cs, u
     return hipGetLastError();
 }
 
-template <int TYPE>
-static hipError_t pf_gemm_type(hipStream_t s, const PfGemmArgs &a, int epi, dim3 grid) {
+// JT tiles of 32 positions per wavefront column: 64 JT positions per workgroup
+template <int TYPE, int JT>
+static hipError_t pf_gemm_type(hipStream_t s, const PfGemmArgs &a, int epi, int64_t rows) {
+    const dim3 grid((unsigned)((a.M + 64 * JT - 1) / (64 * JT)), (unsigned)((rows + 127) / 128));
     switch (epi) {
-    case PF_STORE: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_STORE>), grid, dim3(256), 0, s, a); break;
-    case PF_RESID: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_RESID>), grid, dim3(256), 0, s, a); break;
-    case PF_SWIGLU: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_SWIGLU>), grid, dim3(256), 0, s, a); break;
+    case PF_STORE: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_STORE, JT>), grid, dim3(256), 0, s, a); break;
+    case PF_RESID: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_RESID, JT>), grid, dim3(256), 0, s, a); break;
+    case PF_SWIGLU: hipLaunchKernelGGL((pf_gemm_kernel<TYPE, PF_SWIGLU, JT>), grid, dim3(256), 0, s, a); break;
     default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -576,12 +580,12 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
     a.out_col0 = out_col0;
     a.out_bf = out_bf;
     a.ldb = ldb;
-    const dim3 grid((unsigned)((M + 127) / 128), (unsigned)((rows + 127) / 128));
+    // (a 256-position tile, JT = 4, was measured slower: its 272 registers leave one wavefront per SIMD)
     switch (w[0].type) {
-    case L2H_TYPE_Q4_K: return pf_gemm_type<L2H_TYPE_Q4_K>(s, a, epi, grid);
-    case L2H_TYPE_Q5_K: return pf_gemm_type<L2H_TYPE_Q5_K>(s, a, epi, grid);
-    case L2H_TYPE_Q6_K: return pf_gemm_type<L2H_TYPE_Q6_K>(s, a, epi, grid);
-    case L2H_TYPE_F32: return pf_gemm_type<L2H_TYPE_F32>(s, a, epi, grid);
+    case L2H_TYPE_Q4_K: return pf_gemm_type<L2H_TYPE_Q4_K, 2>(s, a, epi, rows);
+    case L2H_TYPE_Q5_K: return pf_gemm_type<L2H_TYPE_Q5_K, 2>(s, a, epi, rows);
+    case L2H_TYPE_Q6_K: return pf_gemm_type<L2H_TYPE_Q6_K, 2>(s, a, epi, rows);
+    case L2H_TYPE_F32: return pf_gemm_type<L2H_TYPE_F32, 2>(s, a, epi, rows);
     }
     return hipErrorInvalidValue;
 }
