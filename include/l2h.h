@@ -131,6 +131,11 @@ int l2h_generate_greedy_timed(l2h_model *m, const int32_t *prompt, int n_prompt,
  * already be in the cache.  Decoding continues with l2h_generate_greedy(&next, 1, pos0+n, ...).
  * Needs head size 32/64/96/128, dim and hidden_dim multiples of 8, w1 and w3 of one type. */
 int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0, float *last_logits, int32_t *next_token);
+/* The temperature branch of sample() (src/inference.jl:363-367) on the logits the last step left on
+ * the device: logits ./= temperature, softmax!, then wsample's walk with the caller's uniform number
+ * u in [0, 1) in place of the global RNG: token = first index whose cumulative probability reaches
+ * u * sum(p).  probs (vocab floats, may be NULL) receives the probabilities.  temperature > 0. */
+int l2h_sample(l2h_model *m, float temperature, float u, int32_t *token, float *probs);
 /* Copies an activation of the last forward call: which = 0 x, 1 xb, 2 q (rotated), 5 hb,
  * 6 logits (RunState fields, src/inference.jl:72-86; k and v go straight into the cache). */
 int l2h_state_read(l2h_model *m, int which, float *host, int64_t n);

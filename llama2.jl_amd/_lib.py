@@ -55,6 +55,7 @@ SIGNATURES = {
     "l2h_generate_greedy": (_I, [_P, _P, _I, _I, _I, _P, _P]),
     "l2h_generate_greedy_timed": (_I, [_P, _P, _I, _I, _I, _P, _PF]),
     "l2h_prefill": (_I, [_P, _P, _I, _I, _P, _PI32]),
+    "l2h_sample": (_I, [_P, C.c_float, C.c_float, _PI32, _P]),
     "l2h_state_read": (_I, [_P, _I, _P, _I64]),
     "l2h_quantize_q8k": (_I, [_P, _P, _I64, _P]),
     "l2h_dequantize": (_I, [_P, _I, _P, _I64, _P]),

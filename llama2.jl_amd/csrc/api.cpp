@@ -231,6 +231,8 @@ struct l2h_model {
 #ifdef L2H_TIMELINE
     long long *timeline = nullptr, *timeline2 = nullptr;
 #endif
+    float *sample_p = nullptr;  // probabilities of the last l2h_sample call
+    int32_t *sample_out = nullptr;
     // streaming decode kernel
     bool flow = false;
     FlowArgs flow_args{};
@@ -289,6 +291,8 @@ static void model_free_state(l2h_model *m) {
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
     m->pf_cap = 0;
+    m->sample_p = nullptr;
+    m->sample_out = nullptr;
     m->finalized = false;
 }
 
@@ -1097,6 +1101,26 @@ extern "C" int l2h_forward(l2h_model *m, int token, int pos, float *logits, int3
     int rc = generate_impl(m, &tok, 1, pos, 1, &next, logits, nullptr);
     if (rc == L2H_OK && argmax) *argmax = next;
     return rc;
+}
+
+extern "C" int l2h_sample(l2h_model *m, float temperature, float u, int32_t *token, float *probs) {
+    if (!m || !token) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "l2h_sample: NULL argument");
+    l2h_ctx *ctx = m->ctx;
+    if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
+    if (!(temperature > 0.0f) || !(u >= 0.0f && u < 1.0f))
+        return set_err(ctx, L2H_EINVAL, "need temperature > 0 and 0 <= u < 1 (got %g, %g)", (double)temperature, (double)u);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    if (!m->sample_p) {
+        int rc;
+        if ((rc = dalloc(m, &m->sample_p, m->c.vocab_size, false))) return rc;
+        if ((rc = dalloc(m, &m->sample_out, 1, true))) return rc;
+    }
+    HIPCHK(ctx, k_sample(ctx->stream, m->logits, m->c.vocab_size, temperature, u, m->sample_p, m->sample_out));
+    HIPCHK(ctx, hipMemcpyAsync(token, m->sample_out, 4, hipMemcpyDeviceToHost, ctx->stream));
+    if (probs)
+        HIPCHK(ctx, hipMemcpyAsync(probs, m->sample_p, (size_t)m->c.vocab_size * 4, hipMemcpyDeviceToHost, ctx->stream));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    return L2H_OK;
 }
 
 extern "C" int l2h_state_read(l2h_model *m, int which, float *host, int64_t n) {

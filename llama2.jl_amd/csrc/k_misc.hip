@@ -316,3 +316,67 @@ hipError_t k_f32_to_f64(hipStream_t s, const float *x, double *y, int64_t n) {
     hipLaunchKernelGGL(f32_to_f64_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, x, y, n);
     return hipGetLastError();
 }
+
+// ------------------------------------------------------------------------------------------
+// temperature sampling (reference src/inference.jl:363-367): logits ./= T; softmax!; wsample.
+// wsample's walk is reproduced with a host-supplied uniform number u in [0, 1): the pick is the first
+// index whose cumulative weight reaches u * sum(weights).  exp in fp64 rounded to fp32 and the sums
+// in fp64 (as everywhere in this library); one workgroup, thread t owns a contiguous slice.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void sample_kernel(const float *logits, int n, float temperature, float u,
+                                                      float *p, int32_t *out) {
+    __shared__ double redd[16];
+    __shared__ float redf[16];
+    __shared__ double s_cum[1025];
+    const int tid = threadIdx.x;
+    const int per = (n + 1023) / 1024, lo = min(n, tid * per), hi = min(n, lo + per);
+    float mx = -INFINITY;
+    for (int i = lo; i < hi; i++) {
+        const float v = logits[i] / temperature;
+        p[i] = v;
+        mx = fmaxf(mx, v);
+    }
+    mx = block_max_f32(mx, redf);
+    double sum = 0.0;
+    for (int i = lo; i < hi; i++) {
+        const float e = (float)exp((double)(p[i] - mx));
+        p[i] = e;
+        sum += (double)e;
+    }
+    const float sf = (float)block_sum_f64(sum, redd);
+    double mine = 0.0;
+    for (int i = lo; i < hi; i++) {
+        const float pr = p[i] / sf;
+        p[i] = pr;
+        mine += (double)pr;
+    }
+    s_cum[tid + 1] = mine;
+    __syncthreads();
+    if (tid == 0) {
+        s_cum[0] = 0.0;
+        for (int k = 1; k <= 1024; k++) s_cum[k] += s_cum[k - 1];
+    }
+    __syncthreads();
+    const double target = (double)u * s_cum[1024];
+    // the slice in which the cumulative weight first reaches the target (the last non-empty one if
+    // rounding leaves the target just above the total)
+    const bool here = lo < hi && s_cum[tid] < target && (target <= s_cum[tid + 1] || hi == n);
+    const bool first_zero = tid == 0 && target <= 0.0;
+    if (here || first_zero) {
+        double cw = s_cum[tid];
+        int pick = hi - 1;
+        for (int i = lo; i < hi; i++) {
+            cw += (double)p[i];
+            if (cw >= target) {
+                pick = i;
+                break;
+            }
+        }
+        *out = pick;
+    }
+}
+
+hipError_t k_sample(hipStream_t s, const float *logits, int n, float temperature, float u, float *p, int32_t *out) {
+    hipLaunchKernelGGL(sample_kernel, dim3(1), dim3(1024), 0, s, logits, n, temperature, u, p, out);
+    return hipGetLastError();
+}

@@ -142,6 +142,14 @@ class DeviceModel:
                                               C.byref(nxt)))
         return logits, nxt.value
 
+    def sample_token(self, temperature, u, want_probs=False):
+        """Temperature sampling from the logits of the last step (src/inference.jl:363-367) with the
+        uniform number u in [0, 1) standing in for wsample's draw."""
+        probs = np.empty(self.config.vocab_size, np.float32) if want_probs else None
+        tok = C.c_int32()
+        self.ctx.check(_lib.lib().l2h_sample(self.handle, float(temperature), float(u), C.byref(tok), _lib.ptr(probs)))
+        return (tok.value, probs) if want_probs else tok.value
+
     def kv_write(self, layer, pos0, k, v):
         k = np.ascontiguousarray(k, dtype=np.float32)
         v = np.ascontiguousarray(v, dtype=np.float32)
@@ -251,17 +259,15 @@ def sample(model, prompt="", temperature=0.9, stop_on_special_token=True, max_se
             if stop:
                 break
             continue
-        logits, am = state.dev.forward(token, pos)  # :351
+        logits, am = state.dev.forward(token, pos, want_logits=False)  # :351
         generated_seq_len += 1
         if pos + 1 < len(prompt_tokens):
             nxt = prompt_tokens[pos + 1]  # :354-355
         elif temperature == 0.0:
             nxt = am  # :360
         else:
-            logits = logits / np.float32(temperature)  # :363
-            e = np.exp(logits - logits.max())  # softmax!, :365
-            p = e / e.sum()
-            nxt = int(rng.choice(config.vocab_size, p=p.astype(np.float64) / p.astype(np.float64).sum()))  # :367
+            # logits ./= temperature; softmax!; wsample (:363-367) on the device, the draw from this rng
+            nxt = state.dev.sample_token(temperature, min(float(rng.random()), 0.99999994))
         pos += 1
         if stop_on_special_token and nxt in special:
             break

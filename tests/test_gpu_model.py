@@ -220,3 +220,34 @@ def test_generate_argument_checks(pkg):
     with pytest.raises(pkg.L2HError):  # token outside the vocabulary
         dev.generate_greedy([lm.config.vocab_size], 1)
     dev.generate_greedy([1, 2, 3], lm.config.seq_len - 2)  # exactly fills the cache
+
+
+def test_temperature_sampling_on_device(pkg, rng):
+    """l2h_sample: logits ./= T, softmax!, then wsample's cumulative walk (src/inference.jl:363-367)
+    with the caller's uniform number.  Checked against the same procedure in numpy (probabilities to
+    1e-6 relative, the picked index exactly except where u * sum falls within rounding of a
+    cumulative boundary), which makes the distribution of the picks the softmax distribution."""
+    plan, kw = CASES["f32"]
+    lm = _model(pkg, plan, **kw)
+    dev = lm.device()
+    dev.reset()
+    logits, _ = dev.forward(3, 0)
+    for T in (0.9, 0.25, 4.0):
+        xs = (logits / np.float32(T)).astype(np.float32)
+        e = np.exp((xs - xs.max()).astype(np.float64)).astype(np.float32)
+        sf = np.float32(e.astype(np.float64).sum())
+        p = (e / sf).astype(np.float32)
+        cum = np.cumsum(p.astype(np.float64))
+        tok, probs = dev.sample_token(T, 0.5, want_probs=True)
+        assert np.allclose(probs, p, rtol=1e-6, atol=0)
+        us = np.concatenate([[0.0, 0.99999994], rng.random(300)]).astype(np.float32)
+        for u in us:
+            tok = dev.sample_token(T, float(u))
+            target = float(u) * cum[-1]
+            want = min(int(np.searchsorted(cum, target, side="left")), len(p) - 1)
+            if tok != want:  # only acceptable at a boundary
+                assert abs(cum[min(tok, want)] - target) <= 1e-9, (T, u, tok, want)
+    with pytest.raises(pkg.L2HError):
+        dev.sample_token(0.0, 0.5)
+    with pytest.raises(pkg.L2HError):
+        dev.sample_token(1.0, 1.0)
