@@ -116,6 +116,26 @@ end
     sample(m::DeviceModel, model::LanguageModel, prompt=""; temperature=0.9f0, stop_on_special_token=true,
            max_seq_len=typemax(Int), bos_token=true)
 
+# Whole prompt in one pass on the matrix cores (no counterpart in Llama2.jl, which feeds the prompt token
+# by token): fills the cache for positions pos .. pos+length(prompt)-1 and returns the next token (1-based).
+function prefill!(m::DeviceModel, prompt::Vector{Int}; pos::Int = 1)
+    p0 = Int32.(prompt .- 1)
+    next = Ref{Int32}(0)
+    check(m.ctx.handle, ccall((:l2h_prefill, lib), Cint,
+                              (Ptr{Cvoid}, Ptr{Int32}, Cint, Cint, Ptr{Float32}, Ref{Int32}),
+                              m.handle, p0, length(p0), pos - 1, C_NULL, next))
+    return Int(next[]) + 1
+end
+
+# Temperature branch of sample (src/inference.jl:363-367) on the logits the last step left on the device;
+# u stands in for wsample's draw from the global RNG.
+function sample_token(m::DeviceModel, temperature::Float32; u::Float32 = min(rand(Float32), prevfloat(1f0)))
+    tok = Ref{Int32}(0)
+    check(m.ctx.handle, ccall((:l2h_sample, lib), Cint, (Ptr{Cvoid}, Cfloat, Cfloat, Ref{Int32}, Ptr{Float32}),
+                              m.handle, temperature, u, tok, C_NULL))
+    return Int(tok[]) + 1
+end
+
 Same behaviour and output as `Llama2.sample` (src/inference.jl:317-395).
 """
 function sample(m::DeviceModel, model::LanguageModel, prompt::String = ""; temperature::Float32 = 0.9f0,
