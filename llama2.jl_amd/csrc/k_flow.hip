@@ -26,12 +26,6 @@
 #define FLOW_SLOT 1152      // one q4_K piece: 8 headers (128 B) + 8 x 128 B of quants
 #define FLOW_Q6_PIECE 3360  // 16 q6_K super-blocks: ql 2048, qh 1024, scales 256, d 32
 #define FLOW_NW 16
-#ifndef FLOW_FILL
-#define FLOW_FILL 0         // pieces a wavefront may fetch per poll while it waits for activations
-#endif
-#ifndef FLOW_DEFER
-#define FLOW_DEFER 0        // 1: inside a phase's loop fetch only that phase's pieces
-#endif
 #define FLOW_ACT_BYTES 28672
 #define FLOW_MAX_PIECES 1024  // per workgroup and phase
 #define FLOW_MAX_ROWS 512     // per workgroup and phase
@@ -56,6 +50,7 @@ __shared__ float s_rope[256];
 __shared__ double s_red[16];
 __shared__ float s_redf[16];
 __shared__ int s_flag;
+__shared__ __attribute__((aligned(16))) unsigned char s_sink[256];  // target of fetches made only to warm the L2
 
 __device__ __forceinline__ void tag_store(u64 *p, float v, unsigned epoch) {
     __hip_atomic_store(p, ((u64)epoch << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -109,15 +104,16 @@ __host__ __device__ inline void flow_row_src(int kind, int L, int dim, int kv_di
 // ------------------------------------------------------------------------------------------
 // the ring of one wavefront
 // ------------------------------------------------------------------------------------------
-struct Ring;
-__device__ __forceinline__ void ring_uniform(Ring &r);
+// A wavefront's stream is one contiguous run of pieces in the order it uses them, so the fetch side
+// needs no notion of phases: it keeps the ring full (issued - consumed == FLOW_D) until the stream
+// ends, and the slot a piece is fetched into is always the slot that was just emptied.
 struct Ring {
     const unsigned char *gptr;  // next byte of the stream to fetch
     unsigned lds;               // LDS byte address of slot 0
+    int off;                    // byte offset in the ring of the slot to use (and then refill) next
     int issued, consumed;       // pieces fetched / used so far
     int drain_mark;             // pieces known to have landed (issued before the last full wait)
-    int iss_layer, iss_kind, iss_left;
-    int iss_seq;                // phases the fetch cursor has passed: 4 * layer + kind of the phase it is in
+    int left;                   // pieces of the stream not fetched yet
 };
 
 // Headers inside the streams carry the twelve 6-bit scale bytes of a q4_K super-block (reference
@@ -167,76 +163,38 @@ __device__ __forceinline__ void ring_uniform(Ring &r) {
     const unsigned lo = (unsigned)uni((int)(unsigned)p), hi = (unsigned)uni((int)(unsigned)(p >> 32));
     r.gptr = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
     r.lds = (unsigned)uni((int)r.lds);
+    r.off = uni(r.off);
     r.issued = uni(r.issued);
     r.consumed = uni(r.consumed);
     r.drain_mark = uni(r.drain_mark);
-    r.iss_layer = uni(r.iss_layer);
-    r.iss_kind = uni(r.iss_kind);
-    r.iss_left = uni(r.iss_left);
-    r.iss_seq = uni(r.iss_seq);
-}
-
-// Between the phases the bookkeeping lives in LDS (one row per wavefront), so that the staging
-// function, which is a separate function, can keep fetching while it waits for activations.
-__shared__ int s_rs[FLOW_NW][12];
-__device__ __forceinline__ void ring_store(const Ring &r) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if ((threadIdx.x & 63) == 0) {
-        const unsigned long long p = (unsigned long long)r.gptr;
-        int *d = s_rs[wave];
-        d[0] = (int)(unsigned)p;
-        d[1] = (int)(unsigned)(p >> 32);
-        d[2] = (int)r.lds;
-        d[3] = r.issued;
-        d[4] = r.consumed;
-        d[5] = r.drain_mark;
-        d[6] = r.iss_layer;
-        d[7] = r.iss_kind;
-        d[8] = r.iss_left;
-        d[9] = r.iss_seq;
-    }
-}
-__device__ __forceinline__ void ring_load(Ring &r) {
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int *d = s_rs[wave];
-    const unsigned lo = (unsigned)uni(d[0]), hi = (unsigned)uni(d[1]);
-    r.gptr = (const unsigned char *)(((unsigned long long)hi << 32) | lo);
-    r.lds = (unsigned)uni(d[2]);
-    r.issued = uni(d[3]);
-    r.consumed = uni(d[4]);
-    r.drain_mark = uni(d[5]);
-    r.iss_layer = uni(d[6]);
-    r.iss_kind = uni(d[7]);
-    r.iss_left = uni(d[8]);
-    r.iss_seq = uni(d[9]);
+    r.left = uni(r.left);
 }
 
 #define AS1 __attribute__((address_space(1)))
 #define AS3 __attribute__((address_space(3)))
 
-// fetch the next q4_K piece of this wavefront's stream, if the layer phases have one left
-__device__ __forceinline__ void flow_issue_q4(Ring &r, const FlowArgs &a, unsigned char *ring_base, int wg, int wave,
-                                              int lane) {
-    // (the bookkeeping is the same on every lane; saying so where it steers a branch keeps the
-    // branches on the scalar unit)
-    while (uni(r.iss_left) == 0) {
-        r.iss_layer = uni(r.iss_layer);
-        r.iss_kind = uni(r.iss_kind);
-        if (r.iss_layer >= a.n_layers) return;
-        r.iss_seq = uni(r.iss_seq) + 1;
-        if (++r.iss_kind == 4) {
-            r.iss_kind = 0;
-            if (++r.iss_layer >= a.n_layers) return;
-        }
-        r.iss_left = uni(flow_wave_pieces(flow_geom(a, r.iss_kind), wg, wave));
+// fetch the next q4_K piece of the stream into the ring slot at byte offset `off`
+__device__ __forceinline__ void flow_fetch_q4(const unsigned char *g, unsigned char *ring_base, int off, int lane) {
+    // the instruction's immediate offset applies to both the global and the LDS address
+    unsigned char *slot = ring_base + off;
+    const unsigned char *gl = g + lane * 16;
+    if (lane < 8) __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 0, 2);
+    __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 128, 2);
+}
+
+// fill the ring from empty or part-empty: pieces go to the slots after the ones in use
+__device__ __forceinline__ void flow_top_up_q4(Ring &r, unsigned char *ring_base, int lane) {
+#pragma nounroll
+    for (int k = 0; k < FLOW_D; k++) {
+        const int held = uni(r.issued) - uni(r.consumed);
+        if (held >= FLOW_D || uni(r.left) <= 0) break;
+        int o = uni(r.off) + held * FLOW_SLOT;
+        if (o >= FLOW_D * FLOW_SLOT) o -= FLOW_D * FLOW_SLOT;
+        flow_fetch_q4(r.gptr, ring_base, o, lane);
+        r.gptr += FLOW_SLOT;
+        r.issued++;
+        r.left--;
     }
-    unsigned char *slot = ring_base + (uni(r.issued) % FLOW_D) * FLOW_SLOT;
-    const unsigned char *g = r.gptr;
-    if (lane < 8) __builtin_amdgcn_global_load_lds((const AS1 void *)(g + lane * 16), (AS3 void *)slot, 16, 0, 2);
-    __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 128 + lane * 16), (AS3 void *)(slot + 128), 16, 0, 2);
-    r.gptr += FLOW_SLOT;
-    r.issued++;
-    r.iss_left--;
 }
 
 // everything this wavefront has fetched so far has landed
@@ -245,36 +203,13 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
     r.drain_mark = r.issued;
 }
 
-// piece number r.consumed has landed (fetches complete in order; OPS fetch instructions per piece)
-template <int OPS>
-__device__ __forceinline__ void flow_wait_piece(const Ring &r) {
-    if (uni(r.consumed) < uni(r.drain_mark)) return;
-    const int younger = uni(r.issued - 1 - r.consumed);
-    constexpr int DEPTH = OPS == 2 ? FLOW_D : 2;
-    if (younger >= DEPTH - 1) {  // the steady state: a full ring
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * (DEPTH - 1)) : "memory");
-        return;
-    }
-    switch (younger) {
-    case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-    case 1: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * 1) : "memory"); break;
-    case 2: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * 2 > 63 ? 63 : OPS * 2) : "memory"); break;
-    case 3: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * 3 > 63 ? 63 : OPS * 3) : "memory"); break;
-    case 4: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * 4 > 63 ? 63 : OPS * 4) : "memory"); break;
-    default: asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * 5 > 63 ? 63 : OPS * 5) : "memory"); break;
-    }
-}
-
 // ------------------------------------------------------------------------------------------
 // staging: the input vector of a phase -> q8_K in this workgroup's LDS.  Source: tagged words of
 // epoch `epoch`, or (EMB) the embedding row of `tok`.  Returns false if the wait gave up.
 // Separate functions (not inlined): the kernel stays small enough to keep its state in registers.
 // ------------------------------------------------------------------------------------------
-// While it polls, every wavefront keeps fetching pieces of its weight stream into free ring slots
-// (`fill` pieces per poll at most; 0 = not at all): the fetches are issued behind the poll's loads, so
-// the poll does not wait for them, and they use the time in which the arithmetic has nothing to do.
 template <int PRO, bool EMB>
-__device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, const float *normw, int tok, int fill) {
+__device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, const float *normw, int tok) {
     const FlowArgs &a = c_flow;
     int8_t *s_qs = (int8_t *)s_act;
     int16_t *s_bs = (int16_t *)(s_qs + 14336);
@@ -293,9 +228,6 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
         }
     } else {
         unsigned spins = 0;
-        Ring ring;
-        unsigned char *ring_base = s_ring + wave * (FLOW_D * FLOW_SLOT);
-        if (fill > 0) ring_load(ring);
         // first pass: every word; later passes: only the words that did not carry the epoch yet, so
         // that waiting for a slow producer costs next to no traffic
         u64 w[STAGE_MAX_ROUNDS][4];
@@ -307,11 +239,6 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
                 for (int k = 0; k < 4; k++) w[r][k] = tag_load(src + 256 * b + 4 * lane + k);
         }
         for (;;) {
-#pragma nounroll
-            for (int f = 0; f < fill; f++) {
-                if (uni(ring.issued) - uni(ring.consumed) >= FLOW_D) break;
-                flow_issue_q4(ring, a, ring_base, blockIdx.x, wave, lane);
-            }
             bool all = true;
 #pragma unroll
             for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
@@ -320,7 +247,6 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
 #pragma unroll
                     for (int k = 0; k < 4; k++) all = all && tag_is(w[r][k], epoch);
             }
-            // the wavefront leaves the loop as a whole: the fetches above need all of its lanes
             if (__ballot(!all) == 0ull) break;
             if (++spins > a.spin_limit ||
                 ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
@@ -343,7 +269,6 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
 #pragma unroll
                 for (int k = 0; k < 4; k++) xv[r][k] = tag_val(w[r][k]);
         }
-        if (fill > 0) ring_store(ring);
     }
     if (threadIdx.x == 0) s_flag = 0;
     __syncthreads();
@@ -423,76 +348,137 @@ __device__ __forceinline__ XLds flow_x() {
     return x;
 }
 
-// Fetches are issued inside the loop only while pieces of THIS phase are still missing (an issue
-// blocks while the memory pipeline is full, and would hold up the arithmetic); the slots freed
-// beyond that are refilled by the staging function of the following phases while it waits.
-// cur_seq = 4 * layer + kind of the phase, or -1 for the classifier (which has nothing after it).
-__device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg, int cur_seq) {
+// The ring is kept full: as soon as a piece has been read into registers, the next piece of the stream
+// is fetched into its slot, whichever phase that piece belongs to.  The loop's bookkeeping is a handful
+// of scalars (the scalar unit is shared by the 16 wavefronts of the workgroup, so every scalar
+// instruction per piece counts 16-fold):
+//   held   pieces fetched and not yet used          ready   of those, known to have landed
+//   off    byte offset of the slot to use next      left    pieces of the stream not fetched yet
+template <int PIECE_BYTES, int DEPTH, int OPS>
+struct RingLoop {
+    const unsigned char *gp;
+    int off, held, ready, left;
+    __device__ __forceinline__ void begin(const Ring &r) {
+        gp = r.gptr;
+        off = uni(r.off);
+        held = uni(r.issued) - uni(r.consumed);
+        ready = uni(r.drain_mark) - uni(r.consumed);
+        left = uni(r.left);
+    }
+    // the piece in slot `off` has landed when this returns
+    __device__ __forceinline__ void wait() {
+        if (ready == 0) {
+            if (held == DEPTH) {  // the fetches return in order: all but the DEPTH-1 youngest are back
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(OPS * (DEPTH - 1)) : "memory");
+                ready = 1;
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                ready = held;
+            }
+        }
+    }
+    __device__ __forceinline__ void used() {
+        ready--;
+        held--;
+    }
+    __device__ __forceinline__ void fetched() {
+        gp += PIECE_BYTES;
+        left--;
+        held++;
+    }
+    __device__ __forceinline__ void next_slot() {
+        off += PIECE_BYTES;
+        if (off == DEPTH * PIECE_BYTES) off = 0;
+    }
+    __device__ __forceinline__ void end(Ring &r, int n_used, int n_fetched) {
+        r.gptr = gp;
+        r.off = off;
+        r.consumed += n_used;
+        r.issued += n_fetched;
+        r.drain_mark = r.consumed + ready;
+        r.left = left;
+    }
+};
+
+__device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     const XLds x = flow_x();
-    flow_drain(r);
-    // whatever the waits before this phase did not fetch of its pieces is requested now
-#pragma nounroll
-    for (int k = 0; k < FLOW_D; k++) {
-        if (uni(r.issued) - uni(r.consumed) >= FLOW_D) break;
-        if (FLOW_DEFER && !(cur_seq < 0 || uni(r.iss_seq) < cur_seq || (uni(r.iss_seq) == cur_seq && uni(r.iss_left) > 0))) break;
-        flow_issue_q4(r, c_flow, ring_base, wg, wave, lane);
-    }
+    RingLoop<FLOW_SLOT, FLOW_D, 2> q;
+    q.begin(r);
+    const int left0 = q.left;
+    const unsigned rd_w = r.lds + lane * 16, rd_h = r.lds + (lane >> 3) * 16;
+    const int pair = (lane & 7) >> 1;
     int part = uni(start % ppr);
+    int xi = part * 64 + lane;  // index of this lane's 32 activations
+    double *out = s_part + start;
     double acc = 0.0;
-    for (int k = 0; k < cnt; k++) {
-        flow_wait_piece<2>(r);
-        const unsigned slot = r.lds + (unsigned)(uni(r.consumed) % FLOW_D) * FLOW_SLOT;
+#pragma nounroll
+    for (int k = cnt; k > 0; k--) {
+        q.wait();
         Chunk<L2H_TYPE_Q4_K> ch;
         asm volatile("ds_read_b128 %0, %2 offset:128\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
                      : "=&v"(ch.w), "=&v"(ch.hdr)
-                     : "v"(slot + lane * 16), "v"(slot + (lane >> 3) * 16)
+                     : "v"(rd_w + q.off), "v"(rd_h + q.off)
                      : "memory");
-        r.consumed++;
-        if (!FLOW_DEFER || cur_seq < 0 || uni(r.iss_seq) < cur_seq || (uni(r.iss_seq) == cur_seq && uni(r.iss_left) > 0))
-            flow_issue_q4(r, c_flow, ring_base, wg, wave, lane);  // the slot is free again
+        q.used();
+        if (q.left > 0) {  // the slot is free again
+            flow_fetch_q4(q.gp, ring_base, q.off, lane);
+            q.fetched();
+        }
+        q.next_slot();
 #ifdef FLOW_EXP_NOMATH
         acc += (double)(ch.w.x ^ ch.hdr.y);
 #else
         {
             int sc_a, sc_b, m_a, m_b, i_sc, i_min;
-            flow_decode_pair(ch.hdr, (lane & 7) >> 1, sc_a, sc_b, m_a, m_b);
-            acc += q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, part * 64 + lane, x, i_sc, i_min);
+            flow_decode_pair(ch.hdr, pair, sc_a, sc_b, m_a, m_b);
+            acc += q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, xi, x, i_sc, i_min);
         }
 #endif
         // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot
         // in s_part, the run's total goes to its last piece and zero to the others
-        const bool last = k == cnt - 1 || uni(part) == ppr - 1;
-        if (last) {
-            const double v = wave_sum_f64_dpp(acc);
-            if (lane == 0) s_part[start + k] = v;
+        // (every lane stores the same word: no lane-dependent branch in the loop)
+        part++;
+        xi += 64;
+        double v = 0.0;
+        if (k == 1 || part == ppr) {
+            v = wave_sum_f64_dpp(acc);
             acc = 0.0;
-        } else if (lane == 0) {
-            s_part[start + k] = 0.0;
+            xi = lane;
+            part = 0;
         }
-        part = part == ppr - 1 ? 0 : part + 1;
+        *out++ = v;
     }
+    q.end(r, cnt, left0 - q.left);
 }
 
 // classifier pieces (q6_K): 16 super-blocks per piece, lane = (block lane/4, chunk lane%4); the ring
 // holds two pieces
 #define FLOW_Q6_D 2
-__device__ __forceinline__ void flow_issue_q6(Ring &r, unsigned char *ring_base, int lane) {
-    if (uni(r.iss_left) == 0) return;
-    unsigned char *slot = ring_base + (uni(r.issued) % FLOW_Q6_D) * FLOW_Q6_PIECE;
-    const unsigned char *g = r.gptr;
-    __builtin_amdgcn_global_load_lds((const AS1 void *)(g + lane * 16), (AS3 void *)slot, 16, 0, 2);
-    __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 1024 + lane * 16), (AS3 void *)(slot + 1024), 16, 0, 2);
-    __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 2048 + lane * 16), (AS3 void *)(slot + 2048), 16, 0, 2);
-    if (lane < 16)
-        __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 3072 + lane * 16), (AS3 void *)(slot + 3072), 16, 0, 2);
-    if (lane < 2)
-        __builtin_amdgcn_global_load_lds((const AS1 void *)(g + 3328 + lane * 16), (AS3 void *)(slot + 3328), 16, 0, 2);
-    r.gptr += FLOW_Q6_PIECE;
-    r.issued++;
-    r.iss_left--;
+__device__ __forceinline__ void flow_fetch_q6(const unsigned char *g, unsigned char *ring_base, int off, int lane) {
+    unsigned char *slot = ring_base + off;
+    const unsigned char *gl = g + lane * 16;
+    __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 0, 2);
+    __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 1024, 2);
+    __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 2048, 2);
+    if (lane < 16) __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 3072, 2);
+    if (lane < 2) __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 3328, 2);
+}
+
+__device__ __forceinline__ void flow_top_up_q6(Ring &r, unsigned char *ring_base, int lane) {
+#pragma nounroll
+    for (int k = 0; k < FLOW_Q6_D; k++) {
+        const int held = uni(r.issued) - uni(r.consumed);
+        if (held >= FLOW_Q6_D || uni(r.left) <= 0) break;
+        int o = uni(r.off) + held * FLOW_Q6_PIECE;
+        if (o >= FLOW_Q6_D * FLOW_Q6_PIECE) o -= FLOW_Q6_D * FLOW_Q6_PIECE;
+        flow_fetch_q6(r.gptr, ring_base, o, lane);
+        r.gptr += FLOW_Q6_PIECE;
+        r.issued++;
+        r.left--;
+    }
 }
 
 __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
@@ -501,12 +487,15 @@ __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigne
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     const int b = lane >> 2, c = lane & 3, n = c >> 1, h = c & 1;
     const XLds x = flow_x();
-    flow_drain(r);
+    RingLoop<FLOW_Q6_PIECE, FLOW_Q6_D, 5> q;
+    q.begin(r);
+    const int left0 = q.left;
     int part = uni(start % ppr);
     double acc = 0.0;
+#pragma nounroll
     for (int k = 0; k < cnt; k++) {
-        flow_wait_piece<5>(r);
-        const unsigned slot = r.lds + (unsigned)(uni(r.consumed) % FLOW_Q6_D) * FLOW_Q6_PIECE;
+        q.wait();
+        const unsigned slot = r.lds + (unsigned)q.off;
         Chunk<L2H_TYPE_Q6_K> ch;
         uint32_t d16;
         asm volatile("ds_read_b128 %0, %5\n\tds_read_b128 %1, %5 offset:32\n\tds_read_b128 %2, %6 offset:2048\n\t"
@@ -516,10 +505,14 @@ __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigne
                        "v"(slot + (b * 4 + 2 * n + h) * 4), "v"(slot + b * 2)
                      : "memory");
         ch.d = d16;
-        r.consumed++;
-        flow_issue_q6(r, ring_base, lane);
+        q.used();
+        if (q.left > 0) {
+            flow_fetch_q6(q.gp, ring_base, q.off, lane);
+            q.fetched();
+        }
+        q.next_slot();
         acc += chunk_term<false>(ch, part * 64 + lane, x, nullptr, nullptr, 0);
-        const bool last = k == cnt - 1 || uni(part) == ppr - 1;
+        const bool last = k == cnt - 1 || part == ppr - 1;
         if (last) {
             const double v = wave_sum_f64_dpp(acc);
             if (lane == 0) s_part[start + k] = v;
@@ -529,6 +522,7 @@ __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigne
         }
         part = part == ppr - 1 ? 0 : part + 1;
     }
+    q.end(r, cnt, left0 - q.left);
 }
 
 // fp32 value of every local row: the pieces' partial sums added in order
@@ -682,6 +676,38 @@ __device__ __noinline__ void flow_pick_token(int nwg, unsigned e_cls) {
     ctl->pos += 1;
 }
 
+// The cache lines that head h's attention will read (positions before `pos`) are requested early, while
+// the q/k/v matvec still runs: one 4-byte fetch per 128-byte line into a sink in LDS, so that the
+// attention's own loads find the lines in the L2 instead of waiting for HBM twice in a row (scores,
+// then values).  Position `pos` itself is not read from the cache by this launch.
+__device__ __forceinline__ void flow_touch_cache(int layer, int h, int pos) {
+    const FlowArgs &a = c_flow;
+    if (pos <= 0) return;
+    const int hs = a.hs, seq_len = a.seq_len;
+    const int kvh = h / (a.n_heads / a.n_kv_heads);
+    const unsigned char *kc = (const unsigned char *)(a.kc + (int64_t)layer * a.cache_layer_elems);
+    const unsigned char *vc = (const unsigned char *)(a.vc + (int64_t)layer * a.cache_layer_elems);
+    const int lane = threadIdx.x & 63;
+    unsigned char *sink = s_sink;
+    // K: per group of four head dimensions a run of 16 * pos bytes; V: one run of 4 * hs * pos bytes
+    const int k_lines = (16 * pos + 127) / 128 + 1, n_k = (hs >> 2) * k_lines;
+    const int64_t v_bytes = (int64_t)4 * hs * pos;
+    const int n_v = (int)((v_bytes + 127) / 128) + 1;
+    for (int i0 = (threadIdx.x & ~63); i0 < n_k + n_v; i0 += blockDim.x) {
+        const int i = i0 + lane;
+        const unsigned char *g = nullptr;
+        if (i < n_k) {
+            const int j = i / k_lines, ln = i % k_lines;
+            const int64_t lo = ((int64_t)kvh * (hs >> 2) + j) * seq_len * 16, off = (lo & ~(int64_t)127) + 128 * ln;
+            if (off < lo + 16 * pos) g = kc + off;
+        } else if (i < n_k + n_v) {
+            const int64_t lo = (int64_t)kvh * seq_len * hs * 4, off = (lo & ~(int64_t)127) + 128 * (int64_t)(i - n_k);
+            if (off < lo + v_bytes) g = vc + off;
+        }
+        if (g) __builtin_amdgcn_global_load_lds((const AS1 void *)g, (AS3 void *)sink, 4, 0, 0);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // attention of head h by one workgroup (reference src/inference.jl:263-278); q and the current
 // position's k, v arrive as tagged words, earlier positions come from the cache (written by earlier
@@ -695,7 +721,7 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
     const float *vc = a.vc + (int64_t)layer * a.cache_layer_elems;
     double *s_q = (double *)s_act;
     double *s_p = s_q + hs;
-    double *s_r = s_p + seq_len;
+    double *s_r = s_p + ((seq_len + 1) & ~1);  // keeps the float areas behind it 16-byte aligned
     float *s_att = (float *)(s_r + (FLOW_NW * hs > 1024 ? FLOW_NW * hs : 1024));
     float *s_kcur = s_att + ((seq_len + 3) & ~3);
     float *s_vcur = s_kcur + hs;
@@ -752,24 +778,22 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
             const int t = t0 + tl;
             double acc = 0.0;
             if (t < np) {
-                if (t == pos) {
-                    for (int i = 4 * part * per; i < 4 * (part + 1) * per; i++) acc = fma(s_q[i], (double)s_kcur[i], acc);
-                } else {
-                    const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
-                    float4 kv[8];
+                // the current position's key is in LDS, the earlier ones in the cache: same code after the loads
+                const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
+                const float4 *kl = (const float4 *)s_kcur + part * per;
+                float4 kv[8];
 #pragma unroll
-                    for (int u = 0; u < 8; u++)
-                        if (u < per) kv[u] = kp[(int64_t)u * seq_len];
+                for (int u = 0; u < 8; u++)
+                    if (u < per) kv[u] = t == pos ? kl[u] : kp[(int64_t)u * seq_len];
 #pragma unroll
-                    for (int u = 0; u < 8; u++)
-                        if (u < per) {
-                            const double *qq = s_q + 4 * (part * per + u);
-                            acc = fma(qq[0], (double)kv[u].x, acc);
-                            acc = fma(qq[1], (double)kv[u].y, acc);
-                            acc = fma(qq[2], (double)kv[u].z, acc);
-                            acc = fma(qq[3], (double)kv[u].w, acc);
-                        }
-                }
+                for (int u = 0; u < 8; u++)
+                    if (u < per) {
+                        const double *qq = s_q + 4 * (part * per + u);
+                        acc = fma(qq[0], (double)kv[u].x, acc);
+                        acc = fma(qq[1], (double)kv[u].y, acc);
+                        acc = fma(qq[2], (double)kv[u].z, acc);
+                        acc = fma(qq[3], (double)kv[u].w, acc);
+                    }
             }
             s_sp[part * 256 + tl] = acc;
             __syncthreads();
@@ -857,13 +881,13 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     r.gptr = a.stream + a.wave_off[wg * FLOW_NW + wave];
     r.lds = (unsigned)(size_t)ring_base;
     r.issued = r.consumed = r.drain_mark = 0;
-    r.iss_layer = 0;
-    r.iss_kind = 0;
-    r.iss_seq = 0;
-    r.iss_left = flow_wave_pieces(a.qkv, wg, wave);
+    r.off = 0;
+    // the layers' pieces and, where the classifier is q4_K too, its pieces behind them: one stream
+    r.left = a.n_layers * (flow_wave_pieces(a.qkv, wg, wave) + flow_wave_pieces(a.wo, wg, wave) +
+                           flow_wave_pieces(a.w13, wg, wave) + flow_wave_pieces(a.w2, wg, wave)) +
+             (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces(a.cls, wg, wave) : 0);
     ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
-#pragma nounroll
-    for (int k = 0; k < FLOW_D; k++) flow_issue_q4(r, a, ring_base, wg, wave, lane);
+    flow_top_up_q4(r, ring_base, lane);
 
 #ifdef L2H_TIMELINE
     int tl_n = 0;
@@ -876,15 +900,9 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         __syncthreads(); \
         FTL();          \
     } while (0)
-#define FTLD()         \
-    do {               \
-        flow_drain(r); \
-        FTL();         \
-    } while (0)
 #else
 #define FTL()
 #define FTLS()
-#define FTLD()
 #endif
     FTL();
 #define LEAVE()        \
@@ -903,6 +921,10 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         s_rope[2 * tid + 1] = (float)sin((double)theta);
     }
     const unsigned E0 = gen0;
+    // attention of head h runs on workgroup h * stride + h % stride (spread over the XCDs)
+    const int att_stride = nwg / a.n_heads;
+    const int att_h = uni(wg / att_stride);
+    const bool is_att = uni((int)(att_h < a.n_heads && wg % att_stride == att_h % att_stride)) != 0;
     // the rows of x this workgroup adds to after wo (layer 0): straight from the embedding (:236)
     {
         const int lo = wg * a.wo.rpw, n = flow_n_local(a.wo, wg);
@@ -921,32 +943,32 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 #pragma nounroll
         for (int kind = 0; kind < 4; kind++) {
             bool ok;
-            ring_store(r);
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
-                ok = l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok, 0)
-                            : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok, FLOW_FILL);
+                ok = l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok)
+                            : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok);
             } else if (kind == 1) {
-                const int stride = nwg / a.n_heads;
-                const int h = wg / stride;
-                if (h < a.n_heads && wg % stride == h % stride)
-                    if (!uni(flow_attention(l, h, pos, e_q, e_att))) LEAVE();
+                if (is_att)
+                    if (!uni(flow_attention(l, att_h, pos, e_q, e_att))) LEAVE();
                 FTL();
-                ok = flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok, FLOW_FILL);
+                ok = flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok);
             } else if (kind == 2) {
-                ok = flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok, FLOW_FILL);
+                ok = flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
             } else {
-                ok = flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok, FLOW_FILL);
+                ok = flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok);
             }
-            ring_load(r);
             if (!uni(ok)) LEAVE();
             FTL();
             const FlowGeom g = flow_geom(a, kind);
             // the row of x this thread adds to after wo / w2: fetched now, used after the loop
             u64 oldw = 0;
             if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = tag_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
-            FTLD();
-            flow_loop_q4(g, r, ring_base, wg, 4 * l + kind);
+            // what the ring holds has landed by now: after this wait the first FLOW_D pieces need none,
+            // and the cache lines requested next do not stand between the loop and its pieces
+            flow_drain(r);
+            FTL();
+            if (kind == 0 && is_att) flow_touch_cache(l, att_h, pos);
+            flow_loop_q4(g, r, ring_base, wg);
             FTL();
             FTLS();
             if (kind == 0)
@@ -961,23 +983,22 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         }
     }
 
-    // ---- final rmsnorm (:309) + classifier (:312); the ring restarts on the classifier's pieces ----
+    // ---- final rmsnorm (:309) + classifier (:312); q6_K pieces are larger: the ring starts afresh ----
     const unsigned e_fin = E0 + 5u * (unsigned)a.n_layers, e_cls = e_fin + 1;
-    flow_drain(r);
-    r.issued = r.consumed = r.drain_mark = 0;
-    r.iss_layer = a.n_layers;  // the layer phases are over: flow_issue_q4 fetches while iss_left lasts
-    r.iss_left = flow_wave_pieces(a.cls, wg, wave);
-    ring_uniform(r);
     if (T_CLS == L2H_TYPE_Q6_K) {
-        for (int k = 0; k < FLOW_Q6_D; k++) flow_issue_q6(r, ring_base, lane);
-    } else {
-        for (int k = 0; k < FLOW_D; k++) flow_issue_q4(r, a, ring_base, wg, wave, lane);
+        flow_drain(r);
+        r.issued = r.consumed = r.drain_mark = 0;
+        r.off = 0;
+        r.left = flow_wave_pieces(a.cls, wg, wave);
+        ring_uniform(r);
+        flow_top_up_q6(r, ring_base, lane);
     }
-    if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok, 0))) LEAVE();
+    if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok))) LEAVE();
+    flow_drain(r);
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
     else
-        flow_loop_q4(a.cls, r, ring_base, wg, -1);
+        flow_loop_q4(a.cls, r, ring_base, wg);
     flow_finish_cls(wg, e_cls);
     flow_drain(r);
     if (wg == 0) flow_pick_token(nwg, e_cls);
@@ -1071,7 +1092,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     if (cls_type == L2H_TYPE_Q6_K && a.dim % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
     if (a.hidden > 14336 || a.dim > 14336) return no("input vectors longer than 14336");
     if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 128)) return no("head size must be 32, 64 or 128");
-    const size_t att = (size_t)a.hs * 8 + (size_t)a.seq_len * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 +
+    const size_t att = (size_t)a.hs * 8 + (size_t)((a.seq_len + 1) & ~1) * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 +
                        (size_t)((a.seq_len + 3) & ~3) * 4 + (size_t)a.hs * 8;
     if (att > FLOW_ACT_BYTES) return no("sequence too long for the attention area");
     a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim, L2H_TYPE_Q4_K, grid);
