@@ -157,6 +157,15 @@ __device__ __forceinline__ FlowGeom flow_geom(const FlowArgs &a, int kind) {
 
 // the ring's bookkeeping is the same on every lane: keep it in scalar registers
 __device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ unsigned uni(unsigned v) { return (unsigned)__builtin_amdgcn_readfirstlane((int)v); }
+// (arguments of a function that is not inlined arrive in vector registers even when every lane holds
+// the same value; made scalar on entry, the arithmetic on them is scalar too)
+template <typename T>
+__device__ __forceinline__ T *uni(T *p) {
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = uni((unsigned)v), hi = uni((unsigned)(v >> 32));
+    return (T *)(((unsigned long long)hi << 32) | lo);
+}
 
 __device__ __forceinline__ void ring_uniform(Ring &r) {
     const unsigned long long p = (unsigned long long)r.gptr;
@@ -210,6 +219,7 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
 // ------------------------------------------------------------------------------------------
 template <int PRO, bool EMB>
 __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, const float *normw, int tok) {
+    src = uni(src), epoch = uni(epoch), K = uni(K), normw = uni(normw), tok = uni(tok);
     const FlowArgs &a = c_flow;
     int8_t *s_qs = (int8_t *)s_act;
     int16_t *s_bs = (int16_t *)(s_qs + 14336);
@@ -217,7 +227,22 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nb = K >> 8;
     float xv[STAGE_MAX_ROUNDS][4];
+    float wv[STAGE_MAX_ROUNDS][4];
     bool ok = true;
+    // the norm weights are requested before the wait for the input: their latency passes meanwhile
+    if (PRO == PRO_RMSNORM) {
+#pragma unroll
+        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+            const int b = wave + r * FLOW_NW;
+            if (b < nb) {
+                const float4 t = *(const float4 *)(normw + 256 * b + 4 * lane);
+                wv[r][0] = t.x;
+                wv[r][1] = t.y;
+                wv[r][2] = t.z;
+                wv[r][3] = t.w;
+            }
+        }
+    }
     if (EMB) {
 #pragma unroll
         for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
@@ -270,21 +295,13 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
                 for (int k = 0; k < 4; k++) xv[r][k] = tag_val(w[r][k]);
         }
     }
-    if (threadIdx.x == 0) s_flag = 0;
-    __syncthreads();
-    if (!ok) s_flag = 1;
-    float wv[STAGE_MAX_ROUNDS][4];
+    if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
     double acc = 0.0;
     if (PRO == PRO_RMSNORM) {  // rmsnorm! (reference src/inference.jl:102-110)
 #pragma unroll
         for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
             const int b = wave + r * FLOW_NW;
             if (b < nb) {
-                const float4 t = *(const float4 *)(normw + 256 * b + 4 * lane);
-                wv[r][0] = t.x;
-                wv[r][1] = t.y;
-                wv[r][2] = t.z;
-                wv[r][3] = t.w;
 #pragma unroll
                 for (int k = 0; k < 4; k++) acc = fma((double)xv[r][k], (double)xv[r][k], acc);
             }
@@ -539,6 +556,7 @@ __device__ __forceinline__ void flow_row_values(int n_local, int ppr) {
 // ---- epilogues -------------------------------------------------------------------------------
 // rope! (reference src/inference.jl:112-157) and the cache append (:259-260)
 __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
+    l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.qkv, wg), tid = threadIdx.x;
     flow_row_values(n_local, a.qkv.ppr);
@@ -571,6 +589,7 @@ __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_
 // dst = old + result (x .+= ..., :284,305); which = 1 after wo (-> x_b), 3 after w2 (-> x_a); `old` is
 // this thread's row of the other buffer, fetched before the loop
 __device__ __noinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsigned e_src, unsigned e_dst) {
+    which = uni(which), wg = uni(wg), e_src = uni(e_src), e_dst = uni(e_dst);
     const FlowArgs &a = c_flow;
     const FlowGeom &g = which == 1 ? a.wo : a.w2;
     const u64 *src = which == 1 ? a.x_a : a.x_b;
@@ -585,6 +604,7 @@ __device__ __noinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsi
 
 // SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u
 __device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
+    wg = uni(wg), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.w13, wg), tid = threadIdx.x;
     flow_row_values(n_local, a.w13.ppr);
@@ -596,6 +616,7 @@ __device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
 // logits (:312) and this workgroup's first-maximum key: larger value wins, then the lower index
 // (Julia's argmax, :360)
 __device__ __noinline__ void flow_finish_cls(int wg, unsigned e_cls) {
+    wg = uni(wg), e_cls = uni(e_cls);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.cls, wg), tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     flow_row_values(n_local, a.cls.ppr);
@@ -713,19 +734,27 @@ __device__ __forceinline__ void flow_touch_cache(int layer, int h, int pos) {
 // position's k, v arrive as tagged words, earlier positions come from the cache (written by earlier
 // launches).  Same arithmetic, in the same order, as attention_head.
 // ------------------------------------------------------------------------------------------
-__device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned e_in, unsigned e_out) {
+// Caches of up to FLOW_ATT_SHORT positions, the usual case: built for little waiting rather than for
+// throughput (one head is a few hundred KiB at most).  All keys are requested at once, before q has
+// arrived, all values as soon as the scores are done; barriers separate scores | maximum | sum | values.  HS is a
+// template parameter so that nothing below loops or branches on the head size.
+#define FLOW_ATT_SHORT 256
+template <int HS>
+__device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, unsigned e_in, unsigned e_out) {
+    layer = uni(layer), h = uni(h), pos = uni(pos), e_in = uni(e_in), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
-    const int hs = a.hs, seq_len = a.seq_len, np = pos + 1;
+    constexpr int hs = HS, n4 = HS >> 2, ngrp = FLOW_NW * 64 / n4, per = HS >> 4, NV = FLOW_ATT_SHORT / ngrp;
+    const int seq_len = a.seq_len, np = pos + 1;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
     const float *kc = a.kc + (int64_t)layer * a.cache_layer_elems;
     const float *vc = a.vc + (int64_t)layer * a.cache_layer_elems;
-    double *s_q = (double *)s_act;
-    double *s_p = s_q + hs;
-    double *s_r = s_p + ((seq_len + 1) & ~1);  // keeps the float areas behind it 16-byte aligned
-    float *s_att = (float *)(s_r + (FLOW_NW * hs > 1024 ? FLOW_NW * hs : 1024));
-    float *s_kcur = s_att + ((seq_len + 3) & ~3);
+    float *s_q = (float *)s_act;             // fp32 as it arrives; widened where it is used
+    float *s_kcur = s_q + hs;
     float *s_vcur = s_kcur + hs;
-    const int tid = threadIdx.x;
+    float *s_att = s_vcur + hs;              // [FLOW_ATT_SHORT]
+    double *s_p = (double *)(s_att + FLOW_ATT_SHORT);  // [FLOW_ATT_SHORT]
+    double *s_r = s_p + FLOW_ATT_SHORT;      // [FLOW_NW][hs]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     bool ok = true;
 #ifdef L2H_TIMELINE
     int atl = 0;
@@ -751,6 +780,141 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
             }
             w = tag_load(p);
         }
+        s_q[tid] = tag_val(w);  // s_q, s_kcur, s_vcur lie one behind the other
+    }
+    if (!ok) s_flag = 1;
+    // scores: lane = (timestep p16 of the wavefront's 16, quarter of the head dimension);
+    // values: thread = (16-byte group i4 of the head dimension, timestep group grp), timesteps grp + u * ngrp
+    const int p16 = lane & 15, part = lane >> 4, t = 16 * wave + p16;
+    const int i4 = tid & (n4 - 1), grp = tid / n4;
+    float4 kv[per], v[NV];
+    {
+        const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
+#pragma unroll
+        for (int u = 0; u < per; u++)
+            if (t < pos) kv[u] = kp[(int64_t)u * seq_len];
+    }
+    __syncthreads();
+    if (s_flag) {
+        if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return false;
+    }
+    ATL();
+    // the current position's key and value are in LDS, the earlier ones came from the cache
+    if (t == pos) {
+#pragma unroll
+        for (int u = 0; u < per; u++) kv[u] = ((const float4 *)s_kcur)[part * per + u];
+    }
+    const float scale = sqrtf((float)hs);
+    float sc = -INFINITY;
+    {
+        double acc = 0.0;
+        if (t < np) {
+#pragma unroll
+            for (int u = 0; u < per; u++) {
+                const float4 qq = ((const float4 *)s_q)[part * per + u];
+                acc = fma((double)qq.x, (double)kv[u].x, acc);
+                acc = fma((double)qq.y, (double)kv[u].y, acc);
+                acc = fma((double)qq.z, (double)kv[u].z, acc);
+                acc = fma((double)qq.w, (double)kv[u].w, acc);
+            }
+        }
+        // the values are requested now (the keys' registers are free): they arrive during the softmax
+        const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
+#pragma unroll
+        for (int u = 0; u < NV; u++) {
+            const int tv = grp + u * ngrp;
+            v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (tv < pos) v[u] = vp[(int64_t)tv * n4];
+            else if (tv == pos) v[u] = ((const float4 *)s_vcur)[i4];
+        }
+        // the quarters are added in order (fp64)
+        const double a1 = __shfl(acc, p16 + 16, WAVE), a2 = __shfl(acc, p16 + 32, WAVE), a3 = __shfl(acc, p16 + 48, WAVE);
+        if (part == 0 && t < np) sc = (float)(((acc + a1) + a2) + a3) / scale;
+    }
+    float mx = wave_max_f32_dpp(sc);
+    if (lane == 0) s_redf[wave] = mx;
+    ATL();
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < FLOW_NW; w++) mx = fmaxf(mx, s_redf[w]);
+    float e = 0.0f;
+    if (part == 0 && t < np) e = (float)exp((double)(sc - mx));
+    const double sum = wave_sum_f64_dpp((double)e);
+    if (lane == 0) s_red[wave] = sum;
+    __syncthreads();
+    double tot = 0.0;
+#pragma unroll
+    for (int w = 0; w < FLOW_NW; w++) tot += s_red[w];
+    const float sf = (float)tot;
+    if (part == 0 && t < np) s_p[t] = (double)(e / sf);  // softmax!, :169-174
+    __syncthreads();
+    ATL();
+    {
+        double acc[4] = {0.0, 0.0, 0.0, 0.0};
+#pragma unroll
+        for (int u = 0; u < NV; u++) {
+            const int tv = grp + u * ngrp;
+            if (tv < np) {
+                const double p = s_p[tv];
+                acc[0] = fma(p, (double)v[u].x, acc[0]);
+                acc[1] = fma(p, (double)v[u].y, acc[1]);
+                acc[2] = fma(p, (double)v[u].z, acc[2]);
+                acc[3] = fma(p, (double)v[u].w, acc[3]);
+            }
+        }
+#pragma unroll
+        for (int off = n4; off < 64; off <<= 1)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[c] += __shfl_xor(acc[c], off, WAVE);
+        if (lane < n4) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) s_r[wave * hs + 4 * i4 + c] = acc[c];
+        }
+    }
+    __syncthreads();
+    ATL();
+    if (tid < hs) {
+        double acc = 0.0;
+#pragma unroll
+        for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
+        tag_store(a.xb + (int64_t)h * hs + tid, (float)acc, e_out);
+    }
+    __syncthreads();
+    return true;
+}
+#undef ATL
+
+// longer caches: the same arithmetic with loops over the timesteps
+__device__ __noinline__ bool flow_attention_long(int layer, int h, int pos, unsigned e_in, unsigned e_out) {
+    layer = uni(layer), h = uni(h), pos = uni(pos), e_in = uni(e_in), e_out = uni(e_out);
+    const FlowArgs &a = c_flow;
+    const int hs = a.hs, seq_len = a.seq_len, np = pos + 1;
+    const int kvh = h / (a.n_heads / a.n_kv_heads);
+    const float *kc = a.kc + (int64_t)layer * a.cache_layer_elems;
+    const float *vc = a.vc + (int64_t)layer * a.cache_layer_elems;
+    double *s_q = (double *)s_act;
+    double *s_p = s_q + hs;
+    double *s_r = s_p + ((seq_len + 1) & ~1);  // keeps the float areas behind it 16-byte aligned
+    float *s_att = (float *)(s_r + (FLOW_NW * hs > 1024 ? FLOW_NW * hs : 1024));
+    float *s_kcur = s_att + ((seq_len + 3) & ~3);
+    float *s_vcur = s_kcur + hs;
+    const int tid = threadIdx.x;
+    bool ok = true;
+    __syncthreads();  // the activation area is free
+    if (tid < 3 * hs) {
+        const int which = tid / hs, i = tid % hs;
+        const u64 *p = which == 0 ? a.q + (int64_t)h * hs + i : (which == 1 ? a.kcur : a.vcur) + (int64_t)kvh * hs + i;
+        u64 w = tag_load(p);
+        unsigned spins = 0;
+        while (!tag_is(w, e_in)) {
+            if (++spins > a.spin_limit ||
+                ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                ok = false;
+                break;
+            }
+            w = tag_load(p);
+        }
         if (which == 0)
             s_q[i] = (double)tag_val(w);
         else if (which == 1)
@@ -758,15 +922,12 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
         else
             s_vcur[i] = tag_val(w);
     }
-    if (tid == 0) s_flag = 0;
-    __syncthreads();
     if (!ok) s_flag = 1;
     __syncthreads();
     if (s_flag) {
         if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return false;
     }
-    ATL();
     const float scale = sqrtf((float)hs);
     float mx = -INFINITY;
     // scores: thread = (timestep tl of a block of 256, quarter of the head dimension); the quarter's
@@ -806,7 +967,6 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
             __syncthreads();
         }
     }
-    ATL();
     mx = block_max_f32(mx, s_redf);
     double sum = 0.0;
     for (int t = tid; t < np; t += blockDim.x) {
@@ -817,7 +977,6 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
     const float sf = (float)block_sum_f64(sum, s_red);
     for (int t = tid; t < np; t += blockDim.x) s_p[t] = (double)(s_att[t] / sf);
     __syncthreads();
-    ATL();
     // values: thread = (16-byte group i4 of the head dimension, timestep group), up to eight loads in
     // flight; the groups of one wavefront are folded with lane exchanges, the rest through LDS
     const int n4 = hs >> 2;         // a power of two (hs 32, 64, 128)
@@ -857,7 +1016,6 @@ __device__ __noinline__ bool flow_attention(int layer, int h, int pos, unsigned 
         }
     }
     __syncthreads();
-    ATL();
     if (tid < hs) {
         double acc = 0.0;
         for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
@@ -914,6 +1072,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     // ---- this step's token, position and RoPE angles (reference src/inference.jl:122-127) ----
     const int pos = a.ctl->pos;
     const int tok = a.ctl->step < a.ctl->n_prompt ? a.prompt[a.ctl->step] : a.ctl->last_argmax;
+    if (tid == 0) s_flag = 0;
     if (tid < (a.hs >> 1)) {
         float theta = 1.0f * (float)pos;
         for (int k = 0; k < tid; k++) theta *= a.theta_scale;
@@ -948,8 +1107,13 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                 ok = l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok)
                             : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok);
             } else if (kind == 1) {
-                if (is_att)
-                    if (!uni(flow_attention(l, att_h, pos, e_q, e_att))) LEAVE();
+                if (is_att) {
+                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_long(l, att_h, pos, e_q, e_att)
+                                      : a.hs == 128 ? flow_attention_short<128>(l, att_h, pos, e_q, e_att)
+                                      : a.hs == 64  ? flow_attention_short<64>(l, att_h, pos, e_q, e_att)
+                                                    : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
+                    if (!uni((int)fine)) LEAVE();
+                }
                 FTL();
                 ok = flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok);
             } else if (kind == 2) {
