@@ -690,7 +690,8 @@ static int flow_setup(l2h_model *m) {
     TA(a.q, c.dim);
     TA(a.kcur, m->kv_dim);
     TA(a.vcur, m->kv_dim);
-    TA(a.hb, c.hidden_dim);
+    TA(a.hbw, 2 * (int64_t)c.hidden_dim);
+    HIPCHK(ctx, hipMemset(a.hbw, 0xFF, 2 * (size_t)c.hidden_dim * 4));
     TA(a.amax, 2 * grid);
     TA(a.abort_flag, 1);
 #undef TA
@@ -865,6 +866,7 @@ static int mega_check(l2h_model *m) {
         HIPCHK(m->ctx, hipMemcpy(&ab, m->flow_args.abort_flag, 4, hipMemcpyDeviceToHost));
         if (!ab) return L2H_OK;
         HIPCHK(m->ctx, hipMemset(m->flow_args.abort_flag, 0, 4));
+        HIPCHK(m->ctx, hipMemset(m->flow_args.hbw, 0xFF, 2 * (size_t)m->c.hidden_dim * 4));  // all words "not written"
         return set_err(m->ctx, L2H_EHIP, "streaming decode kernel: a wait for activations timed out");
     }
     if (!m->mega) return L2H_OK;

@@ -31,6 +31,7 @@
 #define FLOW_MAX_ROWS 512     // per workgroup and phase
 
 typedef unsigned long long u64;
+typedef unsigned int u32x4v __attribute__((ext_vector_type(4)));
 
 // Arguments of the model being decoded (everything but the epoch of the launch): constant memory,
 // read with scalar loads wherever a phase needs a field.
@@ -60,6 +61,19 @@ __device__ __forceinline__ u64 tag_load(const u64 *p) {
 }
 __device__ __forceinline__ bool tag_is(u64 w, unsigned epoch) { return (unsigned)(w >> 32) == epoch; }
 __device__ __forceinline__ float tag_val(u64 w) { return __uint_as_float((unsigned)w); }
+// The SwiGLU outputs, the largest vector that all workgroups exchange, travel as bare fp32 words, half
+// the bytes of tagged ones.  A word that has not been written holds FLOW_EMPTY, a NaN pattern that no
+// arithmetic here produces (a result that happens to have it is stored as the default NaN).  There are
+// two buffers; the phase with epoch e uses buffer e & 1 (consecutive layers, and the last layer of one
+// launch and the first of the next, differ in that bit), and whoever writes word i of one buffer puts
+// FLOW_EMPTY back into word i of the other: every reader of that one finished with it a phase ago.
+#define FLOW_EMPTY 0xFFFFFFFFu
+__device__ __forceinline__ unsigned bare_load(const unsigned *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void bare_store(unsigned *p, unsigned v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 
 __host__ __device__ inline int flow_n_local(const FlowGeom &g, int wg) {
     const int lo = wg * g.rpw;
@@ -217,8 +231,12 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
 // epoch `epoch`, or (EMB) the embedding row of `tok`.  Returns false if the wait gave up.
 // Separate functions (not inlined): the kernel stays small enough to keep its state in registers.
 // ------------------------------------------------------------------------------------------
-template <int PRO, bool EMB>
-__device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, const float *normw, int tok) {
+// SRC: where the input comes from
+#define SRC_EMB 0     // the embedding row of `tok`
+#define SRC_TAGGED 1  // {fp32, epoch} words; a word is there when it carries `epoch`
+#define SRC_BARE 2    // fp32 words; a word is there when it is not FLOW_EMPTY
+template <int PRO, int SRC>
+__device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, const float *normw, int tok) {
     src = uni(src), epoch = uni(epoch), K = uni(K), normw = uni(normw), tok = uni(tok);
     const FlowArgs &a = c_flow;
     int8_t *s_qs = (int8_t *)s_act;
@@ -243,7 +261,7 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
             }
         }
     }
-    if (EMB) {
+    if (SRC == SRC_EMB) {
 #pragma unroll
         for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
             const int b = wave + r * FLOW_NW;
@@ -252,26 +270,54 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
                 for (int k = 0; k < 4; k++) xv[r][k] = dequant_elem(a.emb, tok, 256 * b + 4 * lane + k);
         }
     } else {
+        // A lane's four words are one contiguous, 16-byte aligned run: fetched with 16-byte loads (agent
+        // scope; every aligned 4- or 8-byte word of such a load is read whole), so that one instruction
+        // asks for whole cache lines.  First pass: every lane; later passes: the lanes that miss a word.
         unsigned spins = 0;
-        // first pass: every word; later passes: only the words that did not carry the epoch yet, so
-        // that waiting for a slow producer costs next to no traffic
-        u64 w[STAGE_MAX_ROUNDS][4];
+        // (the loads name their target registers as read-write operands: the data lands in the registers that
+        // already stand for the words, with no copy in between that could run before it has arrived)
+        u32x4v wl[STAGE_MAX_ROUNDS], wh[STAGE_MAX_ROUNDS];  // tagged: words 0,1 | 2,3; bare: wl only
+#define STAGE_FETCH(r)                                                                                                 \
+    do {                                                                                                               \
+        if (SRC == SRC_TAGGED) {                                                                                       \
+            const u64 *p_ = (const u64 *)src + 256 * (wave + (r)*FLOW_NW) + 4 * lane;                                   \
+            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1"         \
+                         : "+v"(wl[r]), "+v"(wh[r])                                                                    \
+                         : "v"(p_)                                                                                     \
+                         : "memory");                                                                                  \
+        } else {                                                                                                       \
+            const unsigned *p_ = (const unsigned *)src + 256 * (wave + (r)*FLOW_NW) + 4 * lane;                         \
+            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "+v"(wl[r]) : "v"(p_) : "memory");                    \
+        }                                                                                                              \
+    } while (0)
+// the loads above have returned; naming their registers keeps every use behind this point
+#define STAGE_ARRIVED()                                                                                                \
+    do {                                                                                                               \
+        static_assert(STAGE_MAX_ROUNDS == 4, "operand list below");                                                    \
+        if (SRC == SRC_TAGGED)                                                                                         \
+            asm volatile("s_waitcnt vmcnt(0)"                                                                          \
+                         : "+v"(wl[0]), "+v"(wl[1]), "+v"(wl[2]), "+v"(wl[3]), "+v"(wh[0]), "+v"(wh[1]), "+v"(wh[2]),  \
+                           "+v"(wh[3])                                                                                 \
+                         :                                                                                             \
+                         : "memory");                                                                                  \
+        else                                                                                                           \
+            asm volatile("s_waitcnt vmcnt(0)" : "+v"(wl[0]), "+v"(wl[1]), "+v"(wl[2]), "+v"(wl[3]) : : "memory");      \
+    } while (0)
+#define STAGE_COMPLETE(r)                                                                                          \
+    (SRC == SRC_TAGGED ? (wl[r].y == epoch && wl[r].w == epoch && wh[r].y == epoch && wh[r].w == epoch)            \
+                       : (wl[r].x != FLOW_EMPTY && wl[r].y != FLOW_EMPTY && wl[r].z != FLOW_EMPTY && wl[r].w != FLOW_EMPTY))
 #pragma unroll
         for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            const int b = wave + r * FLOW_NW;
-            if (b < nb)
-#pragma unroll
-                for (int k = 0; k < 4; k++) w[r][k] = tag_load(src + 256 * b + 4 * lane + k);
+            wl[r] = (u32x4v){0, 0, 0, 0};
+            wh[r] = (u32x4v){0, 0, 0, 0};
+            if (wave + r * FLOW_NW < nb) STAGE_FETCH(r);
         }
+        STAGE_ARRIVED();
         for (;;) {
             bool all = true;
 #pragma unroll
-            for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-                const int b = wave + r * FLOW_NW;
-                if (b < nb)
-#pragma unroll
-                    for (int k = 0; k < 4; k++) all = all && tag_is(w[r][k], epoch);
-            }
+            for (int r = 0; r < STAGE_MAX_ROUNDS; r++)
+                if (wave + r * FLOW_NW < nb) all = all && STAGE_COMPLETE(r);
             if (__ballot(!all) == 0ull) break;
             if (++spins > a.spin_limit ||
                 ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
@@ -279,20 +325,26 @@ __device__ __noinline__ bool flow_stage(const u64 *src, unsigned epoch, int K, c
                 break;
             }
 #pragma unroll
-            for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-                const int b = wave + r * FLOW_NW;
-                if (b < nb)
-#pragma unroll
-                    for (int k = 0; k < 4; k++)
-                        if (!tag_is(w[r][k], epoch)) w[r][k] = tag_load(src + 256 * b + 4 * lane + k);
-            }
+            for (int r = 0; r < STAGE_MAX_ROUNDS; r++)
+                if (wave + r * FLOW_NW < nb && !STAGE_COMPLETE(r)) STAGE_FETCH(r);
+            STAGE_ARRIVED();
         }
+#undef STAGE_FETCH
+#undef STAGE_ARRIVED
+#undef STAGE_COMPLETE
 #pragma unroll
         for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            const int b = wave + r * FLOW_NW;
-            if (b < nb)
-#pragma unroll
-                for (int k = 0; k < 4; k++) xv[r][k] = tag_val(w[r][k]);
+            if (SRC == SRC_TAGGED) {
+                xv[r][0] = __uint_as_float(wl[r].x);
+                xv[r][1] = __uint_as_float(wl[r].z);
+                xv[r][2] = __uint_as_float(wh[r].x);
+                xv[r][3] = __uint_as_float(wh[r].z);
+            } else {
+                xv[r][0] = __uint_as_float(wl[r].x);
+                xv[r][1] = __uint_as_float(wl[r].y);
+                xv[r][2] = __uint_as_float(wl[r].z);
+                xv[r][3] = __uint_as_float(wl[r].w);
+            }
         }
     }
     if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
@@ -610,7 +662,11 @@ __device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
     flow_row_values(n_local, a.w13.ppr);
     if (tid >= n_local || (tid & 1)) return;
     const int64_t u = ((int64_t)wg * a.w13.rpw + tid) >> 1;
-    tag_store(a.hb + u, swiglu_val(s_val[tid], s_val[tid + 1]), e_out);
+    unsigned v = __float_as_uint(swiglu_val(s_val[tid], s_val[tid + 1]));
+    if (v == FLOW_EMPTY) v = 0x7FC00000u;
+    unsigned *mine = a.hbw + (int64_t)(e_out & 1u) * a.hidden, *other = a.hbw + (int64_t)((e_out & 1u) ^ 1u) * a.hidden;
+    bare_store(mine + u, v);
+    bare_store(other + u, FLOW_EMPTY);
 }
 
 // logits (:312) and this workgroup's first-maximum key: larger value wins, then the lower index
@@ -1104,8 +1160,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             bool ok;
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
-                ok = l == 0 ? flow_stage<PRO_RMSNORM, true>(nullptr, 0, a.dim, nw, tok)
-                            : flow_stage<PRO_RMSNORM, false>(a.x_a, e_x, a.dim, nw, tok);
+                ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, 0, a.dim, nw, tok)
+                            : flow_stage<PRO_RMSNORM, SRC_TAGGED>(a.x_a, e_x, a.dim, nw, tok);
             } else if (kind == 1) {
                 if (is_att) {
                     const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_long(l, att_h, pos, e_q, e_att)
@@ -1115,11 +1171,11 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                     if (!uni((int)fine)) LEAVE();
                 }
                 FTL();
-                ok = flow_stage<PRO_QUANT, false>(a.xb, e_att, a.dim, nullptr, tok);
+                ok = flow_stage<PRO_QUANT, SRC_TAGGED>(a.xb, e_att, a.dim, nullptr, tok);
             } else if (kind == 2) {
-                ok = flow_stage<PRO_RMSNORM, false>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
+                ok = flow_stage<PRO_RMSNORM, SRC_TAGGED>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
             } else {
-                ok = flow_stage<PRO_QUANT, false>(a.hb, e_w13, a.hidden, nullptr, tok);
+                ok = flow_stage<PRO_QUANT, SRC_BARE>(a.hbw + (int64_t)(e_w13 & 1u) * a.hidden, 0, a.hidden, nullptr, tok);
             }
             if (!uni(ok)) LEAVE();
             FTL();
@@ -1157,7 +1213,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         ring_uniform(r);
         flow_top_up_q6(r, ring_base, lane);
     }
-    if (!uni(flow_stage<PRO_RMSNORM, false>(a.x_a, e_fin, a.dim, a.rms_final, tok))) LEAVE();
+    if (!uni(flow_stage<PRO_RMSNORM, SRC_TAGGED>(a.x_a, e_fin, a.dim, a.rms_final, tok))) LEAVE();
     flow_drain(r);
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);

@@ -139,7 +139,8 @@ struct FlowArgs {
     const unsigned char *stream;  // per-wavefront weight streams
     const int64_t *wave_off;      // [grid * 16] byte offset of each wavefront's stream
     // activations as {fp32 value, epoch} words
-    unsigned long long *x_a, *x_b, *xb, *q, *kcur, *vcur, *hb, *amax;
+    unsigned long long *x_a, *x_b, *xb, *q, *kcur, *vcur, *amax;
+    unsigned int *hbw;  // [2][hidden] SwiGLU outputs as bare fp32 words, 0xFFFFFFFF = not written yet
     float *kc, *vc, *logits;
     const float *rms_att, *rms_ffn, *rms_final;
     int64_t norm_stride;  // floats between the norm weights of consecutive layers
