@@ -208,6 +208,32 @@ def test_kv_prefill_and_long_context(pkg, orc, rng, path, seq_len):
     assert _rel(logits, ref_logits) <= 1e-3
 
 
+@pytest.mark.parametrize("n_pre", [250, 300])
+def test_streaming_kernel_long_cache(pkg, orc, rng, n_pre):
+    """Path 3 decoding into a pre-filled cache: from 250 the run crosses position 256, where the kernel
+    changes from its short-cache attention to the one with loops over the timesteps; from 300 it is in
+    the latter throughout."""
+    plan, kw = FLOW_CASES["all_q4"]
+    kw = dict(kw, seq_len=384, n_layers=2)
+    lm = _model(pkg, plan, **kw)
+    cfg = lm.config
+    dev = lm.device(path=3)
+    assert dev.path == 3
+    om = orc.model_from_language_model(lm, nthreads=8)
+    dev.reset()
+    om.reset()
+    kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads
+    for layer in range(cfg.n_layers):
+        k = rng.standard_normal((n_pre, kv_dim)).astype(np.float32)
+        v = rng.standard_normal((n_pre, kv_dim)).astype(np.float32)
+        dev.kv_write(layer, 0, k, v)
+        om.kv_write(layer, 0, k, v)
+    ids, logits = dev.generate_greedy([7], 12, pos0=n_pre, want_logits=True)
+    ref_ids, ref_logits = om.generate_greedy([7], 12, orc.GPU_SPEC, pos0=n_pre)
+    assert ids.tolist() == ref_ids.tolist()
+    assert _rel(logits, ref_logits) <= 1e-3
+
+
 def test_generate_argument_checks(pkg):
     from llama2_jl_amd import synth
     plan, kw = CASES["f32"]
