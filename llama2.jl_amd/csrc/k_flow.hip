@@ -417,6 +417,30 @@ __device__ __forceinline__ XLds flow_x() {
     return x;
 }
 
+// q4_term on operands that are already in registers: w the lane's 16 bytes of quants, xlo / xhi its 2 x 16
+// activations, bs_a / bs_b their block sums, yd the activation block's scale
+__device__ __forceinline__ double flow_q4_term(const uint4 w, uint32_t d_dmin, int sc_a, int sc_b, int m_a, int m_b,
+                                               const uint4 xlo, const uint4 xhi, int bs_a, int bs_b, float yd) {
+    int dot_a, dot_b;
+    // (the first product of each sum in the three-operand form with a literal zero: no register to clear)
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(dot_a) : "v"(w.x & 0x0F0F0F0Fu), "v"(xlo.x));
+    dot_a = sdot4(w.y & 0x0F0F0F0Fu, xlo.y, dot_a);
+    dot_a = sdot4(w.z & 0x0F0F0F0Fu, xlo.z, dot_a);
+    dot_a = sdot4(w.w & 0x0F0F0F0Fu, xlo.w, dot_a);
+    asm("v_dot4_i32_i8 %0, %1, %2, 0" : "=v"(dot_b) : "v"((w.x >> 4) & 0x0F0F0F0Fu), "v"(xhi.x));
+    dot_b = sdot4((w.y >> 4) & 0x0F0F0F0Fu, xhi.y, dot_b);
+    dot_b = sdot4((w.z >> 4) & 0x0F0F0F0Fu, xhi.z, dot_b);
+    dot_b = sdot4((w.w >> 4) & 0x0F0F0F0Fu, xhi.w, dot_b);
+    // every factor fits 24 bits (scales < 64, |dot| <= 16*15*127, |bsum| <= 16*127): full-rate multiplies
+    const int i_sc = mad24(sc_a, dot_a, __mul24(sc_b, dot_b));
+    const int i_min = mad24(m_a, bs_a, __mul24(m_b, bs_b));
+    const float dy = half_bits_to_float((uint16_t)(d_dmin & 0xFFFF)) * yd;
+    const float my = half_bits_to_float((uint16_t)(d_dmin >> 16)) * yd;
+    double t = (double)dy * (double)i_sc;
+    t = fma(-(double)my, (double)i_min, t);
+    return t;
+}
+
 // The ring is kept full: as soon as a piece has been read into registers, the next piece of the stream
 // is fetched into its slot, whichever phase that piece belongs to.  The loop's bookkeeping is a handful
 // of scalars (the scalar unit is shared by the 16 wavefronts of the workgroup, so every scalar
@@ -473,24 +497,38 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
-    const XLds x = flow_x();
     RingLoop<FLOW_SLOT, FLOW_D, 2> q;
     q.begin(r);
     const int left0 = q.left;
     const unsigned rd_w = r.lds + lane * 16, rd_h = r.lds + (lane >> 3) * 16;
     const int pair = (lane & 7) >> 1;
     int part = uni(start % ppr);
-    int xi = part * 64 + lane;  // index of this lane's 32 activations
+    // this lane's activations for piece `part` of a row: block part * 8 + lane / 8, chunk lane % 8
+    const int c8 = lane & 7;
+    // LDS byte addresses of this lane's activations for piece 0 of a row (quants, block sums, scale); piece
+    // `part` lies part * (2048, 256, 32) bytes further on
+    const unsigned act = (unsigned)(size_t)s_act;
+    const unsigned xq0 = act + (lane >> 3) * 256 + 64 * (c8 >> 1) + 16 * (c8 & 1);
+    const unsigned xs0 = act + 14336 + 2 * ((lane >> 3) * 16 + 4 * (c8 >> 1) + (c8 & 1));
+    const unsigned xd0 = act + 14336 + 1792 + 4 * (lane >> 3);
+    int po = part * 32;  // piece index in units that scale to the three strides (2048, 256, 32 bytes)
     double *out = s_part + start;
     double acc = 0.0;
 #pragma nounroll
     for (int k = cnt; k > 0; k--) {
         q.wait();
+        // all LDS reads of the piece in one statement the compiler does not look into: it would otherwise hold
+        // the reads of the activation area back until every asynchronous fetch into the ring had landed
         Chunk<L2H_TYPE_Q4_K> ch;
-        asm volatile("ds_read_b128 %0, %2 offset:128\n\tds_read_b128 %1, %3\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&v"(ch.w), "=&v"(ch.hdr)
-                     : "v"(rd_w + q.off), "v"(rd_h + q.off)
-                     : "memory");
+        uint4 xlo, xhi;
+        int bs_a, bs_b;
+        float yd;
+        asm volatile(
+            "ds_read_b128 %0, %7 offset:128\n\tds_read_b128 %1, %8\n\tds_read_b128 %2, %9\n\tds_read_b128 %3, %9 offset:32\n\t"
+            "ds_read_i16 %4, %10\n\tds_read_i16 %5, %10 offset:4\n\tds_read_b32 %6, %11\n\ts_waitcnt lgkmcnt(0)"
+            : "=&v"(ch.w), "=&v"(ch.hdr), "=&v"(xlo), "=&v"(xhi), "=&v"(bs_a), "=&v"(bs_b), "=&v"(yd)
+            : "v"(rd_w + q.off), "v"(rd_h + q.off), "v"(xq0 + po * 64), "v"(xs0 + po * 8), "v"(xd0 + po)
+            : "memory");
         q.used();
         if (q.left > 0) {  // the slot is free again
             flow_fetch_q4(q.gp, ring_base, q.off, lane);
@@ -501,21 +539,21 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
         acc += (double)(ch.w.x ^ ch.hdr.y);
 #else
         {
-            int sc_a, sc_b, m_a, m_b, i_sc, i_min;
+            int sc_a, sc_b, m_a, m_b;
             flow_decode_pair(ch.hdr, pair, sc_a, sc_b, m_a, m_b);
-            acc += q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, xi, x, i_sc, i_min);
+            acc += flow_q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
         }
 #endif
         // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot
         // in s_part, the run's total goes to its last piece and zero to the others
         // (every lane stores the same word: no lane-dependent branch in the loop)
         part++;
-        xi += 64;
+        po += 32;
         double v = 0.0;
         if (k == 1 || part == ppr) {
             v = wave_sum_f64_dpp(acc);
             acc = 0.0;
-            xi = lane;
+            po = 0;
             part = 0;
         }
         *out++ = v;
