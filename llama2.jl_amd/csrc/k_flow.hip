@@ -133,7 +133,8 @@ struct Ring {
 // Headers inside the streams carry the twelve 6-bit scale bytes of a q4_K super-block (reference
 // src/kquants.jl:80-109) regrouped so that a lane finds the four values of its sub-block pair j in
 // one 24-bit field f_j = sc(2j) | sc(2j+1) << 6 | m(2j) << 12 | m(2j+1) << 18:
-//   word 0 = d | dmin << 16;  word 1+k (k = 0..2) = f_k | byte k of f_3 << 24.
+//   bytes 0-3 = d | dmin << 16;  bytes 4 + 3j .. 6 + 3j = f_j (little endian), j = 0..3.
+// A lane reads the four bytes at 4 + 3j (not aligned; the byte above its field is ignored).
 __host__ __device__ inline uint32_t flow_pair_field(int sc_a, int sc_b, int m_a, int m_b) {
     return (uint32_t)sc_a | (uint32_t)sc_b << 6 | (uint32_t)m_a << 12 | (uint32_t)m_b << 18;
 }
@@ -145,14 +146,15 @@ __device__ __forceinline__ uint4 flow_encode_hdr(const uint4 hdr) {
         kq_scales_pair(hdr, j, sa, sb, ma, mb);
         f[j] = flow_pair_field(sa, sb, ma, mb);
     }
-    return make_uint4(hdr.x, f[0] | (f[3] & 0xFF) << 24, f[1] | ((f[3] >> 8) & 0xFF) << 24, f[2] | (f[3] >> 16) << 24);
+    return make_uint4(hdr.x, f[0] | (f[1] & 0xFF) << 24, (f[1] >> 8) | (f[2] & 0xFFFF) << 16, (f[2] >> 16) | f[3] << 8);
 }
-// this lane's field (j = 0..3 is fixed per lane: the selects use lane-constant conditions)
-__device__ __forceinline__ void flow_decode_pair(const uint4 hdr, int j, int &sc_a, int &sc_b, int &m_a, int &m_b) {
-    const uint32_t fw = j == 0 ? hdr.y : (j == 1 ? hdr.z : hdr.w);
-    const uint32_t t = __builtin_amdgcn_perm(hdr.z, hdr.y, 0x0c0c0703u);  // byte 3 of word 1, byte 3 of word 2
-    const uint32_t g = __builtin_amdgcn_perm(hdr.w, t, 0x0c070100u);      // ... and byte 3 of word 3
-    const uint32_t f = j == 3 ? g : fw;
+// field j out of a whole header (j is fixed per lane: the selects use lane-constant conditions).  LDS
+// reads that are not aligned are slow, so a lane reads the 16 bytes and shifts its field down.
+__device__ __forceinline__ uint32_t flow_field_of(const uint4 hdr, int j) {
+    const uint32_t lo = j < 2 ? hdr.y : (j == 2 ? hdr.z : hdr.w), hi = j == 1 ? hdr.z : hdr.w;
+    return __builtin_amdgcn_alignbit(hi, lo, (24 * j) & 31);
+}
+__device__ __forceinline__ void flow_decode_field(uint32_t f, int &sc_a, int &sc_b, int &m_a, int &m_b) {
     sc_a = (int)(f & 63);
     sc_b = (int)((f >> 6) & 63);
     m_a = (int)((f >> 12) & 63);
@@ -500,6 +502,7 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
     RingLoop<FLOW_SLOT, FLOW_D, 2> q;
     q.begin(r);
     const int left0 = q.left;
+    // this lane's quants, its super-block's d | dmin, and the scale field of its sub-block pair
     const unsigned rd_w = r.lds + lane * 16, rd_h = r.lds + (lane >> 3) * 16;
     const int pair = (lane & 7) >> 1;
     int part = uni(start % ppr);
@@ -519,16 +522,16 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
         q.wait();
         // all LDS reads of the piece in one statement the compiler does not look into: it would otherwise hold
         // the reads of the activation area back until every asynchronous fetch into the ring had landed
-        Chunk<L2H_TYPE_Q4_K> ch;
-        uint4 xlo, xhi;
+        uint4 w, hdr, xlo, xhi;
         int bs_a, bs_b;
         float yd;
         asm volatile(
             "ds_read_b128 %0, %7 offset:128\n\tds_read_b128 %1, %8\n\tds_read_b128 %2, %9\n\tds_read_b128 %3, %9 offset:32\n\t"
             "ds_read_i16 %4, %10\n\tds_read_i16 %5, %10 offset:4\n\tds_read_b32 %6, %11\n\ts_waitcnt lgkmcnt(0)"
-            : "=&v"(ch.w), "=&v"(ch.hdr), "=&v"(xlo), "=&v"(xhi), "=&v"(bs_a), "=&v"(bs_b), "=&v"(yd)
+            : "=&v"(w), "=&v"(hdr), "=&v"(xlo), "=&v"(xhi), "=&v"(bs_a), "=&v"(bs_b), "=&v"(yd)
             : "v"(rd_w + q.off), "v"(rd_h + q.off), "v"(xq0 + po * 64), "v"(xs0 + po * 8), "v"(xd0 + po)
             : "memory");
+        const uint32_t d_dmin = hdr.x, field = flow_field_of(hdr, pair);
         q.used();
         if (q.left > 0) {  // the slot is free again
             flow_fetch_q4(q.gp, ring_base, q.off, lane);
@@ -536,12 +539,12 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
         }
         q.next_slot();
 #ifdef FLOW_EXP_NOMATH
-        acc += (double)(ch.w.x ^ ch.hdr.y);
+        acc += (double)(w.x ^ field);
 #else
         {
             int sc_a, sc_b, m_a, m_b;
-            flow_decode_pair(ch.hdr, pair, sc_a, sc_b, m_a, m_b);
-            acc += flow_q4_term(ch.w, ch.hdr.x, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
+            flow_decode_field(field, sc_a, sc_b, m_a, m_b);
+            acc += flow_q4_term(w, d_dmin, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
         }
 #endif
         // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot
