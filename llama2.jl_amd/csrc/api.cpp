@@ -672,12 +672,12 @@ static int flow_setup(l2h_model *m) {
         const DevTensor wo[1] = {m->L(l, L2H_WO)};
         const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
         const DevTensor w2[1] = {m->L(l, L2H_W2)};
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 0, l, qkv, 3, grid));
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 1, l, wo, 1, grid));
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 2, l, w13, 2, grid));
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 3, l, w2, 1, grid));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 0, l, qkv, 3, grid, cls_type));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 1, l, wo, 1, grid, cls_type));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 2, l, w13, 2, grid, cls_type));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 3, l, w2, 1, grid, cls_type));
     }
-    HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid));
+    HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid, cls_type));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     a.stream = stream;
     a.wave_off = off_dev;

@@ -92,6 +92,22 @@ __host__ __device__ inline int flow_wave_start(const FlowGeom &g, int wg, int wa
     const int base = np / FLOW_NW, rem = np % FLOW_NW;
     return wave * base + (wave < rem ? wave : rem);
 }
+// While a phase waits for its input vector the memory system is idle and the ring is full.  At the start
+// of that wait a wavefront therefore requests the last FLOW_R pieces of its run for the phase into
+// registers; the ring's stream passes over them (they sit in a part of the wavefront's stream of their
+// own).  That moves their share of the HBM time out of the loops; the price is that the wait's first poll
+// returns after them (loads return in order), which is why there are only a few.
+#ifndef FLOW_R
+#define FLOW_R 2
+#endif
+__host__ __device__ inline int flow_reg_pieces(const FlowGeom &g, int wg, int wave) {
+    const int cnt = flow_wave_pieces(g, wg, wave);
+    return cnt < FLOW_R ? cnt : FLOW_R;
+}
+// pieces of a layer phase that go through the ring
+__host__ __device__ inline int flow_ring_pieces(const FlowGeom &g, int wg, int wave) {
+    return flow_wave_pieces(g, wg, wave) - flow_reg_pieces(g, wg, wave);
+}
 
 // logical row L of a phase -> (tensor of the phase, row in it).  Logical rows put the two rows an
 // epilogue combines next to each other: (w1 row u, w3 row u) and the two halves of a RoPE pair.
@@ -495,14 +511,45 @@ struct RingLoop {
     }
 };
 
-__device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
+// the pieces of a phase that a wavefront holds in registers (see flow_reg_pieces): per lane its 16 bytes of
+// quants, its super-block's d | dmin and the scale field of its sub-block pair
+struct RegPieces {
+    u32x4v q[FLOW_R];
+    uint32_t dm[FLOW_R], f[FLOW_R];
+};
+// requests them: n pieces at p (every index below is a constant after unrolling: the arrays stay registers)
+__device__ __forceinline__ void flow_reg_fetch(RegPieces &rp, const unsigned char *p, int n, int lane) {
+    const AS1 unsigned char *g = (const AS1 unsigned char *)p;  // (a global address: plain global loads)
+    const AS1 unsigned char *ph = g + (lane >> 3) * 16, *pq = g + 128 + lane * 16;
+    const int fo = 4 + 3 * ((lane & 7) >> 1);
+#pragma unroll
+    for (int i = 0; i < FLOW_R; i++)
+        if (i < n) {
+            rp.q[i] = __builtin_nontemporal_load((const AS1 u32x4v *)(pq + i * FLOW_SLOT));
+            rp.dm[i] = *(const AS1 uint32_t *)(ph + i * FLOW_SLOT);
+            uint32_t f;
+            __builtin_memcpy(&f, ph + i * FLOW_SLOT + fo, 4);  // not aligned: one load all the same
+            rp.f[i] = f;
+        }
+}
+// After a wait for everything this wavefront has requested: the compiler is told, in its own terms, that
+// the register pieces are there (it would otherwise wait for *all* outstanding requests, the ring's
+// fetches included, at their first use inside the loop).
+__device__ __forceinline__ void flow_reg_arrived(RegPieces &rp) {
+#pragma unroll
+    for (int i = 0; i < FLOW_R; i++) asm volatile("" : "+v"(rp.q[i]), "+v"(rp.dm[i]), "+v"(rp.f[i]));
+}
+
+// REGS: the wavefront's last n_reg pieces are in rp, the ones before them come through the ring
+template <bool REGS>
+__device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg, const RegPieces &rp,
+                                             int n_reg) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     RingLoop<FLOW_SLOT, FLOW_D, 2> q;
     q.begin(r);
     const int left0 = q.left;
-    // this lane's quants, its super-block's d | dmin, and the scale field of its sub-block pair
     const unsigned rd_w = r.lds + lane * 16, rd_h = r.lds + (lane >> 3) * 16;
     const int pair = (lane & 7) >> 1;
     int part = uni(start % ppr);
@@ -517,8 +564,27 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
     int po = part * 32;  // piece index in units that scale to the three strides (2048, 256, 32 bytes)
     double *out = s_part + start;
     double acc = 0.0;
+    int k = cnt;  // pieces to go
+    // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot in s_part,
+    // the run's total goes to its last piece and zero to the others (every lane stores the same word: no
+    // lane-dependent branch in the loop)
+#define FLOW_PIECE_DONE()             \
+    do {                              \
+        part++;                       \
+        po += 32;                     \
+        double v_ = 0.0;              \
+        if (k == 1 || part == ppr) {  \
+            v_ = wave_sum_f64_dpp(acc); \
+            acc = 0.0;                \
+            po = 0;                   \
+            part = 0;                 \
+        }                             \
+        *out++ = v_;                  \
+        k--;                          \
+    } while (0)
+    const int n_ring = REGS ? cnt - n_reg : cnt;
 #pragma nounroll
-    for (int k = cnt; k > 0; k--) {
+    for (int i = 0; i < n_ring; i++) {
         q.wait();
         // all LDS reads of the piece in one statement the compiler does not look into: it would otherwise hold
         // the reads of the activation area back until every asynchronous fetch into the ring had landed
@@ -547,21 +613,29 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
             acc += flow_q4_term(w, d_dmin, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
         }
 #endif
-        // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot
-        // in s_part, the run's total goes to its last piece and zero to the others
-        // (every lane stores the same word: no lane-dependent branch in the loop)
-        part++;
-        po += 32;
-        double v = 0.0;
-        if (k == 1 || part == ppr) {
-            v = wave_sum_f64_dpp(acc);
-            acc = 0.0;
-            po = 0;
-            part = 0;
-        }
-        *out++ = v;
+        FLOW_PIECE_DONE();
     }
-    q.end(r, cnt, left0 - q.left);
+    q.end(r, n_ring, left0 - q.left);
+    if (REGS) {
+#pragma unroll
+        for (int i = 0; i < FLOW_R; i++)
+            if (i < n_reg) {
+                uint4 xlo, xhi;
+                int bs_a, bs_b;
+                float yd;
+                asm volatile("ds_read_b128 %0, %5\n\tds_read_b128 %1, %5 offset:32\n\tds_read_i16 %2, %6\n\t"
+                             "ds_read_i16 %3, %6 offset:4\n\tds_read_b32 %4, %7\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&v"(xlo), "=&v"(xhi), "=&v"(bs_a), "=&v"(bs_b), "=&v"(yd)
+                             : "v"(xq0 + po * 64), "v"(xs0 + po * 8), "v"(xd0 + po)
+                             : "memory");
+                const uint4 w = make_uint4(rp.q[i].x, rp.q[i].y, rp.q[i].z, rp.q[i].w);
+                int sc_a, sc_b, m_a, m_b;
+                flow_decode_field(rp.f[i], sc_a, sc_b, m_a, m_b);
+                acc += flow_q4_term(w, rp.dm[i], sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
+                FLOW_PIECE_DONE();
+            }
+    }
+#undef FLOW_PIECE_DONE
 }
 
 // classifier pieces (q6_K): 16 super-blocks per piece, lane = (block lane/4, chunk lane%4); the ring
@@ -1138,10 +1212,14 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     r.issued = r.consumed = r.drain_mark = 0;
     r.off = 0;
     // the layers' pieces and, where the classifier is q4_K too, its pieces behind them: one stream
-    r.left = a.n_layers * (flow_wave_pieces(a.qkv, wg, wave) + flow_wave_pieces(a.wo, wg, wave) +
-                           flow_wave_pieces(a.w13, wg, wave) + flow_wave_pieces(a.w2, wg, wave)) +
-             (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces(a.cls, wg, wave) : 0);
+    const int ring_layer = flow_ring_pieces(a.qkv, wg, wave) + flow_ring_pieces(a.wo, wg, wave) +
+                           flow_ring_pieces(a.w13, wg, wave) + flow_ring_pieces(a.w2, wg, wave);
+    r.left = a.n_layers * ring_layer + (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces(a.cls, wg, wave) : 0);
     ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
+    // the register pieces follow the ring's part of the stream, in the order in which they are used
+    const unsigned char *reg_ptr = uni(r.gptr + (int64_t)a.n_layers * ring_layer * FLOW_SLOT +
+                                       (int64_t)flow_wave_pieces(a.cls, wg, wave) * (T_CLS == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT));
+    RegPieces rp;
     flow_top_up_q4(r, ring_base, lane);
 
 #ifdef L2H_TIMELINE
@@ -1199,6 +1277,9 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 #pragma nounroll
         for (int kind = 0; kind < 4; kind++) {
             bool ok;
+            const FlowGeom g = flow_geom(a, kind);
+            const int n_reg = uni(flow_reg_pieces(g, wg, wave));
+            if (kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
                 ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, 0, a.dim, nw, tok)
@@ -1211,6 +1292,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                                                     : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
                     if (!uni((int)fine)) LEAVE();
                 }
+                flow_reg_fetch(rp, reg_ptr, n_reg, lane);  // (after the attention: its loads would wait behind these)
                 FTL();
                 ok = flow_stage<PRO_QUANT, SRC_TAGGED>(a.xb, e_att, a.dim, nullptr, tok);
             } else if (kind == 2) {
@@ -1220,16 +1302,17 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             }
             if (!uni(ok)) LEAVE();
             FTL();
-            const FlowGeom g = flow_geom(a, kind);
+            reg_ptr += n_reg * FLOW_SLOT;
             // the row of x this thread adds to after wo / w2: fetched now, used after the loop
             u64 oldw = 0;
             if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = tag_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
             // what the ring holds has landed by now: after this wait the first FLOW_D pieces need none,
             // and the cache lines requested next do not stand between the loop and its pieces
             flow_drain(r);
+            flow_reg_arrived(rp);
             FTL();
             if (kind == 0 && is_att) flow_touch_cache(l, att_h, pos);
-            flow_loop_q4(g, r, ring_base, wg);
+            flow_loop_q4<true>(g, r, ring_base, wg, rp, n_reg);
             FTL();
             FTLS();
             if (kind == 0)
@@ -1259,7 +1342,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
     else
-        flow_loop_q4(a.cls, r, ring_base, wg);
+        flow_loop_q4<false>(a.cls, r, ring_base, wg, rp, 0);
     flow_finish_cls(wg, e_cls);
     flow_drain(r);
     if (wg == 0) flow_pick_token(nwg, e_cls);
@@ -1272,8 +1355,19 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 // bytes a wavefront's stream holds for one layer, and before phase `kind` within a layer
 __host__ __device__ inline int64_t flow_layer_bytes(const FlowGeom *g4, int wg, int wave, int upto) {
     int64_t b = 0;
-    for (int k = 0; k < upto; k++) b += (int64_t)flow_wave_pieces(g4[k], wg, wave) * FLOW_SLOT;
+    for (int k = 0; k < upto; k++) b += (int64_t)flow_ring_pieces(g4[k], wg, wave) * FLOW_SLOT;
     return b;
+}
+// register pieces of a wavefront in one layer, before phase `upto`
+__host__ __device__ inline int flow_layer_regs(const FlowGeom *g4, int wg, int wave, int upto) {
+    int n = 0;
+    for (int k = 0; k < upto; k++) n += flow_reg_pieces(g4[k], wg, wave);
+    return n;
+}
+// a wavefront's stream: the ring's pieces of every layer, the classifier's, then the register pieces of every layer
+__host__ __device__ inline int64_t flow_reg_base(const FlowGeom *g4, const FlowGeom &cls, int cls_piece_bytes, int n_layers,
+                                                 int wg, int wave) {
+    return (int64_t)n_layers * flow_layer_bytes(g4, wg, wave, 4) + (int64_t)flow_wave_pieces(cls, wg, wave) * cls_piece_bytes;
 }
 
 struct FlowRepackArgs {
@@ -1282,7 +1376,7 @@ struct FlowRepackArgs {
     FlowGeom g4[4];
     FlowGeom cls;
     int kind;  // 0..3 layer phases, 4 classifier
-    int layer, n_layers;
+    int layer, n_layers, cls_piece_bytes;
     DevTensor w[3];
     int dim, kv_dim, hs, neox;
 };
@@ -1305,9 +1399,18 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
     const int64_t layer_b = flow_layer_bytes(p.g4, wg, wave, 4);
     const int lane = threadIdx.x;
     if (t.type == L2H_TYPE_Q4_K) {
-        const int64_t off = p.kind == 4 ? (int64_t)p.n_layers * layer_b
-                                        : (int64_t)p.layer * layer_b + flow_layer_bytes(p.g4, wg, wave, p.kind);
-        uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + off + (int64_t)idx * FLOW_SLOT);
+        int64_t off = p.kind == 4 ? (int64_t)p.n_layers * layer_b
+                                  : (int64_t)p.layer * layer_b + flow_layer_bytes(p.g4, wg, wave, p.kind);
+        int at = idx;
+        if (p.kind < 4) {
+            const int n_ring = flow_ring_pieces(g, wg, wave);
+            if (idx >= n_ring) {
+                off = flow_reg_base(p.g4, p.cls, p.cls_piece_bytes, p.n_layers, wg, wave) +
+                      ((int64_t)p.layer * flow_layer_regs(p.g4, wg, wave, 4) + flow_layer_regs(p.g4, wg, wave, p.kind)) * FLOW_SLOT;
+                at = idx - n_ring;
+            }
+        }
+        uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + off + (int64_t)at * FLOW_SLOT);
         const int64_t blk0 = row * t.nb + part * 8;
         if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
         dst[8 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
@@ -1376,15 +1479,15 @@ int64_t k_flow_offsets(const FlowArgs &a, int cls_type, int grid, std::vector<in
     for (int wg = 0; wg < grid; wg++)
         for (int w = 0; w < FLOW_NW; w++) {
             off[(size_t)wg * FLOW_NW + w] = total;
-            total += (int64_t)a.n_layers * flow_layer_bytes(g4, wg, w, 4);
-            total += (int64_t)flow_wave_pieces(a.cls, wg, w) * (cls_type == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT);
+            total += flow_reg_base(g4, a.cls, cls_type == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT, a.n_layers, wg, w);
+            total += (int64_t)a.n_layers * flow_layer_regs(g4, wg, w, 4) * FLOW_SLOT;
             total = (total + 255) & ~(int64_t)255;
         }
     return total + 4096;  // the last fetches of a stream may be issued past a workgroup's final piece: none are, but pad anyway
 }
 
 hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream, const int64_t *wave_off_dev, int kind,
-                         int layer, const DevTensor *w, int nw, int grid) {
+                         int layer, const DevTensor *w, int nw, int grid, int cls_type) {
     FlowRepackArgs p{};
     p.stream = stream;
     p.wave_off = wave_off_dev;
@@ -1396,6 +1499,7 @@ hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream
     p.kind = kind;
     p.layer = layer;
     p.n_layers = a.n_layers;
+    p.cls_piece_bytes = cls_type == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT;
     for (int i = 0; i < nw; i++) p.w[i] = w[i];
     p.dim = a.dim;
     p.kv_dim = a.kv_dim;

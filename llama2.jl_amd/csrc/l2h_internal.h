@@ -163,7 +163,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
 int64_t k_flow_offsets(const FlowArgs &a, int cls_type, int grid, std::vector<int64_t> &off);
 // kind 0 q|k|v, 1 wo, 2 w1|w3, 3 w2 (of `layer`), 4 classifier; w: the phase's tensors
 hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream, const int64_t *wave_off_dev, int kind,
-                         int layer, const DevTensor *w, int nw, int grid);
+                         int layer, const DevTensor *w, int nw, int grid, int cls_type);
 hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a);
 hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid);
 
