@@ -249,10 +249,42 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
 // epoch `epoch`, or (EMB) the embedding row of `tok`.  Returns false if the wait gave up.
 // Separate functions (not inlined): the kernel stays small enough to keep its state in registers.
 // ------------------------------------------------------------------------------------------
+// Polls of activation words.  A lane's four words are one contiguous, 16-byte aligned run: fetched with
+// 16-byte loads (agent scope; every aligned 4- or 8-byte word of such a load is read whole), so that one
+// instruction asks for whole cache lines.  The loads and the wait for them are ONE asm statement: the
+// compiler believes an asm's outputs valid as soon as the statement ends and may copy them at once, so no
+// statement may end with a load still under way.
+#define POLL_TAGGED(lo, hi, p)                                                                                           \
+    asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)" \
+                 : "+v"(lo), "+v"(hi)                                                                                    \
+                 : "v"(p)                                                                                                \
+                 : "memory")
+#define POLL_BARE1(w0, p0) \
+    asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "+v"(w0) : "v"(p0) : "memory")
+#define POLL_BARE2(w0, w1, p0, p1)                                                                                    \
+    asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %3, off sc1\n\ts_waitcnt vmcnt(0)" \
+                 : "+v"(w0), "+v"(w1)                                                                                 \
+                 : "v"(p0), "v"(p1)                                                                                   \
+                 : "memory")
+#define POLL_BARE3(w0, w1, w2, p0, p1, p2)                                                                 \
+    asm volatile("global_load_dwordx4 %0, %3, off sc1\n\tglobal_load_dwordx4 %1, %4, off sc1\n\t"         \
+                 "global_load_dwordx4 %2, %5, off sc1\n\ts_waitcnt vmcnt(0)"                               \
+                 : "+v"(w0), "+v"(w1), "+v"(w2)                                                            \
+                 : "v"(p0), "v"(p1), "v"(p2)                                                               \
+                 : "memory")
+#define POLL_BARE4(w0, w1, w2, w3, p0, p1, p2, p3)                                                         \
+    asm volatile("global_load_dwordx4 %0, %4, off sc1\n\tglobal_load_dwordx4 %1, %5, off sc1\n\t"         \
+                 "global_load_dwordx4 %2, %6, off sc1\n\tglobal_load_dwordx4 %3, %7, off sc1\n\ts_waitcnt vmcnt(0)" \
+                 : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3)                                                  \
+                 : "v"(p0), "v"(p1), "v"(p2), "v"(p3)                                                      \
+                 : "memory")
+
 // SRC: where the input comes from
 #define SRC_EMB 0     // the embedding row of `tok`
 #define SRC_TAGGED 1  // {fp32, epoch} words; a word is there when it carries `epoch`
 #define SRC_BARE 2    // fp32 words; a word is there when it is not FLOW_EMPTY
+// Tagged words, the embedding and norm weights come with vectors of dim <= 4096 only (one q8_K block per
+// wavefront); the bare words of the hidden vector take up to four rounds.
 template <int PRO, int SRC>
 __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, const float *normw, int tok) {
     src = uni(src), epoch = uni(epoch), K = uni(K), normw = uni(normw), tok = uni(tok);
@@ -262,119 +294,89 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
     float *s_d = (float *)(s_qs + 14336 + 1792);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nb = K >> 8;
-    float xv[STAGE_MAX_ROUNDS][4];
-    float wv[STAGE_MAX_ROUNDS][4];
+    static_assert(STAGE_MAX_ROUNDS == 4, "four rounds below");
+    const int rounds = nb > wave ? (nb - wave + FLOW_NW - 1) / FLOW_NW : 0;  // q8_K blocks of this wavefront
+    constexpr bool rms = PRO == PRO_RMSNORM, bare = SRC == SRC_BARE;
+    float xv[4][4];
+    float wv0[4];
     bool ok = true;
     // the norm weights are requested before the wait for the input: their latency passes meanwhile
-    if (PRO == PRO_RMSNORM) {
-#pragma unroll
-        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            const int b = wave + r * FLOW_NW;
-            if (b < nb) {
-                const float4 t = *(const float4 *)(normw + 256 * b + 4 * lane);
-                wv[r][0] = t.x;
-                wv[r][1] = t.y;
-                wv[r][2] = t.z;
-                wv[r][3] = t.w;
-            }
-        }
+    if (rms && rounds > 0) {
+        const float4 t = *(const float4 *)(normw + 256 * wave + 4 * lane);
+        wv0[0] = t.x;
+        wv0[1] = t.y;
+        wv0[2] = t.z;
+        wv0[3] = t.w;
     }
     if (SRC == SRC_EMB) {
+        if (rounds > 0)
 #pragma unroll
-        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            const int b = wave + r * FLOW_NW;
-            if (b < nb)
-#pragma unroll
-                for (int k = 0; k < 4; k++) xv[r][k] = dequant_elem(a.emb, tok, 256 * b + 4 * lane + k);
-        }
+            for (int k = 0; k < 4; k++) xv[0][k] = dequant_elem(a.emb, tok, 256 * wave + 4 * lane + k);
     } else {
-        // A lane's four words are one contiguous, 16-byte aligned run: fetched with 16-byte loads (agent
-        // scope; every aligned 4- or 8-byte word of such a load is read whole), so that one instruction
-        // asks for whole cache lines.  First pass: every lane; later passes: the lanes that miss a word.
         unsigned spins = 0;
-        // (the loads name their target registers as read-write operands: the data lands in the registers that
-        // already stand for the words, with no copy in between that could run before it has arrived)
-        u32x4v wl[STAGE_MAX_ROUNDS], wh[STAGE_MAX_ROUNDS];  // tagged: words 0,1 | 2,3; bare: wl only
-#define STAGE_FETCH(r)                                                                                                 \
-    do {                                                                                                               \
-        if (SRC == SRC_TAGGED) {                                                                                       \
-            const u64 *p_ = (const u64 *)src + 256 * (wave + (r)*FLOW_NW) + 4 * lane;                                   \
-            asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1"         \
-                         : "+v"(wl[r]), "+v"(wh[r])                                                                    \
-                         : "v"(p_)                                                                                     \
-                         : "memory");                                                                                  \
-        } else {                                                                                                       \
-            const unsigned *p_ = (const unsigned *)src + 256 * (wave + (r)*FLOW_NW) + 4 * lane;                         \
-            asm volatile("global_load_dwordx4 %0, %1, off sc1" : "+v"(wl[r]) : "v"(p_) : "memory");                    \
-        }                                                                                                              \
-    } while (0)
-// the loads above have returned; naming their registers keeps every use behind this point
-#define STAGE_ARRIVED()                                                                                                \
-    do {                                                                                                               \
-        static_assert(STAGE_MAX_ROUNDS == 4, "operand list below");                                                    \
-        if (SRC == SRC_TAGGED)                                                                                         \
-            asm volatile("s_waitcnt vmcnt(0)"                                                                          \
-                         : "+v"(wl[0]), "+v"(wl[1]), "+v"(wl[2]), "+v"(wl[3]), "+v"(wh[0]), "+v"(wh[1]), "+v"(wh[2]),  \
-                           "+v"(wh[3])                                                                                 \
-                         :                                                                                             \
-                         : "memory");                                                                                  \
-        else                                                                                                           \
-            asm volatile("s_waitcnt vmcnt(0)" : "+v"(wl[0]), "+v"(wl[1]), "+v"(wl[2]), "+v"(wl[3]) : : "memory");      \
-    } while (0)
-#define STAGE_COMPLETE(r)                                                                                          \
-    (SRC == SRC_TAGGED ? (wl[r].y == epoch && wl[r].w == epoch && wh[r].y == epoch && wh[r].w == epoch)            \
-                       : (wl[r].x != FLOW_EMPTY && wl[r].y != FLOW_EMPTY && wl[r].z != FLOW_EMPTY && wl[r].w != FLOW_EMPTY))
-#pragma unroll
-        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            wl[r] = (u32x4v){0, 0, 0, 0};
-            wh[r] = (u32x4v){0, 0, 0, 0};
-            if (wave + r * FLOW_NW < nb) STAGE_FETCH(r);
-        }
-        STAGE_ARRIVED();
+        // tagged: words 0,1 in w0, 2,3 in wh; bare: round r in w<r>; all start as "not there"
+        const unsigned none = bare ? FLOW_EMPTY : 0u;  // (epochs are never 0)
+        u32x4v w0 = {none, none, none, none}, w1 = w0, w2 = w0, w3 = w0, wh = w0;
+        const u64 *pt = (const u64 *)src + 256 * wave + 4 * lane;
+        const unsigned *pb = (const unsigned *)src + 256 * wave + 4 * lane;
         for (;;) {
             bool all = true;
-#pragma unroll
-            for (int r = 0; r < STAGE_MAX_ROUNDS; r++)
-                if (wave + r * FLOW_NW < nb) all = all && STAGE_COMPLETE(r);
+            if (rounds > 0) {
+                // (a lane that has all its words does not ask again: waiting for a slow producer costs little traffic)
+                if (!bare) {
+                    all = w0.y == epoch && w0.w == epoch && wh.y == epoch && wh.w == epoch;
+                    if (!all) {
+                        POLL_TAGGED(w0, wh, pt);
+                        all = w0.y == epoch && w0.w == epoch && wh.y == epoch && wh.w == epoch;
+                    }
+                } else {
+#define FULL(V_) (V_.x != FLOW_EMPTY && V_.y != FLOW_EMPTY && V_.z != FLOW_EMPTY && V_.w != FLOW_EMPTY)
+                    if (rounds == 1) {
+                        if (!FULL(w0)) POLL_BARE1(w0, pb);
+                        all = FULL(w0);
+                    } else if (rounds == 2) {
+                        if (!(FULL(w0) && FULL(w1))) POLL_BARE2(w0, w1, pb, pb + 256 * FLOW_NW);
+                        all = FULL(w0) && FULL(w1);
+                    } else if (rounds == 3) {
+                        if (!(FULL(w0) && FULL(w1) && FULL(w2))) POLL_BARE3(w0, w1, w2, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW);
+                        all = FULL(w0) && FULL(w1) && FULL(w2);
+                    } else {
+                        if (!(FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3)))
+                            POLL_BARE4(w0, w1, w2, w3, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW, pb + 768 * FLOW_NW);
+                        all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
+                    }
+#undef FULL
+                }
+            }
             if (__ballot(!all) == 0ull) break;
             if (++spins > a.spin_limit ||
                 ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
                 ok = false;
                 break;
             }
-#pragma unroll
-            for (int r = 0; r < STAGE_MAX_ROUNDS; r++)
-                if (wave + r * FLOW_NW < nb && !STAGE_COMPLETE(r)) STAGE_FETCH(r);
-            STAGE_ARRIVED();
         }
-#undef STAGE_FETCH
-#undef STAGE_ARRIVED
-#undef STAGE_COMPLETE
+        if (!bare) {
+            xv[0][0] = __uint_as_float(w0.x);
+            xv[0][1] = __uint_as_float(w0.z);
+            xv[0][2] = __uint_as_float(wh.x);
+            xv[0][3] = __uint_as_float(wh.z);
+        } else {
+            const u32x4v ws[4] = {w0, w1, w2, w3};
 #pragma unroll
-        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            if (SRC == SRC_TAGGED) {
-                xv[r][0] = __uint_as_float(wl[r].x);
-                xv[r][1] = __uint_as_float(wl[r].z);
-                xv[r][2] = __uint_as_float(wh[r].x);
-                xv[r][3] = __uint_as_float(wh[r].z);
-            } else {
-                xv[r][0] = __uint_as_float(wl[r].x);
-                xv[r][1] = __uint_as_float(wl[r].y);
-                xv[r][2] = __uint_as_float(wl[r].z);
-                xv[r][3] = __uint_as_float(wl[r].w);
+            for (int r = 0; r < 4; r++) {
+                xv[r][0] = __uint_as_float(ws[r].x);
+                xv[r][1] = __uint_as_float(ws[r].y);
+                xv[r][2] = __uint_as_float(ws[r].z);
+                xv[r][3] = __uint_as_float(ws[r].w);
             }
         }
     }
     if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
-    double acc = 0.0;
-    if (PRO == PRO_RMSNORM) {  // rmsnorm! (reference src/inference.jl:102-110)
+    if (rms) {  // rmsnorm! (reference src/inference.jl:102-110)
+        double acc = 0.0;
+        if (rounds > 0) {
 #pragma unroll
-        for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
-            const int b = wave + r * FLOW_NW;
-            if (b < nb) {
-#pragma unroll
-                for (int k = 0; k < 4; k++) acc = fma((double)xv[r][k], (double)xv[r][k], acc);
-            }
+            for (int k = 0; k < 4; k++) acc = fma((double)xv[0][k], (double)xv[0][k], acc);
         }
         acc = wave_sum_f64_dpp(acc);
         if (lane == 0) s_red[wave] = acc;
@@ -384,26 +386,24 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
         if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return false;
     }
-    float ss = 1.0f;
-    if (PRO == PRO_RMSNORM) {
+    if (rms) {
         double t = 0.0;
         for (int w = 0; w < FLOW_NW; w++) t += s_red[w];
-        ss = (float)t;
+        float ss = (float)t;
         ss /= (float)K;
         ss += 1e-5f;
         ss = 1.0f / sqrtf(ss);
+#pragma unroll
+        for (int k = 0; k < 4; k++) xv[0][k] = wv0[k] * (ss * xv[0][k]);
     }
 #pragma unroll
-    for (int r = 0; r < STAGE_MAX_ROUNDS; r++) {
+    for (int r = 0; r < 4; r++) {
         const int b = wave + r * FLOW_NW;
-        if (b < nb) {
-            float v[4];
-#pragma unroll
-            for (int k = 0; k < 4; k++) v[k] = PRO == PRO_RMSNORM ? wv[r][k] * (ss * xv[r][k]) : xv[r][k];
+        if (r < rounds && (bare || r == 0)) {
             uint32_t packed;
             int bsum;
             float d;
-            q8k_quantize_wave(v, packed, bsum, d);
+            q8k_quantize_wave(xv[r], packed, bsum, d);
             ((uint32_t *)s_qs)[64 * b + lane] = packed;
             if ((lane & 3) == 0) s_bs[16 * b + (lane >> 2)] = (int16_t)bsum;
             if (lane == 0) s_d[b] = d;
@@ -1454,7 +1454,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     if (cls_type != L2H_TYPE_Q4_K && cls_type != L2H_TYPE_Q6_K) return no("classifier must be q4_K or q6_K");
     if (a.dim % 2048 != 0 || a.hidden % 2048 != 0) return no("dim and hidden_dim must be multiples of 2048");
     if (cls_type == L2H_TYPE_Q6_K && a.dim % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
-    if (a.hidden > 14336 || a.dim > 14336) return no("input vectors longer than 14336");
+    if (a.hidden > 14336 || a.dim > 4096) return no("dim above 4096 or hidden_dim above 14336");
     if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 128)) return no("head size must be 32, 64 or 128");
     const size_t att = (size_t)a.hs * 8 + (size_t)((a.seq_len + 1) & ~1) * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 +
                        (size_t)((a.seq_len + 3) & ~3) * 4 + (size_t)a.hs * 8;
