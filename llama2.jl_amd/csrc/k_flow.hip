@@ -541,7 +541,10 @@ __device__ __forceinline__ void flow_reg_arrived(RegPieces &rp) {
 }
 
 // REGS: the wavefront's last n_reg pieces are in rp, the ones before them come through the ring
-template <bool REGS>
+// QUARTERS: a row's sum is left as the four sums of 16 lanes each (s_part holds four doubles per piece)
+// for flow_row_values to add, in the order in which wave_sum_f64_dpp would have: the loop is shorter by
+// the lane reads and additions; the classifier has too many pieces per workgroup for that layout
+template <bool REGS, bool QUARTERS>
 __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg, const RegPieces &rp,
                                              int n_reg) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -562,7 +565,7 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
     const unsigned xs0 = act + 14336 + 2 * ((lane >> 3) * 16 + 4 * (c8 >> 1) + (c8 & 1));
     const unsigned xd0 = act + 14336 + 1792 + 4 * (lane >> 3);
     int po = part * 32;  // piece index in units that scale to the three strides (2048, 256, 32 bytes)
-    double *out = s_part + start;
+    double *out = QUARTERS ? s_part + 4 * start + (lane >> 4) : s_part + start;
     double acc = 0.0;
     int k = cnt;  // pieces to go
     // a row's consecutive pieces are reduced over the lanes once; every piece has its own slot in s_part,
@@ -574,12 +577,13 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
         po += 32;                     \
         double v_ = 0.0;              \
         if (k == 1 || part == ppr) {  \
-            v_ = wave_sum_f64_dpp(acc); \
+            v_ = QUARTERS ? row16_sum_f64_dpp(acc) : wave_sum_f64_dpp(acc); \
             acc = 0.0;                \
             po = 0;                   \
             part = 0;                 \
         }                             \
-        *out++ = v_;                  \
+        *out = v_;                    \
+        out += QUARTERS ? 4 : 1;      \
         k--;                          \
     } while (0)
     const int n_ring = REGS ? cnt - n_reg : cnt;
@@ -710,11 +714,19 @@ __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigne
 }
 
 // fp32 value of every local row: the pieces' partial sums added in order
+template <bool QUARTERS>
 __device__ __forceinline__ void flow_row_values(int n_local, int ppr) {
     __syncthreads();
     for (int lr = threadIdx.x; lr < n_local; lr += blockDim.x) {
         double v = 0.0;
-        for (int p = 0; p < ppr; p++) v += s_part[lr * ppr + p];
+        for (int p = 0; p < ppr; p++) {
+            if (QUARTERS) {
+                const double *q4 = s_part + 4 * (lr * ppr + p);
+                v += (q4[0] + q4[1]) + (q4[2] + q4[3]);
+            } else {
+                v += s_part[lr * ppr + p];
+            }
+        }
         s_val[lr] = (float)v;
     }
     __syncthreads();
@@ -726,7 +738,7 @@ __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_
     l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.qkv, wg), tid = threadIdx.x;
-    flow_row_values(n_local, a.qkv.ppr);
+    flow_row_values<true>(n_local, a.qkv.ppr);
     if (tid >= n_local) return;
     const int L = wg * a.qkv.rpw + tid;
     int seg, row;
@@ -762,7 +774,7 @@ __device__ __noinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsi
     const u64 *src = which == 1 ? a.x_a : a.x_b;
     u64 *dst = which == 1 ? a.x_b : a.x_a;
     const int n_local = flow_n_local(g, wg), tid = threadIdx.x;
-    flow_row_values(n_local, g.ppr);
+    flow_row_values<true>(n_local, g.ppr);
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
     const float old = tag_is(oldw, e_src) ? tag_val(oldw) : flow_read(src + row, e_src);
@@ -774,7 +786,7 @@ __device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
     wg = uni(wg), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.w13, wg), tid = threadIdx.x;
-    flow_row_values(n_local, a.w13.ppr);
+    flow_row_values<true>(n_local, a.w13.ppr);
     if (tid >= n_local || (tid & 1)) return;
     const int64_t u = ((int64_t)wg * a.w13.rpw + tid) >> 1;
     unsigned v = __float_as_uint(swiglu_val(s_val[tid], s_val[tid + 1]));
@@ -790,7 +802,7 @@ __device__ __noinline__ void flow_finish_cls(int wg, unsigned e_cls) {
     wg = uni(wg), e_cls = uni(e_cls);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.cls, wg), tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    flow_row_values(n_local, a.cls.ppr);
+    flow_row_values<false>(n_local, a.cls.ppr);
     unsigned long long best = 0;
     if (tid < n_local) {
         const int64_t row = (int64_t)wg * a.cls.rpw + tid;
@@ -1312,7 +1324,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             flow_reg_arrived(rp);
             FTL();
             if (kind == 0 && is_att) flow_touch_cache(l, att_h, pos);
-            flow_loop_q4<true>(g, r, ring_base, wg, rp, n_reg);
+            flow_loop_q4<true, true>(g, r, ring_base, wg, rp, n_reg);
             FTL();
             FTLS();
             if (kind == 0)
@@ -1342,7 +1354,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
     else
-        flow_loop_q4<false>(a.cls, r, ring_base, wg, rp, 0);
+        flow_loop_q4<false, false>(a.cls, r, ring_base, wg, rp, 0);
     flow_finish_cls(wg, e_cls);
     flow_drain(r);
     if (wg == 0) flow_pick_token(nwg, e_cls);
@@ -1466,7 +1478,8 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     a.cls = make_geom(a.vocab, a.dim, cls_type, grid);
     const FlowGeom *gs[5] = {&a.qkv, &a.wo, &a.w13, &a.w2, &a.cls};
     for (const FlowGeom *g : gs)
-        if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > FLOW_MAX_PIECES) return no("too many rows per workgroup");
+        if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
+            return no("too many rows per workgroup");  // (layer phases keep four partial sums per piece)
     if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
     return true;
 }

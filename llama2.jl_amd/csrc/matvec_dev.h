@@ -342,6 +342,14 @@ __device__ __forceinline__ double wave_sum_f64_dpp(double v) {
     v += dpp_f64<DPP_ROW_MIRROR>(v);
     return (readlane_f64(v, 0) + readlane_f64(v, 16)) + (readlane_f64(v, 32) + readlane_f64(v, 48));
 }
+// the first four steps of wave_sum_f64_dpp: every lane ends with the sum of its row of 16 lanes
+__device__ __forceinline__ double row16_sum_f64_dpp(double v) {
+    v += dpp_f64<DPP_QUAD_SWAP1>(v);
+    v += dpp_f64<DPP_QUAD_SWAP2>(v);
+    v += dpp_f64<DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f64<DPP_ROW_MIRROR>(v);
+    return v;
+}
 __device__ __forceinline__ float wave_max_f32_dpp(float v) {
     v = fmaxf(v, dpp_f32<DPP_QUAD_SWAP1>(v));
     v = fmaxf(v, dpp_f32<DPP_QUAD_SWAP2>(v));
