@@ -732,18 +732,28 @@ __device__ __forceinline__ void flow_row_values(int n_local, int ppr) {
     __syncthreads();
 }
 
+// the same for one row, straight from the partial sums (the layer epilogues: one barrier instead of two)
+__device__ __forceinline__ float flow_row_value4(int lr, int ppr) {
+    double v = 0.0;
+    for (int p = 0; p < ppr; p++) {
+        const double *q4 = s_part + 4 * (lr * ppr + p);
+        v += (q4[0] + q4[1]) + (q4[2] + q4[3]);
+    }
+    return (float)v;
+}
+
 // ---- epilogues -------------------------------------------------------------------------------
 // rope! (reference src/inference.jl:112-157) and the cache append (:259-260)
 __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
     l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.qkv, wg), tid = threadIdx.x;
-    flow_row_values<true>(n_local, a.qkv.ppr);
+    __syncthreads();
     if (tid >= n_local) return;
     const int L = wg * a.qkv.rpw + tid;
     int seg, row;
     flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
-    const float val = s_val[tid], other = s_val[tid ^ 1];
+    const float val = flow_row_value4(tid, a.qkv.ppr), other = flow_row_value4(tid ^ 1, a.qkv.ppr);
     const int hh = row / a.hs, e = row % a.hs;
     if (seg == 2) {
         (a.vc + (int64_t)l * a.cache_layer_elems)[((int64_t)hh * a.seq_len + pos) * a.hs + e] = val;
@@ -774,11 +784,11 @@ __device__ __noinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsi
     const u64 *src = which == 1 ? a.x_a : a.x_b;
     u64 *dst = which == 1 ? a.x_b : a.x_a;
     const int n_local = flow_n_local(g, wg), tid = threadIdx.x;
-    flow_row_values<true>(n_local, g.ppr);
+    __syncthreads();
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
     const float old = tag_is(oldw, e_src) ? tag_val(oldw) : flow_read(src + row, e_src);
-    tag_store(dst + row, old + s_val[tid], e_dst);
+    tag_store(dst + row, old + flow_row_value4(tid, g.ppr), e_dst);
 }
 
 // SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u
@@ -786,10 +796,10 @@ __device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
     wg = uni(wg), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.w13, wg), tid = threadIdx.x;
-    flow_row_values<true>(n_local, a.w13.ppr);
+    __syncthreads();
     if (tid >= n_local || (tid & 1)) return;
     const int64_t u = ((int64_t)wg * a.w13.rpw + tid) >> 1;
-    unsigned v = __float_as_uint(swiglu_val(s_val[tid], s_val[tid + 1]));
+    unsigned v = __float_as_uint(swiglu_val(flow_row_value4(tid, a.w13.ppr), flow_row_value4(tid + 1, a.w13.ppr)));
     if (v == FLOW_EMPTY) v = 0x7FC00000u;
     unsigned *mine = a.hbw + (int64_t)(e_out & 1u) * a.hidden, *other = a.hbw + (int64_t)((e_out & 1u) ^ 1u) * a.hidden;
     bare_store(mine + u, v);
