@@ -126,8 +126,8 @@ __host__ __device__ inline void flow_row_src(int kind, int L, int dim, int kv_di
     seg = L < dim ? 0 : (L < dim + kv_dim ? 1 : 2);
     row = L - (seg == 0 ? 0 : (seg == 1 ? dim : dim + kv_dim));
     if (neox && seg != 2) {  // neox pairs element i with i + hs/2 (reference src/inference.jl:146)
-        const int h = row / hs, e = row % hs;
-        row = h * hs + (e >> 1) + ((e & 1) ? (hs >> 1) : 0);
+        const int e = row & (hs - 1);  // hs is a power of two (32, 64 or 128)
+        row = (row - e) + (e >> 1) + ((e & 1) ? (hs >> 1) : 0);
     }
 }
 
@@ -754,14 +754,15 @@ __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_
     int seg, row;
     flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
     const float val = flow_row_value4(tid, a.qkv.ppr), other = flow_row_value4(tid ^ 1, a.qkv.ppr);
-    const int hh = row / a.hs, e = row % a.hs;
+    const int hs_log = 31 - __builtin_clz(a.hs);  // a power of two
+    const int hh = row >> hs_log, e = row & (a.hs - 1);
     if (seg == 2) {
         (a.vc + (int64_t)l * a.cache_layer_elems)[((int64_t)hh * a.seq_len + pos) * a.hs + e] = val;
         tag_store(a.vcur + row, val, e_q);
         return;
     }
     const int half = a.hs >> 1;
-    const int i = a.neox ? (e % half) : (e >> 1);
+    const int i = a.neox ? (e & (half - 1)) : (e >> 1);
     const float c = s_rope[2 * i], s = s_rope[2 * i + 1];
     const int rr = tid & 1;
     // complex product (re + i im)(c + i s), each of the four products rounded
