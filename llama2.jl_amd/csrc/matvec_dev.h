@@ -385,17 +385,13 @@ __device__ __forceinline__ void q8k_quantize_wave(const float v[4], uint32_t &pa
         }
     }
     const float wmax = wave_max_f32_dpp(amax);
-    if (wmax == 0.0f) {
-        packed = 0;
-        bsum16 = 0;
-        d = 0.0f;
-        return;
-    }
     // lowest lane whose own extreme reaches the block's: its first such element is the block's first
     const unsigned long long holders = __ballot(amax == wmax);
     const int first = __builtin_ctzll(holders);
     const float bmx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx), first));
-    const float iscale = -127.0f / bmx;
+    // an all-zero block gives q = 0, d = 0 (no branch: several blocks' code can then be interleaved)
+    const bool zero = wmax == 0.0f;
+    const float iscale = zero ? 0.0f : -127.0f / bmx;
     uint32_t word = 0;
     int sum = 0;
 #pragma unroll
@@ -407,7 +403,7 @@ __device__ __forceinline__ void q8k_quantize_wave(const float v[4], uint32_t &pa
     }
     packed = word;
     bsum16 = quad_sum_i32(sum);
-    d = 1.0f / iscale;
+    d = zero ? 0.0f : 1.0f / iscale;
 }
 
 #define STAGE_MAX_ROUNDS 4  // q8_K blocks per wavefront: K <= 4 * 16 * 256
