@@ -1,0 +1,66 @@
+"""The streaming kernel polls activations with loads it issues from inline asm.  The compiler believes
+an asm statement's outputs valid as soon as the statement ends, so a load and the wait for it must be
+one statement; this test compiles k_flow.hip to assembly and checks that no register that such a load
+targets is read or written before the wait that follows it."""
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "llama2.jl_amd", "csrc")
+
+
+def _regs(text):
+    out = set()
+    for m in re.finditer(r"v\[(\d+):(\d+)\]", text):
+        out.update(range(int(m.group(1)), int(m.group(2)) + 1))
+    for m in re.finditer(r"(?<![\w\[])v(\d+)\b", text):
+        out.add(int(m.group(1)))
+    return out
+
+
+def _violations(path):
+    """Linear scan: registers written by the asm-issued coherent 16-byte loads (`... sc1`) stay untouched
+    until an asm-issued s_waitcnt vmcnt."""
+    bad, fn, pending, in_asm, n_loads = [], None, {}, False, 0
+    for ln, line in enumerate(open(path), 1):
+        t = line.strip()
+        m = re.match(r"^(_Z\w+):", t)
+        if m:
+            fn, pending = m.group(1), {}
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if not t or t[0] in ";.":
+            continue
+        if in_asm and "s_waitcnt vmcnt" in t:
+            pending = {}
+            continue
+        if in_asm and t.startswith("global_load_dwordx4") and t.endswith("sc1"):
+            n_loads += 1
+            for r in _regs(t.split(",")[0]):
+                pending[r] = ln
+            continue
+        hit = _regs(t) & set(pending)
+        if hit:
+            bad.append((fn, ln, t, sorted(hit)))
+    return bad, n_loads
+
+
+@pytest.mark.skipif(shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"), reason="no hipcc")
+def test_no_register_of_a_pending_poll_is_touched(tmp_path):
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    out = tmp_path / "k_flow.s"
+    cmd = [hipcc, "-S", "--cuda-device-only", os.path.join(CSRC, "k_flow.hip"), "-o", str(out), "--offload-arch=gfx950", "-O3",
+           "-std=c++17", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I", os.path.join(ROOT, "include"), "-I", CSRC]
+    subprocess.run(cmd, check=True, capture_output=True, timeout=600)
+    bad, n_loads = _violations(str(out))
+    assert n_loads > 0, "no asm-issued polls found: has the kernel changed?"
+    assert not bad, bad[:5]
