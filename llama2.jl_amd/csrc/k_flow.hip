@@ -743,8 +743,11 @@ __device__ __forceinline__ float flow_row_value4(int lr, int ppr) {
 }
 
 // ---- epilogues -------------------------------------------------------------------------------
+// (The layer epilogues are inlined: a function waits before it returns for its stores to be acknowledged,
+// a round trip to memory that would stand between the publication of a phase's results and the next
+// phase's requests.)
 // rope! (reference src/inference.jl:112-157) and the cache append (:259-260)
-__device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
+__device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
     l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.qkv, wg), tid = threadIdx.x;
@@ -778,7 +781,7 @@ __device__ __noinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_
 
 // dst = old + result (x .+= ..., :284,305); which = 1 after wo (-> x_b), 3 after w2 (-> x_a); `old` is
 // this thread's row of the other buffer, fetched before the loop
-__device__ __noinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsigned e_src, unsigned e_dst) {
+__device__ __forceinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsigned e_src, unsigned e_dst) {
     which = uni(which), wg = uni(wg), e_src = uni(e_src), e_dst = uni(e_dst);
     const FlowArgs &a = c_flow;
     const FlowGeom &g = which == 1 ? a.wo : a.w2;
