@@ -686,7 +686,10 @@ static int flow_setup(l2h_model *m) {
         return rc;
     TA(a.x_a, c.dim);
     TA(a.x_b, c.dim);
-    TA(a.xb, c.dim);
+    TA(a.xo, 2 * (int64_t)c.dim);
+    HIPCHK(ctx, hipMemset(a.x_a, 0xFF, (size_t)c.dim * 4));
+    HIPCHK(ctx, hipMemset(a.x_b, 0xFF, (size_t)c.dim * 4));
+    HIPCHK(ctx, hipMemset(a.xo, 0xFF, 2 * (size_t)c.dim * 4));
     TA(a.q, c.dim);
     TA(a.kcur, m->kv_dim);
     TA(a.vcur, m->kv_dim);
@@ -866,7 +869,11 @@ static int mega_check(l2h_model *m) {
         HIPCHK(m->ctx, hipMemcpy(&ab, m->flow_args.abort_flag, 4, hipMemcpyDeviceToHost));
         if (!ab) return L2H_OK;
         HIPCHK(m->ctx, hipMemset(m->flow_args.abort_flag, 0, 4));
-        HIPCHK(m->ctx, hipMemset(m->flow_args.hbw, 0xFF, 2 * (size_t)m->c.hidden_dim * 4));  // all words "not written"
+        // all words "not written"
+        HIPCHK(m->ctx, hipMemset(m->flow_args.hbw, 0xFF, 2 * (size_t)m->c.hidden_dim * 4));
+        HIPCHK(m->ctx, hipMemset(m->flow_args.x_a, 0xFF, (size_t)m->c.dim * 4));
+        HIPCHK(m->ctx, hipMemset(m->flow_args.x_b, 0xFF, (size_t)m->c.dim * 4));
+        HIPCHK(m->ctx, hipMemset(m->flow_args.xo, 0xFF, 2 * (size_t)m->c.dim * 4));
         return set_err(m->ctx, L2H_EHIP, "streaming decode kernel: a wait for activations timed out");
     }
     if (!m->mega) return L2H_OK;

@@ -61,18 +61,31 @@ __device__ __forceinline__ u64 tag_load(const u64 *p) {
 }
 __device__ __forceinline__ bool tag_is(u64 w, unsigned epoch) { return (unsigned)(w >> 32) == epoch; }
 __device__ __forceinline__ float tag_val(u64 w) { return __uint_as_float((unsigned)w); }
-// The SwiGLU outputs, the largest vector that all workgroups exchange, travel as bare fp32 words, half
-// the bytes of tagged ones.  A word that has not been written holds FLOW_EMPTY, a NaN pattern that no
-// arithmetic here produces (a result that happens to have it is stored as the default NaN).  There are
-// two buffers; the phase with epoch e uses buffer e & 1 (consecutive layers, and the last layer of one
-// launch and the first of the next, differ in that bit), and whoever writes word i of one buffer puts
-// FLOW_EMPTY back into word i of the other: every reader of that one finished with it a phase ago.
+// The vectors that every workgroup reads whole — the residual stream x, the attention output, the SwiGLU
+// output — travel as bare fp32 words, half the bytes of tagged ones.  A word that has not been written
+// holds FLOW_EMPTY, a NaN pattern that no arithmetic here produces (a result that happens to have it is
+// stored as the default NaN).  Each comes in two buffers used in turn (x: layer input / after attention;
+// the others: by the low bit of the phase's epoch, which consecutive layers, and the last layer of one
+// launch and the first of the next, differ in), and whoever writes word i of one buffer puts FLOW_EMPTY
+// back into word i of the other: every reader of that one finished with it a phase ago, and it is the
+// same thread that writes word i of either.
 #define FLOW_EMPTY 0xFFFFFFFFu
 __device__ __forceinline__ unsigned bare_load(const unsigned *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ void bare_store(unsigned *p, unsigned v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// the word that stands for v
+__device__ __forceinline__ unsigned bare_of(float v) {
+    const unsigned u = __float_as_uint(v);
+    return u == FLOW_EMPTY ? 0x7FC00000u : u;
+}
+// one bare word, waited for (the caller has usually seen it already)
+__device__ __forceinline__ float bare_read(const unsigned *p, unsigned seen) {
+    unsigned w = seen, spins = 0;
+    while (w == FLOW_EMPTY && ++spins <= c_flow.spin_limit) w = bare_load(p);
+    return __uint_as_float(w);
 }
 
 __host__ __device__ inline int flow_n_local(const FlowGeom &g, int wg) {
@@ -411,14 +424,6 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
     }
     __syncthreads();
     return true;
-}
-
-// one tagged word, waited for (the caller has usually seen it already)
-__device__ __forceinline__ float flow_read(const u64 *p, unsigned epoch) {
-    u64 w = tag_load(p);
-    unsigned spins = 0;
-    while (!tag_is(w, epoch) && ++spins <= c_flow.spin_limit) w = tag_load(p);
-    return tag_val(w);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -780,19 +785,20 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
 }
 
 // dst = old + result (x .+= ..., :284,305); which = 1 after wo (-> x_b), 3 after w2 (-> x_a); `old` is
-// this thread's row of the other buffer, fetched before the loop
-__device__ __forceinline__ void flow_finish_resid(int which, int wg, u64 oldw, unsigned e_src, unsigned e_dst) {
-    which = uni(which), wg = uni(wg), e_src = uni(e_src), e_dst = uni(e_dst);
+// this thread's row of the other buffer, fetched before the loop (the same thread wrote it)
+__device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned oldw) {
+    which = uni(which), wg = uni(wg);
     const FlowArgs &a = c_flow;
     const FlowGeom &g = which == 1 ? a.wo : a.w2;
-    const u64 *src = which == 1 ? a.x_a : a.x_b;
-    u64 *dst = which == 1 ? a.x_b : a.x_a;
+    unsigned *src = which == 1 ? a.x_a : a.x_b;
+    unsigned *dst = which == 1 ? a.x_b : a.x_a;
     const int n_local = flow_n_local(g, wg), tid = threadIdx.x;
     __syncthreads();
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
-    const float old = tag_is(oldw, e_src) ? tag_val(oldw) : flow_read(src + row, e_src);
-    tag_store(dst + row, old + flow_row_value4(tid, g.ppr), e_dst);
+    const float old = bare_read(src + row, oldw);
+    bare_store(dst + row, bare_of(old + flow_row_value4(tid, g.ppr)));
+    bare_store(src + row, FLOW_EMPTY);  // (its readers are through: see FLOW_EMPTY)
 }
 
 // SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u
@@ -1075,7 +1081,8 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
         double acc = 0.0;
 #pragma unroll
         for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
-        tag_store(a.xb + (int64_t)h * hs + tid, (float)acc, e_out);
+        bare_store(a.xo + (int64_t)(e_out & 1u) * a.dim + (int64_t)h * hs + tid, bare_of((float)acc));
+        bare_store(a.xo + (int64_t)((e_out & 1u) ^ 1u) * a.dim + (int64_t)h * hs + tid, FLOW_EMPTY);
     }
     __syncthreads();
     return true;
@@ -1216,7 +1223,8 @@ __device__ __noinline__ bool flow_attention_long(int layer, int h, int pos, unsi
     if (tid < hs) {
         double acc = 0.0;
         for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
-        tag_store(a.xb + (int64_t)h * hs + tid, (float)acc, e_out);
+        bare_store(a.xo + (int64_t)(e_out & 1u) * a.dim + (int64_t)h * hs + tid, bare_of((float)acc));
+        bare_store(a.xo + (int64_t)((e_out & 1u) ^ 1u) * a.dim + (int64_t)h * hs + tid, FLOW_EMPTY);
     }
     __syncthreads();
     return true;
@@ -1288,12 +1296,12 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     // the rows of x this workgroup adds to after wo (layer 0): straight from the embedding (:236)
     {
         const int lo = wg * a.wo.rpw, n = flow_n_local(a.wo, wg);
-        if (tid < n) tag_store(a.x_a + lo + tid, dequant_elem(a.emb, tok, lo + tid), E0);
+        if (tid < n) bare_store(a.x_a + lo + tid, bare_of(dequant_elem(a.emb, tok, lo + tid)));
     }
 
     for (int l = 0; l < a.n_layers; l++) {
         const unsigned e_x = E0 + 5u * (unsigned)l;  // x entering the layer
-        const unsigned e_q = e_x + 1, e_att = e_x + 2, e_wo = e_x + 3, e_w13 = e_x + 4, e_w2 = e_x + 5;
+        const unsigned e_q = e_x + 1, e_att = e_x + 2, e_w13 = e_x + 4;  // (e_x + 3 and e_x + 5: the two residual additions)
         // the four matvec phases of the layer share one copy of the streaming loop (the kernel must stay
         // small enough for the instruction cache):
         //   0  rmsnorm (:244), q, k, v (:247-249), rope (:255-256), cache append (:259-260)
@@ -1309,7 +1317,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
                 ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, 0, a.dim, nw, tok)
-                            : flow_stage<PRO_RMSNORM, SRC_TAGGED>(a.x_a, e_x, a.dim, nw, tok);
+                            : flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, 0, a.dim, nw, tok);
             } else if (kind == 1) {
                 if (is_att) {
                     const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_long(l, att_h, pos, e_q, e_att)
@@ -1320,9 +1328,9 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                 }
                 flow_reg_fetch(rp, reg_ptr, n_reg, lane);  // (after the attention: its loads would wait behind these)
                 FTL();
-                ok = flow_stage<PRO_QUANT, SRC_TAGGED>(a.xb, e_att, a.dim, nullptr, tok);
+                ok = flow_stage<PRO_QUANT, SRC_BARE>(a.xo + (int64_t)(e_att & 1u) * a.dim, 0, a.dim, nullptr, tok);
             } else if (kind == 2) {
-                ok = flow_stage<PRO_RMSNORM, SRC_TAGGED>(a.x_b, e_wo, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
+                ok = flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_b, 0, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
             } else {
                 ok = flow_stage<PRO_QUANT, SRC_BARE>(a.hbw + (int64_t)(e_w13 & 1u) * a.hidden, 0, a.hidden, nullptr, tok);
             }
@@ -1330,8 +1338,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             FTL();
             reg_ptr += n_reg * FLOW_SLOT;
             // the row of x this thread adds to after wo / w2: fetched now, used after the loop
-            u64 oldw = 0;
-            if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = tag_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
+            unsigned oldw = 0;
+            if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = bare_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
             // what the ring holds has landed by now: after this wait the first FLOW_D pieces need none,
             // and the cache lines requested next do not stand between the loop and its pieces
             flow_drain(r);
@@ -1344,11 +1352,11 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             if (kind == 0)
                 flow_finish_qkv(l, wg, pos, e_q);
             else if (kind == 1)
-                flow_finish_resid(1, wg, oldw, e_x, e_wo);
+                flow_finish_resid(1, wg, oldw);
             else if (kind == 2)
                 flow_finish_w13(wg, e_w13);
             else
-                flow_finish_resid(3, wg, oldw, e_wo, e_w2);
+                flow_finish_resid(3, wg, oldw);
             FTL();
         }
     }
@@ -1363,7 +1371,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         ring_uniform(r);
         flow_top_up_q6(r, ring_base, lane);
     }
-    if (!uni(flow_stage<PRO_RMSNORM, SRC_TAGGED>(a.x_a, e_fin, a.dim, a.rms_final, tok))) LEAVE();
+    if (!uni(flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, 0, a.dim, a.rms_final, tok))) LEAVE();
     flow_drain(r);
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
@@ -1495,6 +1503,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
         if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
             return no("too many rows per workgroup");  // (layer phases keep four partial sums per piece)
     if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
+    if (a.wo.rpw != a.w2.rpw) return no("row split of wo and w2 differs");  // (a row of x has one owner)
     return true;
 }
 

@@ -139,8 +139,10 @@ struct FlowArgs {
     const unsigned char *stream;  // per-wavefront weight streams
     const int64_t *wave_off;      // [grid * 16] byte offset of each wavefront's stream
     // activations as {fp32 value, epoch} words
-    unsigned long long *x_a, *x_b, *xb, *q, *kcur, *vcur, *amax;
-    unsigned int *hbw;  // [2][hidden] SwiGLU outputs as bare fp32 words, 0xFFFFFFFF = not written yet
+    unsigned long long *q, *kcur, *vcur, *amax;
+    // activations as bare fp32 words, 0xFFFFFFFF = not written yet: the residual stream in two buffers,
+    // attention outputs [2][dim] and SwiGLU outputs [2][hidden] (the pairs alternate from layer to layer)
+    unsigned int *x_a, *x_b, *xo, *hbw;
     float *kc, *vc, *logits;
     const float *rms_att, *rms_ffn, *rms_final;
     int64_t norm_stride;  // floats between the norm weights of consecutive layers
