@@ -552,7 +552,11 @@ __device__ __forceinline__ void flow_reg_arrived(RegPieces &rp) {
 template <bool REGS, bool QUARTERS>
 __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg, const RegPieces &rp,
                                              int n_reg) {
-    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // (the lane number through an empty asm: what is derived from it is computed here, at every call, and
+    // not once at the top of the kernel, where it would hold registers across all phases and be spilled)
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     RingLoop<FLOW_SLOT, FLOW_D, 2> q;
