@@ -97,6 +97,11 @@ int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t 
  * the choice after finalize (1, 2 or 3). */
 int l2h_model_set_path(l2h_model *m, int path);
 int l2h_model_path(l2h_model *m);
+/* Launch paths 2 and 3 wait on the device for other workgroups' results; every such wait gives up after
+ * `spins` polls (default 2^20 on path 3, about a second), upon which all workgroups leave the kernel and
+ * the call that launched it returns L2H_EHIP; the model stays usable (l2h_state_reset, then decode
+ * again).  This sets the bound for path 3 (after finalize).  No counterpart in the reference. */
+int l2h_model_set_wait_limit(l2h_model *m, unsigned int spins);
 /* RunState(config) (src/inference.jl:88-100): checks every tensor is present, allocates
  * activations and the zeroed KV cache, records the per-token launch sequence. */
 int l2h_model_finalize(l2h_model *m);

@@ -355,6 +355,14 @@ extern "C" int l2h_model_set_tensor(l2h_model *m, int role, int layer, int type,
     return rc;
 }
 
+extern "C" int l2h_model_set_wait_limit(l2h_model *m, unsigned int spins) {
+    if (!m) return L2H_EINVAL;
+    if (!m->flow) return set_err(m->ctx, L2H_ESTATE, "the wait limit applies to launch path 3 after finalize");
+    m->flow_args.spin_limit = spins;
+    if (g_flow_bound == m) g_flow_bound = nullptr;  // the kernel's copy of the arguments is refreshed at the next launch
+    return L2H_OK;
+}
+
 extern "C" int l2h_model_set_path(l2h_model *m, int path) {
     if (!m) return L2H_EINVAL;
     if (m->finalized) return set_err(m->ctx, L2H_ESTATE, "model already finalized");

@@ -110,6 +110,10 @@ class DeviceModel:
     def reset(self):
         self.ctx.check(_lib.lib().l2h_state_reset(self.handle))
 
+    def set_wait_limit(self, spins):
+        """Bound of the streaming kernel's device-side waits (l2h_model_set_wait_limit)."""
+        self.ctx.check(_lib.lib().l2h_model_set_wait_limit(self.handle, int(spins)))
+
     def forward(self, token, pos, want_logits=True):
         """transformer!(token, pos, ...) (src/inference.jl:222-315): returns (logits, argmax)."""
         logits = np.empty(self.config.vocab_size, np.float32) if want_logits else None

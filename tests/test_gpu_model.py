@@ -234,6 +234,29 @@ def test_streaming_kernel_long_cache(pkg, orc, rng, n_pre):
     assert _rel(logits, ref_logits) <= 1e-3
 
 
+def test_streaming_kernel_gives_up_and_recovers(pkg):
+    """A wait bound of zero makes the first poll that finds a word missing give up: every workgroup leaves
+    the kernel, the call fails, and after a reset with the normal bound the model decodes as before (the
+    exchange buffers are put back to "not written")."""
+    from llama2_jl_amd import synth
+    plan, kw = FLOW_CASES["all_q4"]
+    lm = _model(pkg, plan, **kw)
+    dev = lm.device(path=3)
+    assert dev.path == 3
+    prompt = synth.seeded_prompt(11, 6, lm.config.vocab_size)
+    dev.reset()
+    want = dev.generate_greedy(prompt, 10)
+    dev.set_wait_limit(0)
+    dev.reset()
+    with pytest.raises(pkg.L2HError):
+        dev.generate_greedy(prompt, 10)
+    dev.set_wait_limit(1 << 20)
+    for _ in range(2):
+        dev.reset()
+        got = dev.generate_greedy(prompt, 10)
+        assert np.asarray(got).tolist() == np.asarray(want).tolist()
+
+
 def test_generate_argument_checks(pkg):
     from llama2_jl_amd import synth
     plan, kw = CASES["f32"]
