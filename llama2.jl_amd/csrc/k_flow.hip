@@ -8,12 +8,18 @@
 //    pieces ahead of the arithmetic and straight across phase boundaries, so HBM keeps streaming
 //    while a workgroup waits for the activations of the next phase.
 //
-//  * No grid barrier.  Activations that cross workgroups travel as 8-byte words {fp32 value, epoch
-//    tag}, written and read with device-scope relaxed atomics.  A consumer polls the words it needs
-//    until they carry the epoch of the producing phase: data and "ready" arrive in one transaction.
-//    Each buffer is rewritten only two or more phases after its last read, and reaching a phase
-//    requires every workgroup to have finished the phase before the previous one, so a word is never
-//    overwritten while somebody may still want its old value.
+//  * No grid barrier.  Activations that cross workgroups carry their own "ready": the long vectors that
+//    every workgroup reads whole (residual stream, attention output, SwiGLU output) are bare fp32 words
+//    in which a reserved NaN pattern means "not written yet" (see FLOW_EMPTY), the short ones (q, k, v of
+//    the current position, the per-workgroup argmax keys) are 8-byte words {fp32 value, epoch tag}.  All
+//    are written and read with device-scope relaxed atomics or their 16-byte equivalent; a consumer polls
+//    until its words are there: data and "ready" arrive in one transaction.  Each buffer is rewritten (or
+//    marked empty again) only two or more phases after its last read, and reaching a phase requires every
+//    workgroup to have finished the phase before the previous one, so a word is never overwritten while
+//    somebody may still want its old value.
+//
+//  Besides: a few pieces per phase travel through registers, requested while the phase waits for its
+//  input (see flow_reg_pieces), and the attention is built for low latency (flow_attention_short).
 //
 // The arithmetic is the same as in the per-phase kernels (matvec_dev.h): q8_K activations, integer
 // dot products, fp64 sums rounded once.  Every wait is bounded; a workgroup that gives up raises
@@ -267,11 +273,6 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
 // instruction asks for whole cache lines.  The loads and the wait for them are ONE asm statement: the
 // compiler believes an asm's outputs valid as soon as the statement ends and may copy them at once, so no
 // statement may end with a load still under way.
-#define POLL_TAGGED(lo, hi, p)                                                                                           \
-    asm volatile("global_load_dwordx4 %0, %2, off sc1\n\tglobal_load_dwordx4 %1, %2, off offset:16 sc1\n\ts_waitcnt vmcnt(0)" \
-                 : "+v"(lo), "+v"(hi)                                                                                    \
-                 : "v"(p)                                                                                                \
-                 : "memory")
 #define POLL_BARE1(w0, p0) \
     asm volatile("global_load_dwordx4 %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "+v"(w0) : "v"(p0) : "memory")
 #define POLL_BARE2(w0, w1, p0, p1)                                                                                    \
@@ -294,13 +295,12 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
 
 // SRC: where the input comes from
 #define SRC_EMB 0     // the embedding row of `tok`
-#define SRC_TAGGED 1  // {fp32, epoch} words; a word is there when it carries `epoch`
 #define SRC_BARE 2    // fp32 words; a word is there when it is not FLOW_EMPTY
-// Tagged words, the embedding and norm weights come with vectors of dim <= 4096 only (one q8_K block per
-// wavefront); the bare words of the hidden vector take up to four rounds.
+// The embedding and norm weights come with vectors of dim <= 4096 only (one q8_K block per wavefront);
+// the words of the hidden vector take up to four rounds.
 template <int PRO, int SRC>
-__device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, const float *normw, int tok) {
-    src = uni(src), epoch = uni(epoch), K = uni(K), normw = uni(normw), tok = uni(tok);
+__device__ __noinline__ bool flow_stage(const void *src, int K, const float *normw, int tok) {
+    src = uni(src), K = uni(K), normw = uni(normw), tok = uni(tok);
     const FlowArgs &a = c_flow;
     int8_t *s_qs = (int8_t *)s_act;
     int16_t *s_bs = (int16_t *)(s_qs + 14336);
@@ -309,7 +309,7 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
     const int nb = K >> 8;
     static_assert(STAGE_MAX_ROUNDS == 4, "four rounds below");
     const int rounds = nb > wave ? (nb - wave + FLOW_NW - 1) / FLOW_NW : 0;  // q8_K blocks of this wavefront
-    constexpr bool rms = PRO == PRO_RMSNORM, bare = SRC == SRC_BARE;
+    constexpr bool rms = PRO == PRO_RMSNORM;
     float xv[4][4];
     float wv0[4];
     bool ok = true;
@@ -327,40 +327,28 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
             for (int k = 0; k < 4; k++) xv[0][k] = dequant_elem(a.emb, tok, 256 * wave + 4 * lane + k);
     } else {
         unsigned spins = 0;
-        // tagged: words 0,1 in w0, 2,3 in wh; bare: round r in w<r>; all start as "not there"
-        const unsigned none = bare ? FLOW_EMPTY : 0u;  // (epochs are never 0)
-        u32x4v w0 = {none, none, none, none}, w1 = w0, w2 = w0, w3 = w0, wh = w0;
-        const u64 *pt = (const u64 *)src + 256 * wave + 4 * lane;
+        // round r in w<r>; all start as "not there"
+        u32x4v w0 = {FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY}, w1 = w0, w2 = w0, w3 = w0;
         const unsigned *pb = (const unsigned *)src + 256 * wave + 4 * lane;
         for (;;) {
             bool all = true;
-            if (rounds > 0) {
-                // (a lane that has all its words does not ask again: waiting for a slow producer costs little traffic)
-                if (!bare) {
-                    all = w0.y == epoch && w0.w == epoch && wh.y == epoch && wh.w == epoch;
-                    if (!all) {
-                        POLL_TAGGED(w0, wh, pt);
-                        all = w0.y == epoch && w0.w == epoch && wh.y == epoch && wh.w == epoch;
-                    }
-                } else {
+            // (a lane that has all its words does not ask again: waiting for a slow producer costs little traffic)
 #define FULL(V_) (V_.x != FLOW_EMPTY && V_.y != FLOW_EMPTY && V_.z != FLOW_EMPTY && V_.w != FLOW_EMPTY)
-                    if (rounds == 1) {
-                        if (!FULL(w0)) POLL_BARE1(w0, pb);
-                        all = FULL(w0);
-                    } else if (rounds == 2) {
-                        if (!(FULL(w0) && FULL(w1))) POLL_BARE2(w0, w1, pb, pb + 256 * FLOW_NW);
-                        all = FULL(w0) && FULL(w1);
-                    } else if (rounds == 3) {
-                        if (!(FULL(w0) && FULL(w1) && FULL(w2))) POLL_BARE3(w0, w1, w2, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW);
-                        all = FULL(w0) && FULL(w1) && FULL(w2);
-                    } else {
-                        if (!(FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3)))
-                            POLL_BARE4(w0, w1, w2, w3, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW, pb + 768 * FLOW_NW);
-                        all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
-                    }
-#undef FULL
-                }
+            if (rounds == 1) {
+                if (!FULL(w0)) POLL_BARE1(w0, pb);
+                all = FULL(w0);
+            } else if (rounds == 2) {
+                if (!(FULL(w0) && FULL(w1))) POLL_BARE2(w0, w1, pb, pb + 256 * FLOW_NW);
+                all = FULL(w0) && FULL(w1);
+            } else if (rounds == 3) {
+                if (!(FULL(w0) && FULL(w1) && FULL(w2))) POLL_BARE3(w0, w1, w2, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW);
+                all = FULL(w0) && FULL(w1) && FULL(w2);
+            } else if (rounds == 4) {
+                if (!(FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3)))
+                    POLL_BARE4(w0, w1, w2, w3, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW, pb + 768 * FLOW_NW);
+                all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
             }
+#undef FULL
             if (__ballot(!all) == 0ull) break;
             if (++spins > a.spin_limit ||
                 ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
@@ -368,20 +356,13 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
                 break;
             }
         }
-        if (!bare) {
-            xv[0][0] = __uint_as_float(w0.x);
-            xv[0][1] = __uint_as_float(w0.z);
-            xv[0][2] = __uint_as_float(wh.x);
-            xv[0][3] = __uint_as_float(wh.z);
-        } else {
-            const u32x4v ws[4] = {w0, w1, w2, w3};
+        const u32x4v ws[4] = {w0, w1, w2, w3};
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                xv[r][0] = __uint_as_float(ws[r].x);
-                xv[r][1] = __uint_as_float(ws[r].y);
-                xv[r][2] = __uint_as_float(ws[r].z);
-                xv[r][3] = __uint_as_float(ws[r].w);
-            }
+        for (int r = 0; r < 4; r++) {
+            xv[r][0] = __uint_as_float(ws[r].x);
+            xv[r][1] = __uint_as_float(ws[r].y);
+            xv[r][2] = __uint_as_float(ws[r].z);
+            xv[r][3] = __uint_as_float(ws[r].w);
         }
     }
     if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
@@ -412,7 +393,7 @@ __device__ __noinline__ bool flow_stage(const void *src, unsigned epoch, int K, 
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const int b = wave + r * FLOW_NW;
-        if (r < rounds && (bare || r == 0)) {
+        if (r < rounds && (SRC == SRC_BARE || r == 0)) {
             uint32_t packed;
             int bsum;
             float d;
@@ -1320,8 +1301,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             if (kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
-                ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, 0, a.dim, nw, tok)
-                            : flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, 0, a.dim, nw, tok);
+                ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, a.dim, nw, tok)
+                            : flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, nw, tok);
             } else if (kind == 1) {
                 if (is_att) {
                     const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_long(l, att_h, pos, e_q, e_att)
@@ -1332,11 +1313,11 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                 }
                 flow_reg_fetch(rp, reg_ptr, n_reg, lane);  // (after the attention: its loads would wait behind these)
                 FTL();
-                ok = flow_stage<PRO_QUANT, SRC_BARE>(a.xo + (int64_t)(e_att & 1u) * a.dim, 0, a.dim, nullptr, tok);
+                ok = flow_stage<PRO_QUANT, SRC_BARE>(a.xo + (int64_t)(e_att & 1u) * a.dim, a.dim, nullptr, tok);
             } else if (kind == 2) {
-                ok = flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_b, 0, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
+                ok = flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_b, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
             } else {
-                ok = flow_stage<PRO_QUANT, SRC_BARE>(a.hbw + (int64_t)(e_w13 & 1u) * a.hidden, 0, a.hidden, nullptr, tok);
+                ok = flow_stage<PRO_QUANT, SRC_BARE>(a.hbw + (int64_t)(e_w13 & 1u) * a.hidden, a.hidden, nullptr, tok);
             }
             if (!uni(ok)) LEAVE();
             FTL();
@@ -1375,7 +1356,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         ring_uniform(r);
         flow_top_up_q6(r, ring_base, lane);
     }
-    if (!uni(flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, 0, a.dim, a.rms_final, tok))) LEAVE();
+    if (!uni(flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, a.rms_final, tok))) LEAVE();
     flow_drain(r);
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
