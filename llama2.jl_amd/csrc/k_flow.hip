@@ -505,6 +505,7 @@ struct RegPieces {
 };
 // requests them: n pieces at p (every index below is a constant after unrolling: the arrays stay registers)
 __device__ __forceinline__ void flow_reg_fetch(RegPieces &rp, const unsigned char *p, int n, int lane) {
+    asm volatile("" : "+v"(lane));  // (the addresses below are computed here, not kept in registers across the kernel)
     const AS1 unsigned char *g = (const AS1 unsigned char *)p;  // (a global address: plain global loads)
     const AS1 unsigned char *ph = g + (lane >> 3) * 16, *pq = g + 128 + lane * 16;
     const int fo = 4 + 3 * ((lane & 7) >> 1);
@@ -740,7 +741,9 @@ __device__ __forceinline__ float flow_row_value4(int lr, int ppr) {
 __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
     l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
-    const int n_local = flow_n_local(a.qkv, wg), tid = threadIdx.x;
+    const int n_local = flow_n_local(a.qkv, wg);
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));  // (what derives from it is computed here and not kept across the kernel)
     __syncthreads();
     if (tid >= n_local) return;
     const int L = wg * a.qkv.rpw + tid;
@@ -777,7 +780,9 @@ __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned ol
     const FlowGeom &g = which == 1 ? a.wo : a.w2;
     unsigned *src = which == 1 ? a.x_a : a.x_b;
     unsigned *dst = which == 1 ? a.x_b : a.x_a;
-    const int n_local = flow_n_local(g, wg), tid = threadIdx.x;
+    const int n_local = flow_n_local(g, wg);
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
     __syncthreads();
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
@@ -790,7 +795,9 @@ __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned ol
 __device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
     wg = uni(wg), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
-    const int n_local = flow_n_local(a.w13, wg), tid = threadIdx.x;
+    const int n_local = flow_n_local(a.w13, wg);
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
     __syncthreads();
     if (tid >= n_local || (tid & 1)) return;
     const int64_t u = ((int64_t)wg * a.w13.rpw + tid) >> 1;
@@ -1296,6 +1303,10 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 #pragma nounroll
         for (int kind = 0; kind < 4; kind++) {
             bool ok;
+            // (thread and lane number anew in every phase: see flow_loop_q4)
+            int tid = threadIdx.x;
+            asm volatile("" : "+v"(tid));
+            const int lane = tid & 63;
             const FlowGeom g = flow_geom(a, kind);
             const int n_reg = uni(flow_reg_pieces(g, wg, wave));
             if (kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
