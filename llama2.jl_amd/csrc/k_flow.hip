@@ -791,18 +791,26 @@ __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned ol
     bare_store(src + row, FLOW_EMPTY);  // (its readers are through: see FLOW_EMPTY)
 }
 
-// SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u
-__device__ __noinline__ void flow_finish_w13(int wg, unsigned e_out) {
-    wg = uni(wg), e_out = uni(e_out);
+// SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u.  The arithmetic (an fp64 exp) is a
+// function of its own for the registers it takes; the stores are the caller's: a function that stores
+// waits before it returns until the stores are acknowledged.
+__device__ __noinline__ unsigned flow_w13_word(int wg) {
+    wg = uni(wg);
     const FlowArgs &a = c_flow;
     const int n_local = flow_n_local(a.w13, wg);
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
     __syncthreads();
-    if (tid >= n_local || (tid & 1)) return;
+    if (tid >= n_local || (tid & 1)) return 0u;
+    return bare_of(swiglu_val(flow_row_value4(tid, a.w13.ppr), flow_row_value4(tid + 1, a.w13.ppr)));
+}
+__device__ __forceinline__ void flow_finish_w13(int wg, unsigned e_out) {
+    const FlowArgs &a = c_flow;
+    const unsigned v = flow_w13_word(wg);
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    if (tid >= flow_n_local(a.w13, wg) || (tid & 1)) return;
     const int64_t u = ((int64_t)wg * a.w13.rpw + tid) >> 1;
-    unsigned v = __float_as_uint(swiglu_val(flow_row_value4(tid, a.w13.ppr), flow_row_value4(tid + 1, a.w13.ppr)));
-    if (v == FLOW_EMPTY) v = 0x7FC00000u;
     unsigned *mine = a.hbw + (int64_t)(e_out & 1u) * a.hidden, *other = a.hbw + (int64_t)((e_out & 1u) ^ 1u) * a.hidden;
     bare_store(mine + u, v);
     bare_store(other + u, FLOW_EMPTY);
