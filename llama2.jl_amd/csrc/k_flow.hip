@@ -599,15 +599,11 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
             q.fetched();
         }
         q.next_slot();
-#ifdef FLOW_EXP_NOMATH
-        acc += (double)(w.x ^ field);
-#else
         {
             int sc_a, sc_b, m_a, m_b;
             flow_decode_field(field, sc_a, sc_b, m_a, m_b);
             acc += flow_q4_term(w, d_dmin, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
         }
-#endif
         FLOW_PIECE_DONE();
     }
     q.end(r, n_ring, left0 - q.left);
