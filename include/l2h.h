@@ -102,6 +102,11 @@ int l2h_model_path(l2h_model *m);
  * the call that launched it returns L2H_EHIP; the model stays usable (l2h_state_reset, then decode
  * again).  This sets the bound for path 3 (after finalize).  No counterpart in the reference. */
 int l2h_model_set_wait_limit(l2h_model *m, unsigned int spins);
+/* l2h_prefill keeps a bf16 copy of the layer matrices (2 bytes per weight, made at its first call
+ * when that fits beside 2 GiB of free device memory) and multiplies from it; on = 0 makes it
+ * expand the quantized blocks inside the product kernel on every call instead (no extra memory,
+ * slower).  The results are the same bit for bit.  Default 1.  No counterpart in the reference. */
+int l2h_model_set_prefill_copy(l2h_model *m, int on);
 /* RunState(config) (src/inference.jl:88-100): checks every tensor is present, allocates
  * activations and the zeroed KV cache, records the per-token launch sequence. */
 int l2h_model_finalize(l2h_model *m);

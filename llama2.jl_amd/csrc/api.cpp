@@ -243,6 +243,11 @@ struct l2h_model {
     float *pf_x = nullptr, *pf_raw = nullptr, *pf_cs = nullptr;
     uint16_t *pf_xn = nullptr, *pf_q = nullptr, *pf_att = nullptr, *pf_hb = nullptr;
     int32_t *pf_tok = nullptr;
+    // bf16 copy of the layer matrices for the prompt pass: per layer q|k|v rows, wo, w1/w3 rows in turn, w2
+    int pf_copy_mode = 1;          // 0 never, 1 when it fits
+    bool pf_copy_tried = false;
+    uint16_t *pf_wbf = nullptr;
+    int64_t pf_wbf_layer = 0, pf_off_wo = 0, pf_off_w13 = 0, pf_off_w2 = 0;  // elements
     std::vector<void *> allocs;
 
     DevTensor &L(int layer_idx, int role) { return layer[(size_t)layer_idx * L2H_N_ROLES + role]; }
@@ -291,6 +296,8 @@ static void model_free_state(l2h_model *m) {
     for (void *p : m->allocs) (void)hipFree(p);
     m->allocs.clear();
     m->pf_cap = 0;
+    m->pf_wbf = nullptr;
+    m->pf_copy_tried = false;
     m->sample_p = nullptr;
     m->sample_out = nullptr;
     m->finalized = false;
@@ -360,6 +367,13 @@ extern "C" int l2h_model_set_wait_limit(l2h_model *m, unsigned int spins) {
     if (!m->flow) return set_err(m->ctx, L2H_ESTATE, "the wait limit applies to launch path 3 after finalize");
     m->flow_args.spin_limit = spins;
     if (g_flow_bound == m) g_flow_bound = nullptr;  // the kernel's copy of the arguments is refreshed at the next launch
+    return L2H_OK;
+}
+
+extern "C" int l2h_model_set_prefill_copy(l2h_model *m, int on) {
+    if (!m) return L2H_EINVAL;
+    if (on != 0 && on != 1) return set_err(m->ctx, L2H_EINVAL, "on must be 0 or 1");
+    m->pf_copy_mode = on;
     return L2H_OK;
 }
 
@@ -1013,6 +1027,45 @@ static int prefill_buffers(l2h_model *m, int cap) {
     return L2H_OK;
 }
 
+// Expands every layer matrix to bf16 once (the values the fused product kernel would form in LDS), so
+// that later prompt passes run plain bf16 products.  2 bytes per weight stay resident; when that does
+// not fit beside 2 GiB of head room, or dim or hidden_dim is not a multiple of 64, the fused kernels
+// stay in use.
+static int prefill_weights(l2h_model *m) {
+    if (m->pf_copy_tried) return L2H_OK;
+    m->pf_copy_tried = true;
+    const l2h_config &c = m->c;
+    const int64_t dim = c.dim, kvd = m->kv_dim, hid = c.hidden_dim;
+    if (dim % 64 != 0 || hid % 64 != 0) return L2H_OK;
+    auto pad128 = [](int64_t r) { return (r + 127) / 128 * 128; };
+    m->pf_off_wo = pad128(dim + 2 * kvd) * dim;
+    m->pf_off_w13 = m->pf_off_wo + pad128(dim) * dim;
+    m->pf_off_w2 = m->pf_off_w13 + pad128(2 * hid) * dim;
+    m->pf_wbf_layer = m->pf_off_w2 + pad128(dim) * hid;
+    const size_t bytes = (size_t)m->pf_wbf_layer * c.n_layers * 2;
+    size_t free_b = 0, total_b = 0;
+    HIPCHK(m->ctx, hipMemGetInfo(&free_b, &total_b));
+    if (free_b < bytes + ((size_t)2 << 30)) return L2H_OK;
+    uint16_t *buf = nullptr;
+    int rc;
+    if ((rc = dalloc(m, &buf, (int64_t)(bytes / 2), false))) return rc;
+    hipStream_t s = m->ctx->stream;
+    for (int l = 0; l < c.n_layers; l++) {
+        uint16_t *base = buf + (int64_t)l * m->pf_wbf_layer;
+        const DevTensor w[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
+        const int64_t row0[3] = {0, dim, dim + kvd};
+        for (int i = 0; i < 3; i++) HIPCHK(m->ctx, k_pf_expand(s, w + i, 1, 0, dim, base, row0[i], i == 2));
+        const DevTensor wo = m->L(l, L2H_WO), w2 = m->L(l, L2H_W2);
+        const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
+        HIPCHK(m->ctx, k_pf_expand(s, &wo, 1, 0, dim, base + m->pf_off_wo, 0, 1));
+        HIPCHK(m->ctx, k_pf_expand(s, w13, 2, 1, dim, base + m->pf_off_w13, 0, 1));
+        HIPCHK(m->ctx, k_pf_expand(s, &w2, 1, 0, hid, base + m->pf_off_w2, 0, 1));
+    }
+    HIPCHK(m->ctx, hipStreamSynchronize(s));
+    m->pf_wbf = buf;
+    return L2H_OK;
+}
+
 static hipError_t prefill_chunk(l2h_model *m, int M, int pos0) {
     hipStream_t s = m->ctx->stream;
     const l2h_config &c = m->c;
@@ -1029,25 +1082,35 @@ static hipError_t prefill_chunk(l2h_model *m, int M, int pos0) {
         float *kc = m->kc + (int64_t)l * m->cache_layer_elems;
         float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
         CK(k_pf_rmsnorm(s, m->pf_x, m->L(l, L2H_RMS_ATT).f32, m->pf_xn, M, dim));
-        // q | k | v columns of pf_raw; consecutive tensors of one type share a launch
-        const DevTensor w[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
-        const int64_t col[3] = {0, dim, dim + kvd};
-        for (int i = 0; i < 3;) {
-            int j = i + 1;
-            while (j < 3 && w[j].type == w[i].type) j++;
-            CK(k_pf_gemm(s, w + i, j - i, 0, m->pf_xn, M, dim, PF_STORE, m->pf_raw, dim + 2 * kvd, col[i], nullptr, 0));
-            i = j;
+        const uint16_t *wb = (m->pf_wbf && m->pf_copy_mode) ? m->pf_wbf + (int64_t)l * m->pf_wbf_layer : nullptr;
+        if (wb) {
+            CK(k_pf_gemm(s, nullptr, 0, 0, wb, dim + 2 * kvd, m->pf_xn, M, dim, PF_STORE, m->pf_raw, dim + 2 * kvd, 0,
+                         nullptr, 0));
+        } else {
+            // q | k | v columns of pf_raw; consecutive tensors of one type share a launch
+            const DevTensor w[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
+            const int64_t col[3] = {0, dim, dim + kvd};
+            for (int i = 0; i < 3;) {
+                int j = i + 1;
+                while (j < 3 && w[j].type == w[i].type) j++;
+                CK(k_pf_gemm(s, w + i, j - i, 0, nullptr, 0, m->pf_xn, M, dim, PF_STORE, m->pf_raw, dim + 2 * kvd,
+                             col[i], nullptr, 0));
+                i = j;
+            }
         }
         CK(k_pf_rope_scatter(s, m->pf_raw, m->pf_cs, m->pf_q, kc, vc, M, pos0, dim, kvd, m->hs, c.seq_len,
                              c.rope_is_neox));
         CK(k_pf_attention(s, m->pf_q, m->pf_att, kc, vc, M, pos0, m->hs, c.n_heads, c.n_kv_heads, c.seq_len, dim));
         const DevTensor wo = m->L(l, L2H_WO);
-        CK(k_pf_gemm(s, &wo, 1, 0, m->pf_att, M, dim, PF_RESID, m->pf_x, dim, 0, nullptr, 0));
+        CK(k_pf_gemm(s, &wo, 1, 0, wb ? wb + m->pf_off_wo : nullptr, dim, m->pf_att, M, dim, PF_RESID, m->pf_x, dim, 0,
+                     nullptr, 0));
         CK(k_pf_rmsnorm(s, m->pf_x, m->L(l, L2H_RMS_FFN).f32, m->pf_xn, M, dim));
         const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
-        CK(k_pf_gemm(s, w13, 2, 1, m->pf_xn, M, dim, PF_SWIGLU, nullptr, 0, 0, m->pf_hb, c.hidden_dim));
+        CK(k_pf_gemm(s, w13, 2, 1, wb ? wb + m->pf_off_w13 : nullptr, 2 * (int64_t)c.hidden_dim, m->pf_xn, M, dim,
+                     PF_SWIGLU, nullptr, 0, 0, m->pf_hb, c.hidden_dim));
         const DevTensor w2 = m->L(l, L2H_W2);
-        CK(k_pf_gemm(s, &w2, 1, 0, m->pf_hb, M, c.hidden_dim, PF_RESID, m->pf_x, dim, 0, nullptr, 0));
+        CK(k_pf_gemm(s, &w2, 1, 0, wb ? wb + m->pf_off_w2 : nullptr, dim, m->pf_hb, M, c.hidden_dim, PF_RESID, m->pf_x,
+                     dim, 0, nullptr, 0));
     }
 #undef CK
     return hipSuccess;
@@ -1074,6 +1137,7 @@ extern "C" int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0,
     HIPCHK(ctx, hipSetDevice(ctx->device));
     int rc;
     if ((rc = prefill_buffers(m, std::min(n, L2H_PREFILL_CHUNK)))) return rc;
+    if (m->pf_copy_mode && (rc = prefill_weights(m))) return rc;
     int M = 0;
     for (int c0 = 0; c0 < n; c0 += M) {
         M = std::min(m->pf_cap, n - c0);

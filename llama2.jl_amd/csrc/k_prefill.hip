@@ -106,6 +106,7 @@ struct PfGemmArgs {
     int64_t ldo, out_col0;
     uint16_t *out_bf;  // SWIGLU: bf16 [M][ldb], column L/2
     int64_t ldb;
+    const uint16_t *wbf;  // pf_gemm_bf16_kernel: the weights expanded beforehand (pf_expand_kernel's tiles)
 };
 
 struct PfRow {
@@ -254,6 +255,93 @@ __device__ __forceinline__ void pf_convert(const PfRaw &r, const PfRowPtr &p, in
     for (int c = 0; c < 4; c++) out[c] = make_uint4(pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]);
 }
 
+// the stream pointers of logical weight row L
+template <int TYPE>
+__device__ __forceinline__ void pf_row_ptr(const PfGemmArgs &a, int64_t L, PfRow &lr, PfRowPtr &rp) {
+    lr = pf_row(a, L);
+    const int sg = lr.seg;
+#define PICK(F) (sg == 0 ? a.w[0].F : (sg == 1 ? a.w[1].F : a.w[2].F))
+    rp.hdr = PICK(hdr);
+    rp.qs = PICK(qs);
+    rp.qh = PICK(qh);
+    rp.sc6 = PICK(sc6);
+    rp.d6 = PICK(d6);
+    rp.f32 = PICK(f32);
+    rp.nb = PICK(nb);
+    rp.ne0 = PICK(ne0);
+#undef PICK
+    rp.valid = lr.valid;
+}
+
+// One thread expands 32 consecutive weights of one logical row to bf16, with the arithmetic the fused
+// product kernel uses on them.  The destination is a sequence of 16 KB tiles, tile (nt, kt) = weight
+// rows 128 nt.. x inputs 64 kt.. at ((nt K/64) + kt) * 8192 elements, and inside a tile the image the
+// product kernels keep in LDS: the 16-byte chunk c of row r at chunk index 8 r + (c ^ (r & 7)).  Logical
+// row L goes to row dst_row0 + L; rows from n_rows up to rows_end (padding of the last tile) are zero.
+template <int TYPE>
+__global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *dst, int64_t dst_row0, int64_t rows_end) {
+    const int64_t groups = a.K >> 5, nk = a.K >> 6;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= rows_end * groups) return;
+    const int64_t L = idx / groups, g = idx - L * groups, k0 = 32 * g;
+    PfRow lr;
+    PfRowPtr rp;
+    pf_row_ptr<TYPE>(a, L, lr, rp);
+    PfRaw raw;
+    pf_load_raw<TYPE>(raw, rp, lr.row, k0, a.K);
+    uint4 wv[4];
+    pf_convert<TYPE>(raw, rp, lr.row, k0, a.K, wv);
+    const int64_t R = dst_row0 + L, nt = R >> 7, kt = g >> 1;
+    const int r = (int)(R & 127);
+    uint4 *tile = (uint4 *)(dst + (nt * nk + kt) * 8192);
+#pragma unroll
+    for (int cc = 0; cc < 4; cc++) {
+        const int c = 4 * (int)(g & 1) + cc;
+        tile[r * 8 + (c ^ (r & 7))] = wv[cc];
+    }
+}
+
+// Results of one workgroup tile: a lane holds position m0 + 32 JT wm + 32 j + lane%32 and, in register r
+// of tile i, logical weight row n0 + 64 wn + 32 i + 8 (r/4) + 4 (lane/32) + r%4.
+template <int EPI, int JT>
+__device__ __forceinline__ void pf_epilogue(const PfGemmArgs &a, f32x16 (&acc)[2][JT], int64_t n0, int m0, int wn, int wm,
+                                            int lane) {
+#pragma unroll
+    for (int j = 0; j < JT; j++) {
+        const int m = m0 + 32 * JT * wm + 32 * j + (lane & 31);
+        if (m >= a.M) continue;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+#pragma unroll
+            for (int rq = 0; rq < 4; rq++) {
+                const int64_t L = n0 + 64 * wn + 32 * i + 8 * rq + 4 * (lane >> 5);
+                if (L >= a.n_rows) continue;
+                const float v0 = acc[i][j][4 * rq], v1 = acc[i][j][4 * rq + 1], v2 = acc[i][j][4 * rq + 2],
+                            v3 = acc[i][j][4 * rq + 3];
+                if (EPI == PF_SWIGLU) {  // (w1 row u, w3 row u) = logical rows (2u, 2u+1), src/inference.jl:295-299
+                    const float h0 = swiglu_val(v0, v1), h1 = swiglu_val(v2, v3);
+                    uint16_t *o = a.out_bf + (int64_t)m * a.ldb + (L >> 1);
+                    if (L + 3 < a.n_rows)
+                        *(uint32_t *)o = pack_bf16(h0, h1);  // L/2 is even and ldb is even: aligned
+                    else
+                        ((__bf16 *)o)[0] = (__bf16)h0;
+                } else {
+                    float *o = a.out + (int64_t)m * a.ldo + a.out_col0 + L;
+                    const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (L + e >= a.n_rows) break;
+                        if (EPI == PF_RESID)
+                            o[e] += v[e];  // x .+= ... (src/inference.jl:284,305)
+                        else
+                            o[e] = v[e];
+                    }
+                }
+            }
+        }
+    }
+}
+
 // Workgroup tile: 128 weight rows x 128 positions, K in steps of 64; 4 wavefronts, each 64 x 64 as
 // 2 x 2 tiles of 32 x 32.  Weights are the A operand (rows), positions the B operand (columns), so
 // a lane ends up holding one position and groups of 4 consecutive weight rows: neighbours such as a
@@ -271,22 +359,9 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 
     // the weight row this thread dequantizes: row t/2 of the tile, elements 32*(t&1).. of each K step
     const int wr = t >> 1, whh = t & 1;
-    const PfRow lr = pf_row(a, n0 + wr);
+    PfRow lr;
     PfRowPtr rp;
-    {
-        const int sg = lr.seg;
-#define PICK(F) (sg == 0 ? a.w[0].F : (sg == 1 ? a.w[1].F : a.w[2].F))
-        rp.hdr = PICK(hdr);
-        rp.qs = PICK(qs);
-        rp.qh = PICK(qh);
-        rp.sc6 = PICK(sc6);
-        rp.d6 = PICK(d6);
-        rp.f32 = PICK(f32);
-        rp.nb = PICK(nb);
-        rp.ne0 = PICK(ne0);
-#undef PICK
-        rp.valid = lr.valid;
-    }
+    pf_row_ptr<TYPE>(a, n0 + wr, lr, rp);
     // activations: 2 JT chunks of 16 bytes per thread and K step: position (t>>3) + 32*i, chunk t&7
     constexpr int XL = 2 * JT;
     const int xc = t & 7;
@@ -357,42 +432,134 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
         __syncthreads();
     }
 
-    // lane: position m0 + 32 JT wm + 32 j + lane%32; register r of tile i: logical weight row
-    // n0 + 64 wn + 32 i + 8 (r/4) + 4 (lane/32) + r%4
+    pf_epilogue<EPI, JT>(a, acc, n0, m0, wn, wm, lane);
+}
+
+#define PF_AS1 __attribute__((address_space(1)))
+#define PF_AS3 __attribute__((address_space(3)))
+
+// The same product from weights expanded beforehand (pf_expand_kernel): no arithmetic on the operands.
+// Both tiles of a K step travel from global memory straight into LDS (16 bytes per lane and load, a
+// wavefront's load filling 1 KB of LDS in lane order): the weight tile is a linear copy of its 16 KB
+// image, the position tile gets the c ^ (r & 7) placement by the choice of the address each lane reads.
+// Two LDS stages: the loads of step kt + 1 are in flight during the products of step kt, one barrier
+// per step.  Workgroups are dealt to the 8 XCDs in turn, so workgroup w takes tile (w % 8) * per + w / 8:
+// each XCD works through a contiguous run of tiles, positions fastest, and the workgroups that share a
+// weight tile share an L2.
+typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
+
+// the operands of one 16-wide slice of the K step (2 weight row groups, 2 position groups) from LDS stage
+// at byte offset OFF; loads and their wait are one statement, so no register of a load under way is visible
+#define PF_LDS_SLICE(OFF, KK)                                                                                       \
+    asm volatile("ds_read_b128 %0, %4 offset:" #OFF "\n\tds_read_b128 %1, %5 offset:" #OFF                         \
+                 "\n\tds_read_b128 %2, %6 offset:" #OFF "\n\tds_read_b128 %3, %7 offset:" #OFF                     \
+                 "\n\ts_waitcnt lgkmcnt(0)"                                                                         \
+                 : "=&v"(fa0), "=&v"(fa1), "=&v"(fb0), "=&v"(fb1)                                                   \
+                 : "v"(aw[0][KK]), "v"(aw[1][KK]), "v"(ax[0][KK]), "v"(ax[1][KK])                                   \
+                 : "memory")
+
+template <int EPI>
+__global__ __launch_bounds__(256) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned n_mt, unsigned n_tiles, unsigned per) {
+    constexpr int JT = 2;
+    // two stages of 32 KB: weight tile (16 KB), then position tile (16 KB)
+    __shared__ uint4 s_all[4096];
+    const unsigned tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+    if (tile >= n_tiles) return;
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wn = wave & 1, wm = wave >> 1;
+    const unsigned mt = tile % n_mt, nt = tile / n_mt;
+    const int64_t n0 = (int64_t)nt * 128;
+    const int m0 = (int)mt * 128;
+    const int64_t K = a.K, nk = K >> 6;
+
+    // weights: this wavefront copies bytes [4096 wave, +4096) of every tile, 1 KB per load
+    const unsigned char *gw = (const unsigned char *)(a.wbf + (int64_t)nt * nk * 8192) + wave * 4096 + lane * 16;
+    // positions: load i of this wavefront fills chunks 64 (4 wave + i) + lane: row 8 (4 wave + i) + lane / 8,
+    // placed chunk lane % 8 = the data chunk (lane % 8) ^ (row % 8)
+    const int xc = (lane & 7) ^ ((lane >> 3) & 7);
+    const unsigned char *gx[4];
 #pragma unroll
-    for (int j = 0; j < JT; j++) {
-        const int m = m0 + 32 * JT * wm + 32 * j + (lane & 31);
-        if (m >= a.M) continue;
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-#pragma unroll
-            for (int rq = 0; rq < 4; rq++) {
-                const int64_t L = n0 + 64 * wn + 32 * i + 8 * rq + 4 * (lane >> 5);
-                if (L >= a.n_rows) continue;
-                const float v0 = acc[i][j][4 * rq], v1 = acc[i][j][4 * rq + 1], v2 = acc[i][j][4 * rq + 2],
-                            v3 = acc[i][j][4 * rq + 3];
-                if (EPI == PF_SWIGLU) {  // (w1 row u, w3 row u) = logical rows (2u, 2u+1), src/inference.jl:295-299
-                    const float h0 = swiglu_val(v0, v1), h1 = swiglu_val(v2, v3);
-                    uint16_t *o = a.out_bf + (int64_t)m * a.ldb + (L >> 1);
-                    if (L + 3 < a.n_rows)
-                        *(uint32_t *)o = pack_bf16(h0, h1);  // L/2 is even and ldb is even: aligned
-                    else
-                        ((__bf16 *)o)[0] = (__bf16)h0;
-                } else {
-                    float *o = a.out + (int64_t)m * a.ldo + a.out_col0 + L;
-                    const float v[4] = {v0, v1, v2, v3};
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        if (L + e >= a.n_rows) break;
-                        if (EPI == PF_RESID)
-                            o[e] += v[e];  // x .+= ... (src/inference.jl:284,305)
-                        else
-                            o[e] = v[e];
-                    }
-                }
-            }
-        }
+    for (int i = 0; i < 4; i++) {
+        int m = m0 + 8 * (4 * wave + i) + (lane >> 3);
+        m = m < a.M ? m : a.M - 1;  // rows past the end repeat the last one; their results are not stored
+        gx[i] = (const unsigned char *)(a.act + (int64_t)m * K + 8 * xc);
     }
+    // LDS byte addresses of this lane's operands in stage 0: slice kk holds chunk 2 kk + lane / 32 of its rows
+    unsigned aw[2][4], ax[2][4];
+    {
+        const unsigned base = (unsigned)(size_t)s_all;
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int kk = 0; kk < 4; kk++) {
+                const int c = 2 * kk + (lane >> 5);
+                const int ra = 64 * wn + 32 * i + (lane & 31), rb = 64 * wm + 32 * i + (lane & 31);
+                aw[i][kk] = base + 16u * (unsigned)(ra * 8 + (c ^ (ra & 7)));
+                ax[i][kk] = base + 16384u + 16u * (unsigned)(rb * 8 + (c ^ (rb & 7)));
+            }
+    }
+
+    f32x16 acc[2][JT];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < JT; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+#define PF_ISSUE(STAGE)                                                                                               \
+    do {                                                                                                              \
+        unsigned char *lw = (unsigned char *)s_all + (STAGE) * 32768 + wave * 4096, *lx = lw + 16384;                 \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 0, 0);                       \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 1024, 0);                    \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 2048, 0);                    \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 3072, 0);                    \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[0], (PF_AS3 void *)lx, 16, 0, 0);                    \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[1], (PF_AS3 void *)(lx + 1024), 16, 0, 0);           \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[2], (PF_AS3 void *)(lx + 2048), 16, 0, 0);           \
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[3], (PF_AS3 void *)(lx + 3072), 16, 0, 0);           \
+        gw += 16384;                                                                                                  \
+        gx[0] += 128;                                                                                                 \
+        gx[1] += 128;                                                                                                 \
+        gx[2] += 128;                                                                                                 \
+        gx[3] += 128;                                                                                                 \
+    } while (0)
+
+#define PF_SLICE(OFF, KK)                                                                                   \
+    do {                                                                                                    \
+        pf_u32x4 fa0, fa1, fb0, fb1;                                                                        \
+        PF_LDS_SLICE(OFF, KK);                                                                              \
+        const bf16x8 A0 = __builtin_bit_cast(bf16x8, fa0), A1 = __builtin_bit_cast(bf16x8, fa1);            \
+        const bf16x8 B0 = __builtin_bit_cast(bf16x8, fb0), B1 = __builtin_bit_cast(bf16x8, fb1);            \
+        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, B0, acc[0][0], 0, 0, 0);                    \
+        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, B1, acc[0][1], 0, 0, 0);                    \
+        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, B0, acc[1][0], 0, 0, 0);                    \
+        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, B1, acc[1][1], 0, 0, 0);                    \
+    } while (0)
+
+    // a step: this wavefront's loads of the stage have landed; the barrier says the same of the others' and
+    // that everyone is done reading the other stage, which the next loads then overwrite
+#define PF_STEP(STAGE, OFF, MORE)                            \
+    do {                                                     \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     \
+        __syncthreads();                                     \
+        if (MORE) PF_ISSUE(1 - (STAGE));                     \
+        PF_SLICE(OFF, 0);                                    \
+        PF_SLICE(OFF, 1);                                    \
+        PF_SLICE(OFF, 2);                                    \
+        PF_SLICE(OFF, 3);                                    \
+    } while (0)
+
+    PF_ISSUE(0);
+    int64_t kt = 0;
+    for (; kt + 2 <= nk; kt += 2) {
+        PF_STEP(0, 0, true);
+        PF_STEP(1, 32768, kt + 2 < nk);
+    }
+    if (kt < nk) PF_STEP(0, 0, false);
+#undef PF_STEP
+#undef PF_SLICE
+#undef PF_ISSUE
+    pf_epilogue<EPI, JT>(a, acc, n0, m0, wn, wm, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -557,22 +724,39 @@ static hipError_t pf_gemm_type(hipStream_t s, const PfGemmArgs &a, int epi, int6
     return hipGetLastError();
 }
 
-// w: nseg tensors of one type sharing the input; see PfGemmArgs for the outputs
-hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *act, int M, int64_t K,
-                     int epi, float *out, int64_t ldo, int64_t out_col0, uint16_t *out_bf, int64_t ldb) {
-    PfGemmArgs a{};
+static hipError_t pf_weight_args(PfGemmArgs &a, const DevTensor *w, int nseg, int interleave, int64_t K) {
     int64_t rows = 0;
+    if (nseg < 1 || nseg > 3) return hipErrorInvalidValue;
     for (int i = 0; i < nseg; i++) {
         if (w[i].type != w[0].type || w[i].ne0 != K) return hipErrorInvalidValue;
         a.w[i] = w[i];
         rows += w[i].ne1;
     }
     if (interleave && (nseg != 2 || w[0].ne1 != w[1].ne1)) return hipErrorInvalidValue;
-    if (K % 8 != 0 || M < 1) return hipErrorInvalidValue;
     a.nseg = nseg;
     a.interleave = interleave;
     a.n_rows = rows;
     a.K = K;
+    return hipSuccess;
+}
+
+// w: nseg tensors of one type sharing the input, or (wbf != nullptr) n_rows_bf rows expanded by
+// k_pf_expand; see PfGemmArgs for the outputs
+hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *wbf, int64_t n_rows_bf,
+                     const uint16_t *act, int M, int64_t K, int epi, float *out, int64_t ldo, int64_t out_col0,
+                     uint16_t *out_bf, int64_t ldb) {
+    PfGemmArgs a{};
+    if (wbf) {
+        if (K % 64 != 0) return hipErrorInvalidValue;
+        a.n_rows = n_rows_bf;
+        a.K = K;
+        a.wbf = wbf;
+    } else {
+        const hipError_t e = pf_weight_args(a, w, nseg, interleave, K);
+        if (e != hipSuccess) return e;
+    }
+    if (K % 8 != 0 || M < 1) return hipErrorInvalidValue;
+    const int64_t rows = a.n_rows;
     a.act = act;
     a.M = M;
     a.out = out;
@@ -580,6 +764,18 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
     a.out_col0 = out_col0;
     a.out_bf = out_bf;
     a.ldb = ldb;
+    if (wbf) {
+        const unsigned n_mt = (unsigned)((M + 127) / 128), n_tiles = n_mt * (unsigned)((rows + 127) / 128);
+        const unsigned per = (n_tiles + 7) / 8;
+        const dim3 grid(8 * per);
+        switch (epi) {
+        case PF_STORE: hipLaunchKernelGGL((pf_gemm_bf16_kernel<PF_STORE>), grid, dim3(256), 0, s, a, n_mt, n_tiles, per); break;
+        case PF_RESID: hipLaunchKernelGGL((pf_gemm_bf16_kernel<PF_RESID>), grid, dim3(256), 0, s, a, n_mt, n_tiles, per); break;
+        case PF_SWIGLU: hipLaunchKernelGGL((pf_gemm_bf16_kernel<PF_SWIGLU>), grid, dim3(256), 0, s, a, n_mt, n_tiles, per); break;
+        default: return hipErrorInvalidValue;
+        }
+        return hipGetLastError();
+    }
     // (a 256-position tile, JT = 4, was measured slower: its 272 registers leave one wavefront per SIMD)
     switch (w[0].type) {
     case L2H_TYPE_Q4_K: return pf_gemm_type<L2H_TYPE_Q4_K, 2>(s, a, epi, rows);
@@ -588,6 +784,31 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
     case L2H_TYPE_F32: return pf_gemm_type<L2H_TYPE_F32, 2>(s, a, epi, rows);
     }
     return hipErrorInvalidValue;
+}
+
+// Expands the rows of the nseg tensors (one after another, or w1/w3 rows in turn when interleave is set) to
+// bf16 into the tiled matrix dst (see pf_expand_kernel) from row dst_row0 on; with pad the rows up to the
+// next multiple of 128 are zeroed.  K a multiple of 64.
+hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interleave, int64_t K, uint16_t *dst,
+                       int64_t dst_row0, int pad) {
+    PfGemmArgs a{};
+    const hipError_t e = pf_weight_args(a, w, nseg, interleave, K);
+    if (e != hipSuccess) return e;
+    if (K % 64 != 0) return hipErrorInvalidValue;
+    int64_t rows_end = a.n_rows;
+    if (pad) rows_end = (dst_row0 + a.n_rows + 127) / 128 * 128 - dst_row0;
+    const int64_t n = rows_end * (K >> 5);
+    const dim3 grid((unsigned)((n + 255) / 256));
+#define GO(T) hipLaunchKernelGGL((pf_expand_kernel<T>), grid, dim3(256), 0, s, a, dst, dst_row0, rows_end)
+    switch (w[0].type) {
+    case L2H_TYPE_Q4_K: GO(L2H_TYPE_Q4_K); break;
+    case L2H_TYPE_Q5_K: GO(L2H_TYPE_Q5_K); break;
+    case L2H_TYPE_Q6_K: GO(L2H_TYPE_Q6_K); break;
+    case L2H_TYPE_F32: GO(L2H_TYPE_F32); break;
+    default: return hipErrorInvalidValue;
+    }
+#undef GO
+    return hipGetLastError();
 }
 
 bool k_pf_attention_supported(int hs) { return hs == 32 || hs == 64 || hs == 96 || hs == 128; }

@@ -210,8 +210,11 @@ hipError_t k_pf_rope_table(hipStream_t s, float *cs, int pos0, int M, int half, 
 hipError_t k_pf_rmsnorm(hipStream_t s, const float *X, const float *w, uint16_t *out, int M, int64_t K);
 hipError_t k_pf_rope_scatter(hipStream_t s, const float *raw, const float *cs, uint16_t *Qb, float *kc, float *vc, int M,
                              int pos0, int dim, int kv_dim, int hs, int seq_len, int neox);
-hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *act, int M, int64_t K,
-                     int epi, float *out, int64_t ldo, int64_t out_col0, uint16_t *out_bf, int64_t ldb);
+hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *wbf, int64_t n_rows_bf,
+                     const uint16_t *act, int M, int64_t K, int epi, float *out, int64_t ldo, int64_t out_col0,
+                     uint16_t *out_bf, int64_t ldb);
+hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interleave, int64_t K, uint16_t *dst,
+                       int64_t dst_row0, int pad);
 bool k_pf_attention_supported(int hs);
 hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const float *kc, const float *vc, int M,
                           int qpos0, int hs, int n_heads, int n_kv, int seq_len, int dim);

@@ -114,6 +114,10 @@ class DeviceModel:
         """Bound of the streaming kernel's device-side waits (l2h_model_set_wait_limit)."""
         self.ctx.check(_lib.lib().l2h_model_set_wait_limit(self.handle, int(spins)))
 
+    def set_prefill_copy(self, on):
+        """Whether prefill multiplies from a resident bf16 copy of the weights (l2h_model_set_prefill_copy)."""
+        self.ctx.check(_lib.lib().l2h_model_set_prefill_copy(self.handle, 1 if on else 0))
+
     def forward(self, token, pos, want_logits=True):
         """transformer!(token, pos, ...) (src/inference.jl:222-315): returns (logits, argmax)."""
         logits = np.empty(self.config.vocab_size, np.float32) if want_logits else None

@@ -72,6 +72,32 @@ def test_prefill_then_decode_matches_decode_only(pkg):
     assert err <= 5e-2  # bf16 prompt pass vs q8_K per-token pass: two different roundings of the same sum
 
 
+@pytest.mark.parametrize("case", sorted(CASES))
+def test_prefill_weight_copy_changes_nothing(pkg, case):
+    """l2h_prefill multiplies from a resident bf16 copy of the weights (default) or expands the quantized
+    blocks inside the product kernel (l2h_model_set_prefill_copy(m, 0)): the same bf16 values either way,
+    so logits and cache are equal bit for bit."""
+    from llama2_jl_amd import synth
+    plan, kw = CASES[case]
+    lm = _model(pkg, plan, **kw)
+    cfg = lm.config
+    n = cfg.seq_len - 3
+    prompt = synth.seeded_prompt(8, n, cfg.vocab_size)
+    dev = lm.device()
+    got = []
+    for on in (True, False, True):
+        dev.set_prefill_copy(on)
+        dev.reset()
+        logits, nxt = dev.prefill(prompt, 0)
+        k, v = dev.kv_read(cfg.n_layers - 1, 0, n)
+        got.append((logits.copy(), nxt, k.copy(), v.copy()))
+    dev.set_prefill_copy(True)
+    for other in got[1:]:
+        assert other[1] == got[0][1]
+        assert np.array_equal(other[0], got[0][0])
+        assert np.array_equal(other[2], got[0][2]) and np.array_equal(other[3], got[0][3])
+
+
 def test_prefill_longer_than_one_chunk(pkg, orc):
     """More positions than one internal chunk (2048): the second chunk's queries attend to the first's keys."""
     from llama2_jl_amd import synth
