@@ -600,7 +600,7 @@ __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16
     float mrun = -INFINITY, lrun = 0.0f;
     const int wave_qmax = min(M - 1, q0 + 32 * wave + 31), wg_qmax = min(M - 1, q0 + 127);
     const int nkt = (qpos0 + wg_qmax) / 32 + 1;
-    const float scale = sqrtf((float)HS);
+    const float c_log2 = 1.44269504088896341f / sqrtf((float)HS);
     for (int kt = 0; kt < nkt; kt++) {
         const int key0 = 32 * kt;
         __syncthreads();
@@ -636,32 +636,40 @@ __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16
             const bf16x8 A = as_bf16x8(*(const uint4 *)(s_k + ql * KROW + (16 * kk + 8 * g) * 2));
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, qf[kk], s, 0, 0, 0);
         }
+        // scores in units of log2 e: softmax(s / sqrt(hs)) = 2^(c s - max) / sum with c = log2 e / sqrt(hs)
+        // (att ./= sqrt(hs); softmax!, src/inference.jl:268-270); only a tile on the diagonal needs the mask
         float tmax = -INFINITY;
+        const bool diagonal = key0 + 31 > qpos0 + q0 + 32 * wave || !qvalid;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const int key = key0 + 8 * (r >> 2) + 4 * g + (r & 3);
-            float v = s[r] / scale;  // att ./= sqrt(hs) (src/inference.jl:268)
-            if (!qvalid || key > qpos0 + myq) v = -INFINITY;
+            float v = s[r] * c_log2;
+            if (diagonal) {
+                const int key = key0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (!qvalid || key > qpos0 + myq) v = -INFINITY;
+            }
             s[r] = v;
             tmax = fmaxf(tmax, v);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
         const float mnew = fmaxf(mrun, tmax);
-        const float alpha = (mnew == -INFINITY) ? 1.0f : expf(mrun - mnew);
+        const float msub = (mnew == -INFINITY) ? 0.0f : mnew;  // a row with nothing visible yet: all terms 0
+        const float alpha = __builtin_amdgcn_exp2f(mrun - msub);
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-            const float pv = (s[r] == -INFINITY) ? 0.0f : expf(s[r] - mnew);
+            const float pv = __builtin_amdgcn_exp2f(s[r] - msub);
             s[r] = pv;
             psum += pv;
         }
         psum += __shfl_xor(psum, 32, WAVE);
         lrun = lrun * alpha + psum;
         mrun = mnew;
+        if (__any(alpha != 1.0f)) {  // the running maximum moved for some query of the wavefront
 #pragma unroll
-        for (int d = 0; d < DT; d++)
+            for (int d = 0; d < DT; d++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+                for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+        }
 #pragma unroll
         for (int st = 0; st < 2; st++) {
             const uint4 pb = make_uint4(pack_bf16(s[8 * st], s[8 * st + 1]), pack_bf16(s[8 * st + 2], s[8 * st + 3]),
