@@ -243,6 +243,8 @@ struct l2h_model {
     float *pf_x = nullptr, *pf_raw = nullptr, *pf_cs = nullptr;
     uint16_t *pf_xn = nullptr, *pf_q = nullptr, *pf_att = nullptr, *pf_hb = nullptr;
     int32_t *pf_tok = nullptr;
+    unsigned char *pf_kvt = nullptr;  // one layer's K / V^T as bf16 tiles of 32 keys (k_pf_kv_tiles)
+    int pf_kvt_tiles = 0;             // tiles per KV head
     // bf16 copy of the layer matrices for the prompt pass: per layer q|k|v rows, wo, w1/w3 rows in turn, w2
     int pf_copy_mode = 1;          // 0 never, 1 when it fits
     bool pf_copy_tried = false;
@@ -1022,6 +1024,8 @@ static int prefill_buffers(l2h_model *m, int cap) {
     DA(m->pf_att, (int64_t)cap * c.dim);
     DA(m->pf_hb, (int64_t)cap * c.hidden_dim);
     DA(m->pf_tok, cap);
+    m->pf_kvt_tiles = (c.seq_len + 31) / 32;
+    DA(m->pf_kvt, (int64_t)c.n_kv_heads * m->pf_kvt_tiles * k_pf_kv_tile_bytes(m->hs));
 #undef DA
     m->pf_cap = cap;
     return L2H_OK;
@@ -1100,7 +1104,8 @@ static hipError_t prefill_chunk(l2h_model *m, int M, int pos0) {
         }
         CK(k_pf_rope_scatter(s, m->pf_raw, m->pf_cs, m->pf_q, kc, vc, M, pos0, dim, kvd, m->hs, c.seq_len,
                              c.rope_is_neox));
-        CK(k_pf_attention(s, m->pf_q, m->pf_att, kc, vc, M, pos0, m->hs, c.n_heads, c.n_kv_heads, c.seq_len, dim));
+        CK(k_pf_kv_tiles(s, kc, vc, m->pf_kvt, (pos0 + M + 31) / 32, m->pf_kvt_tiles, m->hs, c.n_kv_heads, c.seq_len));
+        CK(k_pf_attention(s, m->pf_q, m->pf_att, m->pf_kvt, m->pf_kvt_tiles, M, pos0, m->hs, c.n_heads, c.n_kv_heads, dim));
         const DevTensor wo = m->L(l, L2H_WO);
         CK(k_pf_gemm(s, &wo, 1, 0, wb ? wb + m->pf_off_wo : nullptr, dim, m->pf_att, M, dim, PF_RESID, m->pf_x, dim, 0,
                      nullptr, 0));

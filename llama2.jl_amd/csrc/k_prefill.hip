@@ -569,18 +569,94 @@ __global__ __launch_bounds__(256) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigne
 //   running max / sum per query (a lane holds one query: 16 of the 32 keys, the lane 32 further the rest)
 //   O^T += V_tile^T P^T       A = V^T rows (head dims), B = P^T columns (queries)
 // The k index of the second product is a permutation of the keys chosen so that the lane's own
-// probabilities are its B operand without any exchange; V^T is staged in LDS in that key order.
+// probabilities are its B operand without any exchange; V^T is kept in that key order.
+//
+// The fp32 cache is first rewritten, once per layer, as bf16 tiles that are the very bytes the attention
+// workgroups want in LDS (pf_kv_tiles_kernel): per KV head and 32 keys, the K rows (key-major, 16 bytes of
+// padding per row to spread the banks) followed by V^T (head-dim-major, keys permuted, padded rows).  The 64
+// workgroups that need a tile (4 heads of the group x 16 query blocks) then only copy it.
 // ------------------------------------------------------------------------------------------
 template <int HS>
-__global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const float *kc,
-                                                      const float *vc, int M, int qpos0, int n_heads, int n_kv,
-                                                      int seq_len, int dim) {
-    constexpr int KSTEPS = HS / 16, DT = HS / 32;
-    constexpr int KROW = HS * 2 + 16;  // bytes per key row: +16 spreads the rows over the banks
-    constexpr int VROW = 80;           // bytes per head-dim row of V^T: 32 keys + 16 bytes of padding
-    __shared__ __align__(16) unsigned char s_k[32 * KROW];
-    __shared__ __align__(16) unsigned char s_v[HS * VROW];
-    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, g = lane >> 5, ql = lane & 31;
+struct PfKvTile {
+    static constexpr int KROW = HS * 2 + 16;  // bytes per key row
+    static constexpr int VROW = 80;           // bytes per head-dim row of V^T: 32 keys + 16 bytes of padding
+    static constexpr int K_BYTES = 32 * KROW, V_BYTES = HS * VROW;
+    static constexpr int BYTES = (K_BYTES + V_BYTES + 1023) / 1024 * 1024;  // copied 1 KB at a time
+};
+
+template <int HS>
+__global__ __launch_bounds__(256) void pf_kv_tiles_kernel(const float *kc, const float *vc, unsigned char *tiles,
+                                                          int seq_len, int n_tiles_max) {
+    typedef PfKvTile<HS> T;
+    __shared__ __align__(16) unsigned char s_img[T::BYTES];
+    unsigned char *s_k = s_img, *s_v = s_img + T::K_BYTES;
+    const int t = threadIdx.x, kt = blockIdx.x, kvh = blockIdx.y, key0 = 32 * kt;
+    for (int c = t; c < T::BYTES / 16; c += 256) ((uint4 *)s_img)[c] = make_uint4(0, 0, 0, 0);
+    __syncthreads();
+    for (int idx = t; idx < 32 * (HS / 4); idx += 256) {  // K tile -> bf16 rows
+        const int key = idx & 31, i4 = idx >> 5;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (key0 + key < seq_len) v = *(const float4 *)(kc + (((int64_t)kvh * (HS / 4) + i4) * seq_len + key0 + key) * 4);
+        uint2 w;
+        w.x = pack_bf16(v.x, v.y);
+        w.y = pack_bf16(v.z, v.w);
+        *(uint2 *)(s_k + key * T::KROW + i4 * 8) = w;
+    }
+    for (int idx = t; idx < 32 * (HS / 4); idx += 256) {  // V tile -> bf16, transposed, keys permuted
+        const int d4 = idx % (HS / 4), key = idx / (HS / 4);
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (key0 + key < seq_len) v = *(const float4 *)(vc + ((int64_t)kvh * seq_len + key0 + key) * HS + 4 * d4);
+        // key = 16 s + 8 a + 4 g + b  ->  slot 16 s + 8 g + 4 a + b
+        const int rem = key & 15;
+        const int slot = (key & 16) + 8 * ((rem >> 2) & 1) + 4 * (rem >> 3) + (rem & 3);
+        __bf16 *dst = (__bf16 *)(s_v + (4 * d4) * T::VROW) + slot;
+        dst[0] = (__bf16)v.x;
+        dst[T::VROW / 2] = (__bf16)v.y;
+        dst[T::VROW] = (__bf16)v.z;
+        dst[3 * T::VROW / 2] = (__bf16)v.w;
+    }
+    __syncthreads();
+    uint4 *dst = (uint4 *)(tiles + ((int64_t)kvh * n_tiles_max + kt) * T::BYTES);
+    for (int c = t; c < T::BYTES / 16; c += 256) dst[c] = ((const uint4 *)s_img)[c];
+}
+
+typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
+
+// N 16-byte LDS reads STRIDE bytes apart, complete on return: the reads and their wait are one statement, so
+// the compiler never sees a register of a read under way, and (being asm) the reads are not made to wait for
+// the tile copies in flight into the other stage
+template <int N, int STRIDE>
+__device__ __forceinline__ void pf_lds_read(pf_u32x4 (&o)[4], unsigned addr) {
+    static_assert(N >= 1 && N <= 4 && 3 * STRIDE < 65536, "");
+    if constexpr (N == 1)
+        asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(o[0]) : "v"(addr) : "memory");
+    else if constexpr (N == 2)
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(o[0]), "=&v"(o[1])
+                     : "v"(addr), "n"(STRIDE)
+                     : "memory");
+    else if constexpr (N == 3)
+        asm volatile("ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:%4\n\tds_read_b128 %2, %3 offset:%5\n\t"
+                     "s_waitcnt lgkmcnt(0)"
+                     : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2])
+                     : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE)
+                     : "memory");
+    else
+        asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:%5\n\tds_read_b128 %2, %4 offset:%6\n\t"
+                     "ds_read_b128 %3, %4 offset:%7\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3])
+                     : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE), "n"(3 * STRIDE)
+                     : "memory");
+}
+
+template <int HS>
+__global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles,
+                                                      int n_tiles_max, int M, int qpos0, int n_heads, int n_kv, int dim) {
+    typedef PfKvTile<HS> T;
+    constexpr int KSTEPS = HS / 16, DT = HS / 32, KH = KSTEPS / 2;
+    // two stages: the copy of tile kt + 1 is in flight during the products of tile kt, one barrier per tile
+    __shared__ __align__(16) unsigned char s_t[2 * T::BYTES];
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), g = lane >> 5, ql = lane & 31;
     const int h = blockIdx.y, kvh = h / (n_heads / n_kv);
     const int q0 = blockIdx.x * 128;
     const int myq = q0 + 32 * wave + ql;
@@ -601,40 +677,37 @@ __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16
     const int wave_qmax = min(M - 1, q0 + 32 * wave + 31), wg_qmax = min(M - 1, q0 + 127);
     const int nkt = (qpos0 + wg_qmax) / 32 + 1;
     const float c_log2 = 1.44269504088896341f / sqrtf((float)HS);
+    const unsigned char *src = tiles + (int64_t)kvh * n_tiles_max * T::BYTES + lane * 16;
+    const unsigned lds0 = (unsigned)(size_t)s_t;
+    const unsigned k_addr = lds0 + (unsigned)(ql * T::KROW + 16 * g), v_addr = lds0 + (unsigned)(T::K_BYTES + ql * T::VROW + 16 * g);
+    // this wavefront copies KB wave, wave + 4, ... of a tile, a KB per load (16 bytes per lane, lane order)
+    auto issue = [&](int stage, int kt) {
+        const unsigned char *gp = src + (int64_t)kt * T::BYTES;
+        unsigned char *lp = s_t + stage * T::BYTES;
+#pragma unroll
+        for (int b = 0; b < T::BYTES / 1024; b += 4)
+            if (b + wave < T::BYTES / 1024)
+                __builtin_amdgcn_global_load_lds((const PF_AS1 void *)(gp + (b + wave) * 1024),
+                                                 (PF_AS3 void *)(lp + (b + wave) * 1024), 16, 0, 0);
+    };
+    issue(0, 0);
     for (int kt = 0; kt < nkt; kt++) {
-        const int key0 = 32 * kt;
-        __syncthreads();
-        for (int idx = t; idx < 32 * (HS / 4); idx += 256) {  // K tile -> bf16 rows
-            const int key = idx & 31, i4 = idx >> 5;
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (key0 + key < seq_len) v = *(const float4 *)(kc + (((int64_t)kvh * (HS / 4) + i4) * seq_len + key0 + key) * 4);
-            uint2 w;
-            w.x = pack_bf16(v.x, v.y);
-            w.y = pack_bf16(v.z, v.w);
-            *(uint2 *)(s_k + key * KROW + i4 * 8) = w;
-        }
-        for (int idx = t; idx < 32 * (HS / 4); idx += 256) {  // V tile -> bf16, transposed, keys permuted
-            const int d4 = idx % (HS / 4), key = idx / (HS / 4);
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (key0 + key < seq_len) v = *(const float4 *)(vc + ((int64_t)kvh * seq_len + key0 + key) * HS + 4 * d4);
-            // key = 16 s + 8 a + 4 g + b  ->  slot 16 s + 8 g + 4 a + b
-            const int rem = key & 15;
-            const int slot = (key & 16) + 8 * ((rem >> 2) & 1) + 4 * (rem >> 3) + (rem & 3);
-            __bf16 *dst = (__bf16 *)(s_v + (4 * d4) * VROW) + slot;
-            dst[0] = (__bf16)v.x;
-            dst[VROW / 2] = (__bf16)v.y;
-            dst[VROW] = (__bf16)v.z;
-            dst[3 * VROW / 2] = (__bf16)v.w;
-        }
-        __syncthreads();
+        const int key0 = 32 * kt, stage = kt & 1;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wavefront's part of the tile has landed
+        __syncthreads();                                  // ... and everyone's; the other stage is free
+        if (kt + 1 < nkt) issue(stage ^ 1, kt + 1);
         if (key0 > qpos0 + wave_qmax) continue;  // every key of the tile lies in this wavefront's future
+        const unsigned so = (unsigned)(stage * T::BYTES);
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.0f;
 #pragma unroll
-        for (int kk = 0; kk < KSTEPS; kk++) {
-            const bf16x8 A = as_bf16x8(*(const uint4 *)(s_k + ql * KROW + (16 * kk + 8 * g) * 2));
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, qf[kk], s, 0, 0, 0);
+        for (int half = 0; half < 2; half++) {
+            pf_u32x4 ka[4];
+            pf_lds_read<KH, 32>(ka, k_addr + so + (unsigned)(32 * KH * half));
+#pragma unroll
+            for (int i = 0; i < KH; i++)
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qf[KH * half + i], s, 0, 0, 0);
         }
         // scores in units of log2 e: softmax(s / sqrt(hs)) = 2^(c s - max) / sum with c = log2 e / sqrt(hs)
         // (att ./= sqrt(hs); softmax!, src/inference.jl:268-270); only a tile on the diagonal needs the mask
@@ -675,11 +748,11 @@ __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16
             const uint4 pb = make_uint4(pack_bf16(s[8 * st], s[8 * st + 1]), pack_bf16(s[8 * st + 2], s[8 * st + 3]),
                                         pack_bf16(s[8 * st + 4], s[8 * st + 5]), pack_bf16(s[8 * st + 6], s[8 * st + 7]));
             const bf16x8 B = as_bf16x8(pb);
+            pf_u32x4 va[4];
+            pf_lds_read<DT, 32 * T::VROW>(va, v_addr + so + (unsigned)(32 * st));
 #pragma unroll
-            for (int d = 0; d < DT; d++) {
-                const bf16x8 A = as_bf16x8(*(const uint4 *)(s_v + (32 * d + ql) * VROW + (16 * st + 8 * g) * 2));
-                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A, B, o[d], 0, 0, 0);
-            }
+            for (int d = 0; d < DT; d++)
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[d]), B, o[d], 0, 0, 0);
         }
     }
     if (!qvalid) return;
@@ -821,10 +894,39 @@ hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interlea
 
 bool k_pf_attention_supported(int hs) { return hs == 32 || hs == 64 || hs == 96 || hs == 128; }
 
-hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const float *kc, const float *vc, int M,
-                          int qpos0, int hs, int n_heads, int n_kv, int seq_len, int dim) {
+int64_t k_pf_kv_tile_bytes(int hs) {
+    switch (hs) {
+    case 32: return PfKvTile<32>::BYTES;
+    case 64: return PfKvTile<64>::BYTES;
+    case 96: return PfKvTile<96>::BYTES;
+    case 128: return PfKvTile<128>::BYTES;
+    }
+    return 0;
+}
+
+// tiles: n_kv x n_tiles_max tiles of k_pf_kv_tile_bytes(hs); the first n_tiles of every KV head are rewritten
+hipError_t k_pf_kv_tiles(hipStream_t s, const float *kc, const float *vc, unsigned char *tiles, int n_tiles,
+                         int n_tiles_max, int hs, int n_kv, int seq_len) {
+    if (n_tiles < 1 || n_tiles > n_tiles_max) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)n_tiles, (unsigned)n_kv);
+#define GO(HS) hipLaunchKernelGGL((pf_kv_tiles_kernel<HS>), grid, dim3(256), 0, s, kc, vc, tiles, seq_len, n_tiles_max)
+    switch (hs) {
+    case 32: GO(32); break;
+    case 64: GO(64); break;
+    case 96: GO(96); break;
+    case 128: GO(128); break;
+    default: return hipErrorInvalidValue;
+    }
+#undef GO
+    return hipGetLastError();
+}
+
+// tiles must hold the keys 0 .. qpos0 + M - 1 (k_pf_kv_tiles)
+hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles, int n_tiles_max,
+                          int M, int qpos0, int hs, int n_heads, int n_kv, int dim) {
+    if ((qpos0 + M + 31) / 32 > n_tiles_max) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((M + 127) / 128), (unsigned)n_heads);
-#define GO(HS) hipLaunchKernelGGL((pf_attn_kernel<HS>), grid, dim3(256), 0, s, Qb, Att, kc, vc, M, qpos0, n_heads, n_kv, seq_len, dim)
+#define GO(HS) hipLaunchKernelGGL((pf_attn_kernel<HS>), grid, dim3(256), 0, s, Qb, Att, tiles, n_tiles_max, M, qpos0, n_heads, n_kv, dim)
     switch (hs) {
     case 32: GO(32); break;
     case 64: GO(64); break;

@@ -216,8 +216,11 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
 hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interleave, int64_t K, uint16_t *dst,
                        int64_t dst_row0, int pad);
 bool k_pf_attention_supported(int hs);
-hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const float *kc, const float *vc, int M,
-                          int qpos0, int hs, int n_heads, int n_kv, int seq_len, int dim);
+int64_t k_pf_kv_tile_bytes(int hs);
+hipError_t k_pf_kv_tiles(hipStream_t s, const float *kc, const float *vc, unsigned char *tiles, int n_tiles,
+                         int n_tiles_max, int hs, int n_kv, int seq_len);
+hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles, int n_tiles_max,
+                          int M, int qpos0, int hs, int n_heads, int n_kv, int dim);
 
 static inline int64_t l2h_gguf_block_bytes(int type) {
     switch (type) {
