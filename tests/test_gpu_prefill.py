@@ -72,13 +72,18 @@ def test_prefill_then_decode_matches_decode_only(pkg):
     assert err <= 5e-2  # bf16 prompt pass vs q8_K per-token pass: two different roundings of the same sum
 
 
-@pytest.mark.parametrize("case", sorted(CASES))
+# a wider model than CASES holds: many K steps per product, several position tiles, the last one part filled
+WIDE = ("PLAN_Q5_K_M", dict(dim=512, hidden_dim=1536, n_layers=2, n_heads=8, n_kv_heads=4, vocab_size=512, seq_len=330,
+                            rope_freq_base=10000.0, rope_is_neox=False))
+
+
+@pytest.mark.parametrize("case", sorted(CASES) + ["wide"])
 def test_prefill_weight_copy_changes_nothing(pkg, case):
     """l2h_prefill multiplies from a resident bf16 copy of the weights (default) or expands the quantized
     blocks inside the product kernel (l2h_model_set_prefill_copy(m, 0)): the same bf16 values either way,
     so logits and cache are equal bit for bit."""
     from llama2_jl_amd import synth
-    plan, kw = CASES[case]
+    plan, kw = WIDE if case == "wide" else CASES[case]
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
     n = cfg.seq_len - 3
