@@ -255,6 +255,12 @@ __device__ __forceinline__ void pf_convert(const PfRaw &r, const PfRowPtr &p, in
     for (int c = 0; c < 4; c++) out[c] = make_uint4(pk[4 * c], pk[4 * c + 1], pk[4 * c + 2], pk[4 * c + 3]);
 }
 
+// Placement of the 16-byte chunks of a 128-byte tile row in LDS.  The LDS has 64 banks of 4 bytes and serves
+// 16-byte accesses 16 lanes at a time; lanes read one chunk index of 16 consecutive rows, which the
+// exclusive-or with (r >> 1) % 8 sends to the 16 different 16-byte slots of the 256-byte bank row (the row's
+// parity picks the half).  With r % 8 instead, rows r and r + 8 collide: half the LDS cycles were conflicts.
+__host__ __device__ __forceinline__ int pf_swz(int r) { return (r >> 1) & 7; }
+
 // the stream pointers of logical weight row L
 template <int TYPE>
 __device__ __forceinline__ void pf_row_ptr(const PfGemmArgs &a, int64_t L, PfRow &lr, PfRowPtr &rp) {
@@ -276,7 +282,7 @@ __device__ __forceinline__ void pf_row_ptr(const PfGemmArgs &a, int64_t L, PfRow
 // One thread expands 32 consecutive weights of one logical row to bf16, with the arithmetic the fused
 // product kernel uses on them.  The destination is a sequence of 16 KB tiles, tile (nt, kt) = weight
 // rows 128 nt.. x inputs 64 kt.. at ((nt K/64) + kt) * 8192 elements, and inside a tile the image the
-// product kernels keep in LDS: the 16-byte chunk c of row r at chunk index 8 r + (c ^ (r & 7)).  Logical
+// product kernels keep in LDS: the 16-byte chunk c of row r at chunk index 8 r + (c ^ pf_swz(r)).  Logical
 // row L goes to row dst_row0 + L; rows from n_rows up to rows_end (padding of the last tile) are zero.
 template <int TYPE>
 __global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *dst, int64_t dst_row0, int64_t rows_end) {
@@ -297,7 +303,7 @@ __global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *
 #pragma unroll
     for (int cc = 0; cc < 4; cc++) {
         const int c = 4 * (int)(g & 1) + cc;
-        tile[r * 8 + (c ^ (r & 7))] = wv[cc];
+        tile[r * 8 + (c ^ pf_swz(r))] = wv[cc];
     }
 }
 
@@ -346,7 +352,7 @@ __device__ __forceinline__ void pf_epilogue(const PfGemmArgs &a, f32x16 (&acc)[2
 // 2 x 2 tiles of 32 x 32.  Weights are the A operand (rows), positions the B operand (columns), so
 // a lane ends up holding one position and groups of 4 consecutive weight rows: neighbours such as a
 // w1/w3 pair sit in one lane.  LDS rows are 64 bf16 = 8 chunks of 16 bytes, chunk c of row r kept at
-// c ^ (r & 7) so that the 8 lanes of a 128-byte access phase hit distinct banks.
+// c ^ pf_swz(r).
 template <int TYPE, int EPI, int JT>
 __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
     constexpr int MT = 64 * JT;  // positions per workgroup: 2 wavefront columns x JT tiles of 32
@@ -401,11 +407,11 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
             q.valid = rp.valid && (k0 + 32 * whh < K);
             pf_convert<TYPE>(raw, q, lr.row, k0 + 32 * whh, K, wv);
 #pragma unroll
-            for (int c = 0; c < 4; c++) s_w[wr * 8 + ((4 * whh + c) ^ (wr & 7))] = wv[c];
+            for (int c = 0; c < 4; c++) s_w[wr * 8 + ((4 * whh + c) ^ pf_swz(wr))] = wv[c];
 #pragma unroll
             for (int i = 0; i < XL; i++) {
                 const int r = (t >> 3) + 32 * i;
-                s_x[r * 8 + (xc ^ (r & 7))] = xreg[i];
+                s_x[r * 8 + (xc ^ pf_swz(r))] = xreg[i];
             }
         }
         __syncthreads();
@@ -417,12 +423,12 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 const int ra = 64 * wn + 32 * i + (lane & 31);
-                A[i] = as_bf16x8(s_w[ra * 8 + (c ^ (ra & 7))]);
+                A[i] = as_bf16x8(s_w[ra * 8 + (c ^ pf_swz(ra))]);
             }
 #pragma unroll
             for (int j = 0; j < JT; j++) {
                 const int rb = 32 * JT * wm + 32 * j + (lane & 31);
-                B[j] = as_bf16x8(s_x[rb * 8 + (c ^ (rb & 7))]);
+                B[j] = as_bf16x8(s_x[rb * 8 + (c ^ pf_swz(rb))]);
             }
 #pragma unroll
             for (int i = 0; i < 2; i++)
@@ -441,7 +447,7 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 // The same product from weights expanded beforehand (pf_expand_kernel): no arithmetic on the operands.
 // Both tiles of a K step travel from global memory straight into LDS (16 bytes per lane and load, a
 // wavefront's load filling 1 KB of LDS in lane order): the weight tile is a linear copy of its 16 KB
-// image, the position tile gets the c ^ (r & 7) placement by the choice of the address each lane reads.
+// image, the position tile gets the c ^ pf_swz(r) placement by the choice of the address each lane reads.
 // Two LDS stages: the loads of step kt + 1 are in flight during the products of step kt, one barrier
 // per step.  Workgroups are dealt to the 8 XCDs in turn, so workgroup w takes tile (w % 8) * per + w / 8:
 // each XCD works through a contiguous run of tiles, positions fastest, and the workgroups that share a
@@ -474,14 +480,14 @@ __global__ __launch_bounds__(256) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigne
     // weights: this wavefront copies bytes [4096 wave, +4096) of every tile, 1 KB per load
     const unsigned char *gw = (const unsigned char *)(a.wbf + (int64_t)nt * nk * 8192) + wave * 4096 + lane * 16;
     // positions: load i of this wavefront fills chunks 64 (4 wave + i) + lane: row 8 (4 wave + i) + lane / 8,
-    // placed chunk lane % 8 = the data chunk (lane % 8) ^ (row % 8)
-    const int xc = (lane & 7) ^ ((lane >> 3) & 7);
+    // placed chunk lane % 8 = the data chunk (lane % 8) ^ pf_swz(row)
     const unsigned char *gx[4];
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-        int m = m0 + 8 * (4 * wave + i) + (lane >> 3);
+        const int r = 8 * (4 * wave + i) + (lane >> 3);
+        int m = m0 + r;
         m = m < a.M ? m : a.M - 1;  // rows past the end repeat the last one; their results are not stored
-        gx[i] = (const unsigned char *)(a.act + (int64_t)m * K + 8 * xc);
+        gx[i] = (const unsigned char *)(a.act + (int64_t)m * K + 8 * ((lane & 7) ^ pf_swz(r)));
     }
     // LDS byte addresses of this lane's operands in stage 0: slice kk holds chunk 2 kk + lane / 32 of its rows
     unsigned aw[2][4], ax[2][4];
@@ -493,8 +499,8 @@ __global__ __launch_bounds__(256) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigne
             for (int kk = 0; kk < 4; kk++) {
                 const int c = 2 * kk + (lane >> 5);
                 const int ra = 64 * wn + 32 * i + (lane & 31), rb = 64 * wm + 32 * i + (lane & 31);
-                aw[i][kk] = base + 16u * (unsigned)(ra * 8 + (c ^ (ra & 7)));
-                ax[i][kk] = base + 16384u + 16u * (unsigned)(rb * 8 + (c ^ (rb & 7)));
+                aw[i][kk] = base + 16u * (unsigned)(ra * 8 + (c ^ pf_swz(ra)));
+                ax[i][kk] = base + 16384u + 16u * (unsigned)(rb * 8 + (c ^ pf_swz(rb)));
             }
     }
 
