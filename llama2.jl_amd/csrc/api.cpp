@@ -1041,11 +1041,11 @@ static int prefill_weights(l2h_model *m) {
     const l2h_config &c = m->c;
     const int64_t dim = c.dim, kvd = m->kv_dim, hid = c.hidden_dim;
     if (dim % 64 != 0 || hid % 64 != 0) return L2H_OK;
-    auto pad128 = [](int64_t r) { return (r + 127) / 128 * 128; };
-    m->pf_off_wo = pad128(dim + 2 * kvd) * dim;
-    m->pf_off_w13 = m->pf_off_wo + pad128(dim) * dim;
-    m->pf_off_w2 = m->pf_off_w13 + pad128(2 * hid) * dim;
-    m->pf_wbf_layer = m->pf_off_w2 + pad128(dim) * hid;
+    auto pad_rows = [](int64_t r) { return (r + 255) / 256 * 256; };  // whole tiles of 256 rows
+    m->pf_off_wo = pad_rows(dim + 2 * kvd) * dim;
+    m->pf_off_w13 = m->pf_off_wo + pad_rows(dim) * dim;
+    m->pf_off_w2 = m->pf_off_w13 + pad_rows(2 * hid) * dim;
+    m->pf_wbf_layer = m->pf_off_w2 + pad_rows(dim) * hid;
     const size_t bytes = (size_t)m->pf_wbf_layer * c.n_layers * 2;
     size_t free_b = 0, total_b = 0;
     HIPCHK(m->ctx, hipMemGetInfo(&free_b, &total_b));

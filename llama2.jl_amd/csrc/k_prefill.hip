@@ -280,9 +280,9 @@ __device__ __forceinline__ void pf_row_ptr(const PfGemmArgs &a, int64_t L, PfRow
 }
 
 // One thread expands 32 consecutive weights of one logical row to bf16, with the arithmetic the fused
-// product kernel uses on them.  The destination is a sequence of 16 KB tiles, tile (nt, kt) = weight
-// rows 128 nt.. x inputs 64 kt.. at ((nt K/64) + kt) * 8192 elements, and inside a tile the image the
-// product kernels keep in LDS: the 16-byte chunk c of row r at chunk index 8 r + (c ^ pf_swz(r)).  Logical
+// product kernel uses on them.  The destination is a sequence of 32 KB tiles, tile (nt, kt) = weight
+// rows 256 nt.. x inputs 64 kt.. at ((nt K/64) + kt) * 16384 elements, and inside a tile the image the
+// product kernel keeps in LDS: the 16-byte chunk c of row r at chunk index 8 r + (c ^ pf_swz(r)).  Logical
 // row L goes to row dst_row0 + L; rows from n_rows up to rows_end (padding of the last tile) are zero.
 template <int TYPE>
 __global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *dst, int64_t dst_row0, int64_t rows_end) {
@@ -297,9 +297,9 @@ __global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *
     pf_load_raw<TYPE>(raw, rp, lr.row, k0, a.K);
     uint4 wv[4];
     pf_convert<TYPE>(raw, rp, lr.row, k0, a.K, wv);
-    const int64_t R = dst_row0 + L, nt = R >> 7, kt = g >> 1;
-    const int r = (int)(R & 127);
-    uint4 *tile = (uint4 *)(dst + (nt * nk + kt) * 8192);
+    const int64_t R = dst_row0 + L, nt = R >> 8, kt = g >> 1;
+    const int r = (int)(R & 255);
+    uint4 *tile = (uint4 *)(dst + (nt * nk + kt) * 16384);
 #pragma unroll
     for (int cc = 0; cc < 4; cc++) {
         const int c = 4 * (int)(g & 1) + cc;
@@ -445,64 +445,61 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #define PF_AS3 __attribute__((address_space(3)))
 
 // The same product from weights expanded beforehand (pf_expand_kernel): no arithmetic on the operands.
-// Both tiles of a K step travel from global memory straight into LDS (16 bytes per lane and load, a
-// wavefront's load filling 1 KB of LDS in lane order): the weight tile is a linear copy of its 16 KB
-// image, the position tile gets the c ^ pf_swz(r) placement by the choice of the address each lane reads.
-// Two LDS stages: the loads of step kt + 1 are in flight during the products of step kt, one barrier
-// per step.  Workgroups are dealt to the 8 XCDs in turn, so workgroup w takes tile (w % 8) * per + w / 8:
-// each XCD works through a contiguous run of tiles, positions fastest, and the workgroups that share a
-// weight tile share an L2.
+// What bounds such a product on this chip is the path from L2 into the CU (64 bytes per clock): a 128 x 128
+// tile fetches 32 KB per 64 inputs and keeps that path busier than the matrix cores.  So the tile is 256
+// weight rows x 64 JT positions (JT = 4: 256, half the bytes per product; JT = 2: 128, for matrices with
+// too few rows to give every CU a 256 x 256 tile), worked on by 8 wavefronts, 4 row groups x 2 position
+// groups, each 64 rows x 32 JT positions.  Both operand tiles of a K step travel from global memory
+// straight into LDS (16 bytes per lane and load, a wavefront's load filling 1 KB in lane order): the weight
+// tile is a linear copy of its 32 KB image, the position tile gets the c ^ pf_swz(r) placement by the choice
+// of the address each lane reads.  Two LDS stages: the loads of step kt + 1 are in flight during the products
+// of step kt, one barrier per step.  Workgroups are dealt to the 8 XCDs in turn, so workgroup w takes tile
+// (w % 8) * per + w / 8: each XCD works through a contiguous run of tiles, positions fastest, and the
+// workgroups that share a weight tile share an L2.
 typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 
-// the operands of one 16-wide slice of the K step (2 weight row groups, 2 position groups) from LDS stage
-// at byte offset OFF; loads and their wait are one statement, so no register of a load under way is visible
-#define PF_LDS_SLICE(OFF, KK)                                                                                       \
-    asm volatile("ds_read_b128 %0, %4 offset:" #OFF "\n\tds_read_b128 %1, %5 offset:" #OFF                         \
-                 "\n\tds_read_b128 %2, %6 offset:" #OFF "\n\tds_read_b128 %3, %7 offset:" #OFF                     \
-                 "\n\ts_waitcnt lgkmcnt(0)"                                                                         \
-                 : "=&v"(fa0), "=&v"(fa1), "=&v"(fb0), "=&v"(fb1)                                                   \
-                 : "v"(aw[0][KK]), "v"(aw[1][KK]), "v"(ax[0][KK]), "v"(ax[1][KK])                                   \
-                 : "memory")
-
-template <int EPI>
-__global__ __launch_bounds__(256) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned n_mt, unsigned n_tiles, unsigned per) {
-    constexpr int JT = 2;
-    // two stages of 32 KB: weight tile (16 KB), then position tile (16 KB)
-    __shared__ uint4 s_all[4096];
+template <int EPI, int JT>
+__global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned n_mt, unsigned n_tiles, unsigned per) {
+    constexpr int MT = 64 * JT;                   // positions per workgroup
+    constexpr int STAGE = 32768 + MT * 128;       // bytes: weight tile, then position tile
+    extern __shared__ uint4 s_all[];              // two stages
     const unsigned tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
     if (tile >= n_tiles) return;
-    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wn = wave & 1, wm = wave >> 1;
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wn = wave & 3, wm = wave >> 2;
     const unsigned mt = tile % n_mt, nt = tile / n_mt;
-    const int64_t n0 = (int64_t)nt * 128;
-    const int m0 = (int)mt * 128;
+    const int64_t n0 = (int64_t)nt * 256;
+    const int m0 = (int)mt * MT;
     const int64_t K = a.K, nk = K >> 6;
 
     // weights: this wavefront copies bytes [4096 wave, +4096) of every tile, 1 KB per load
-    const unsigned char *gw = (const unsigned char *)(a.wbf + (int64_t)nt * nk * 8192) + wave * 4096 + lane * 16;
-    // positions: load i of this wavefront fills chunks 64 (4 wave + i) + lane: row 8 (4 wave + i) + lane / 8,
+    const unsigned char *gw = (const unsigned char *)(a.wbf + (int64_t)nt * nk * 16384) + wave * 4096 + lane * 16;
+    // positions: load i of this wavefront fills chunks 64 (JT wave + i) + lane: row 8 (JT wave + i) + lane / 8,
     // placed chunk lane % 8 = the data chunk (lane % 8) ^ pf_swz(row)
-    const unsigned char *gx[4];
+    const unsigned char *gx[JT];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int r = 8 * (4 * wave + i) + (lane >> 3);
+    for (int i = 0; i < JT; i++) {
+        const int r = 8 * (JT * wave + i) + (lane >> 3);
         int m = m0 + r;
         m = m < a.M ? m : a.M - 1;  // rows past the end repeat the last one; their results are not stored
         gx[i] = (const unsigned char *)(a.act + (int64_t)m * K + 8 * ((lane & 7) ^ pf_swz(r)));
     }
-    // LDS byte addresses of this lane's operands in stage 0: slice kk holds chunk 2 kk + lane / 32 of its rows
-    unsigned aw[2][4], ax[2][4];
-    {
-        const unsigned base = (unsigned)(size_t)s_all;
+    // LDS byte offsets of this lane's operands inside a stage: slice kk holds chunk 2 kk + lane / 32 of its rows
+    unsigned aw[2][4], ax[JT][4];
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+    for (int kk = 0; kk < 4; kk++) {
+        const int c = 2 * kk + (lane >> 5);
 #pragma unroll
-            for (int kk = 0; kk < 4; kk++) {
-                const int c = 2 * kk + (lane >> 5);
-                const int ra = 64 * wn + 32 * i + (lane & 31), rb = 64 * wm + 32 * i + (lane & 31);
-                aw[i][kk] = base + 16u * (unsigned)(ra * 8 + (c ^ pf_swz(ra)));
-                ax[i][kk] = base + 16384u + 16u * (unsigned)(rb * 8 + (c ^ pf_swz(rb)));
-            }
+        for (int i = 0; i < 2; i++) {
+            const int ra = 64 * wn + 32 * i + (lane & 31);
+            aw[i][kk] = 16u * (unsigned)(ra * 8 + (c ^ pf_swz(ra)));
+        }
+#pragma unroll
+        for (int j = 0; j < JT; j++) {
+            const int rb = 32 * JT * wm + 32 * j + (lane & 31);
+            ax[j][kk] = 32768u + 16u * (unsigned)(rb * 8 + (c ^ pf_swz(rb)));
+        }
     }
+    const unsigned lds0 = (unsigned)(size_t)s_all;
 
     f32x16 acc[2][JT];
 #pragma unroll
@@ -512,59 +509,62 @@ __global__ __launch_bounds__(256) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigne
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-#define PF_ISSUE(STAGE)                                                                                               \
-    do {                                                                                                              \
-        unsigned char *lw = (unsigned char *)s_all + (STAGE) * 32768 + wave * 4096, *lx = lw + 16384;                 \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 0, 0);                       \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 1024, 0);                    \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 2048, 0);                    \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 3072, 0);                    \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[0], (PF_AS3 void *)lx, 16, 0, 0);                    \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[1], (PF_AS3 void *)(lx + 1024), 16, 0, 0);           \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[2], (PF_AS3 void *)(lx + 2048), 16, 0, 0);           \
-        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[3], (PF_AS3 void *)(lx + 3072), 16, 0, 0);           \
-        gw += 16384;                                                                                                  \
-        gx[0] += 128;                                                                                                 \
-        gx[1] += 128;                                                                                                 \
-        gx[2] += 128;                                                                                                 \
-        gx[3] += 128;                                                                                                 \
-    } while (0)
+    auto issue = [&](int stage) {
+        unsigned char *lw = (unsigned char *)s_all + stage * STAGE + wave * 4096;
+        unsigned char *lx = (unsigned char *)s_all + stage * STAGE + 32768 + wave * (1024 * JT);
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 1024, 0);
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 2048, 0);
+        __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gw, (PF_AS3 void *)lw, 16, 3072, 0);
+#pragma unroll
+        for (int i = 0; i < JT; i++) {
+            __builtin_amdgcn_global_load_lds((const PF_AS1 void *)gx[i], (PF_AS3 void *)(lx + 1024 * i), 16, 0, 0);
+            gx[i] += 128;
+        }
+        gw += 32768;
+    };
 
-#define PF_SLICE(OFF, KK)                                                                                   \
-    do {                                                                                                    \
-        pf_u32x4 fa0, fa1, fb0, fb1;                                                                        \
-        PF_LDS_SLICE(OFF, KK);                                                                              \
-        const bf16x8 A0 = __builtin_bit_cast(bf16x8, fa0), A1 = __builtin_bit_cast(bf16x8, fa1);            \
-        const bf16x8 B0 = __builtin_bit_cast(bf16x8, fb0), B1 = __builtin_bit_cast(bf16x8, fb1);            \
-        acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, B0, acc[0][0], 0, 0, 0);                    \
-        acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, B1, acc[0][1], 0, 0, 0);                    \
-        acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, B0, acc[1][0], 0, 0, 0);                    \
-        acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, B1, acc[1][1], 0, 0, 0);                    \
-    } while (0)
+    // one 16-wide slice: operands from the stage at LDS address sb (reads and their wait are one statement, so
+    // no register of a read under way is visible; being asm, they are not made to wait for the copies in flight
+    // into the other stage), then 2 JT products
+    auto slice = [&](unsigned sb, int kk) {
+        pf_u32x4 fa0, fa1, fb[JT];
+        if constexpr (JT == 2) {
+            asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
+                         "\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&v"(fa0), "=&v"(fa1), "=&v"(fb[0]), "=&v"(fb[1])
+                         : "v"(sb + aw[0][kk]), "v"(sb + aw[1][kk]), "v"(sb + ax[0][kk]), "v"(sb + ax[1][kk])
+                         : "memory");
+        } else {
+            asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %7\n\tds_read_b128 %2, %8\n\tds_read_b128 %3, %9"
+                         "\n\tds_read_b128 %4, %10\n\tds_read_b128 %5, %11\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&v"(fa0), "=&v"(fa1), "=&v"(fb[0]), "=&v"(fb[1]), "=&v"(fb[2]), "=&v"(fb[3])
+                         : "v"(sb + aw[0][kk]), "v"(sb + aw[1][kk]), "v"(sb + ax[0][kk]), "v"(sb + ax[1][kk]),
+                           "v"(sb + ax[2][kk]), "v"(sb + ax[3][kk])
+                         : "memory");
+        }
+        const bf16x8 A0 = __builtin_bit_cast(bf16x8, fa0), A1 = __builtin_bit_cast(bf16x8, fa1);
+#pragma unroll
+        for (int j = 0; j < JT; j++) {
+            const bf16x8 B = __builtin_bit_cast(bf16x8, fb[j]);
+            acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, B, acc[0][j], 0, 0, 0);
+            acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, B, acc[1][j], 0, 0, 0);
+        }
+    };
 
-    // a step: this wavefront's loads of the stage have landed; the barrier says the same of the others' and
-    // that everyone is done reading the other stage, which the next loads then overwrite
-#define PF_STEP(STAGE, OFF, MORE)                            \
-    do {                                                     \
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     \
-        __syncthreads();                                     \
-        if (MORE) PF_ISSUE(1 - (STAGE));                     \
-        PF_SLICE(OFF, 0);                                    \
-        PF_SLICE(OFF, 1);                                    \
-        PF_SLICE(OFF, 2);                                    \
-        PF_SLICE(OFF, 3);                                    \
-    } while (0)
-
-    PF_ISSUE(0);
-    int64_t kt = 0;
-    for (; kt + 2 <= nk; kt += 2) {
-        PF_STEP(0, 0, true);
-        PF_STEP(1, 32768, kt + 2 < nk);
+    issue(0);
+    for (int64_t kt = 0; kt < nk; kt++) {
+        const int stage = (int)(kt & 1);
+        // this wavefront's loads of the stage have landed; the barrier says the same of the others' and that
+        // everyone is done reading the other stage (its reads were complete when their statements returned),
+        // which the next loads then overwrite
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        if (kt + 1 < nk) issue(stage ^ 1);
+        const unsigned sb = lds0 + (unsigned)(stage * STAGE);
+#pragma unroll
+        for (int kk = 0; kk < 4; kk++) slice(sb, kk);
     }
-    if (kt < nk) PF_STEP(0, 0, false);
-#undef PF_STEP
-#undef PF_SLICE
-#undef PF_ISSUE
     pf_epilogue<EPI, JT>(a, acc, n0, m0, wn, wm, lane);
 }
 
@@ -625,8 +625,6 @@ __global__ __launch_bounds__(256) void pf_kv_tiles_kernel(const float *kc, const
     uint4 *dst = (uint4 *)(tiles + ((int64_t)kvh * n_tiles_max + kt) * T::BYTES);
     for (int c = t; c < T::BYTES / 16; c += 256) dst[c] = ((const uint4 *)s_img)[c];
 }
-
-typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 
 // N 16-byte LDS reads STRIDE bytes apart, complete on return: the reads and their wait are one statement, so
 // the compiler never sees a register of a read under way, and (being asm) the reads are not made to wait for
@@ -852,15 +850,40 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
     a.out_bf = out_bf;
     a.ldb = ldb;
     if (wbf) {
-        const unsigned n_mt = (unsigned)((M + 127) / 128), n_tiles = n_mt * (unsigned)((rows + 127) / 128);
+        // 256 x 256 tiles when they give every CU work (n_cu = 256), else 256 rows x 128 positions
+        const unsigned n_nt = (unsigned)((rows + 255) / 256);
+        const int jt = n_nt * (unsigned)((M + 255) / 256) >= 256 ? 4 : 2;
+        const unsigned n_mt = (unsigned)((M + 64 * jt - 1) / (64 * jt)), n_tiles = n_mt * n_nt;
         const unsigned per = (n_tiles + 7) / 8;
         const dim3 grid(8 * per);
-        switch (epi) {
-        case PF_STORE: hipLaunchKernelGGL((pf_gemm_bf16_kernel<PF_STORE>), grid, dim3(256), 0, s, a, n_mt, n_tiles, per); break;
-        case PF_RESID: hipLaunchKernelGGL((pf_gemm_bf16_kernel<PF_RESID>), grid, dim3(256), 0, s, a, n_mt, n_tiles, per); break;
-        case PF_SWIGLU: hipLaunchKernelGGL((pf_gemm_bf16_kernel<PF_SWIGLU>), grid, dim3(256), 0, s, a, n_mt, n_tiles, per); break;
-        default: return hipErrorInvalidValue;
+        const size_t lds = 2 * (size_t)(32768 + 64 * jt * 128);
+#define GO(E, J)                                                                                              \
+    do {                                                                                                      \
+        static bool attr_set = false;                                                                         \
+        if (!attr_set) {                                                                                      \
+            const hipError_t e = hipFuncSetAttribute((const void *)pf_gemm_bf16_kernel<E, J>,                 \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
+            if (e != hipSuccess) return e;                                                                    \
+            attr_set = true;                                                                                  \
+        }                                                                                                     \
+        hipLaunchKernelGGL((pf_gemm_bf16_kernel<E, J>), grid, dim3(512), lds, s, a, n_mt, n_tiles, per);      \
+    } while (0)
+        if (jt == 4) {
+            switch (epi) {
+            case PF_STORE: GO(PF_STORE, 4); break;
+            case PF_RESID: GO(PF_RESID, 4); break;
+            case PF_SWIGLU: GO(PF_SWIGLU, 4); break;
+            default: return hipErrorInvalidValue;
+            }
+        } else {
+            switch (epi) {
+            case PF_STORE: GO(PF_STORE, 2); break;
+            case PF_RESID: GO(PF_RESID, 2); break;
+            case PF_SWIGLU: GO(PF_SWIGLU, 2); break;
+            default: return hipErrorInvalidValue;
+            }
         }
+#undef GO
         return hipGetLastError();
     }
     // (a 256-position tile, JT = 4, was measured slower: its 272 registers leave one wavefront per SIMD)
@@ -875,7 +898,7 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
 
 // Expands the rows of the nseg tensors (one after another, or w1/w3 rows in turn when interleave is set) to
 // bf16 into the tiled matrix dst (see pf_expand_kernel) from row dst_row0 on; with pad the rows up to the
-// next multiple of 128 are zeroed.  K a multiple of 64.
+// next multiple of 256 are zeroed.  K a multiple of 64.
 hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interleave, int64_t K, uint16_t *dst,
                        int64_t dst_row0, int pad) {
     PfGemmArgs a{};
@@ -883,7 +906,7 @@ hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interlea
     if (e != hipSuccess) return e;
     if (K % 64 != 0) return hipErrorInvalidValue;
     int64_t rows_end = a.n_rows;
-    if (pad) rows_end = (dst_row0 + a.n_rows + 127) / 128 * 128 - dst_row0;
+    if (pad) rows_end = (dst_row0 + a.n_rows + 255) / 256 * 256 - dst_row0;
     const int64_t n = rows_end * (K >> 5);
     const dim3 grid((unsigned)((n + 255) / 256));
 #define GO(T) hipLaunchKernelGGL((pf_expand_kernel<T>), grid, dim3(256), 0, s, a, dst, dst_row0, rows_end)
