@@ -444,12 +444,55 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #define PF_AS1 __attribute__((address_space(1)))
 #define PF_AS3 __attribute__((address_space(3)))
 
+// Results of a workgroup tile of pf_gemm_bf16_kernel, which multiplies with the positions as the A operand:
+// a lane holds logical weight row n0 + 64 wn + 32 i + lane%32 and, in register r of tile (j, i), position
+// m0 + 32 JT wm + 32 j + 8 (r/4) + 4 (lane/32) + r%4.  The outputs are contiguous along the weight rows, so a
+// store of one register covers two runs of 32 consecutive elements.
+template <int EPI, int JT>
+__device__ __forceinline__ void pf_epilogue_rows(const PfGemmArgs &a, f32x16 (&acc)[JT][2], int64_t n0, int m0, int wn,
+                                                 int wm, int lane) {
+#pragma unroll
+    for (int j = 0; j < JT; j++)
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int64_t L = n0 + 64 * wn + 32 * i + (lane & 31);
+            const bool lvalid = L < a.n_rows;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = m0 + 32 * JT * wm + 32 * j + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const float v = acc[j][i][r];
+                if (EPI == PF_SWIGLU) {
+                    // (w1 row u, w3 row u) = logical rows (2u, 2u+1) (src/inference.jl:295-299) sit in lanes 2u, 2u+1;
+                    // lane 4k then stores columns 2k, 2k+1 of hb as one word
+                    const float other = __shfl_xor(v, 1, WAVE);
+                    const float h = swiglu_val(v, other);  // meaningful in even lanes
+                    const float h2 = __shfl_xor(h, 2, WAVE);
+                    if (m < a.M && lvalid && !(lane & 1)) {
+                        uint16_t *o = a.out_bf + (int64_t)m * a.ldb + (L >> 1);
+                        if (L + 3 < a.n_rows) {
+                            if (!(lane & 2)) *(uint32_t *)o = pack_bf16(h, h2);  // L/2 is even and ldb is even: aligned
+                        } else {
+                            ((__bf16 *)o)[0] = (__bf16)h;
+                        }
+                    }
+                } else if (m < a.M && lvalid) {
+                    float *o = a.out + (int64_t)m * a.ldo + a.out_col0 + L;
+                    if (EPI == PF_RESID)
+                        *o += v;  // x .+= ... (src/inference.jl:284,305)
+                    else
+                        *o = v;
+                }
+            }
+        }
+}
+
 // The same product from weights expanded beforehand (pf_expand_kernel): no arithmetic on the operands.
 // What bounds such a product on this chip is the path from L2 into the CU (64 bytes per clock): a 128 x 128
 // tile fetches 32 KB per 64 inputs and keeps that path busier than the matrix cores.  So the tile is 256
 // weight rows x 64 JT positions (JT = 4: 256, half the bytes per product; JT = 2: 128, for matrices with
 // too few rows to give every CU a 256 x 256 tile), worked on by 8 wavefronts, 4 row groups x 2 position
-// groups, each 64 rows x 32 JT positions.  Both operand tiles of a K step travel from global memory
+// groups, each 64 rows x 32 JT positions (the positions are the A operand of the matrix instructions, so
+// that a lane ends up with one weight row and the stores run along the outputs' contiguous dimension).  Both operand tiles of a K step travel from global memory
 // straight into LDS (16 bytes per lane and load, a wavefront's load filling 1 KB in lane order): the weight
 // tile is a linear copy of its 32 KB image, the position tile gets the c ^ pf_swz(r) placement by the choice
 // of the address each lane reads.  Two LDS stages: the loads of step kt + 1 are in flight during the products
@@ -524,47 +567,82 @@ __global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigne
         gw += 32768;
     };
 
-    // one 16-wide slice: operands from the stage at LDS address sb (reads and their wait are one statement, so
-    // no register of a read under way is visible; being asm, they are not made to wait for the copies in flight
-    // into the other stage), then 2 JT products
-    auto slice = [&](unsigned sb, int kk) {
-        pf_u32x4 fa0, fa1, fb[JT];
-        if constexpr (JT == 2) {
-            asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
-                         "\n\ts_waitcnt lgkmcnt(0)"
-                         : "=&v"(fa0), "=&v"(fa1), "=&v"(fb[0]), "=&v"(fb[1])
-                         : "v"(sb + aw[0][kk]), "v"(sb + aw[1][kk]), "v"(sb + ax[0][kk]), "v"(sb + ax[1][kk])
-                         : "memory");
-        } else {
-            asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %7\n\tds_read_b128 %2, %8\n\tds_read_b128 %3, %9"
-                         "\n\tds_read_b128 %4, %10\n\tds_read_b128 %5, %11\n\ts_waitcnt lgkmcnt(0)"
-                         : "=&v"(fa0), "=&v"(fa1), "=&v"(fb[0]), "=&v"(fb[1]), "=&v"(fb[2]), "=&v"(fb[3])
-                         : "v"(sb + aw[0][kk]), "v"(sb + aw[1][kk]), "v"(sb + ax[0][kk]), "v"(sb + ax[1][kk]),
-                           "v"(sb + ax[2][kk]), "v"(sb + ax[3][kk])
-                         : "memory");
-        }
-        const bf16x8 A0 = __builtin_bit_cast(bf16x8, fa0), A1 = __builtin_bit_cast(bf16x8, fa1);
-#pragma unroll
-        for (int j = 0; j < JT; j++) {
-            const bf16x8 B = __builtin_bit_cast(bf16x8, fb[j]);
-            acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A0, B, acc[0][j], 0, 0, 0);
-            acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(A1, B, acc[1][j], 0, 0, 0);
-        }
-    };
+    // The operands of a 16-wide slice (2 weight groups, JT position groups) are read from LDS one slice ahead
+    // of the products that use them, into two register sets used in turn, so that a wavefront's LDS latency
+    // lies under its own products.  Reads and waits are asm: the compiler then does not make them wait for the
+    // copies in flight into the other stage.  Between a PF_READ and the PF_WAIT that retires it the registers
+    // of the set hold nothing yet: the set only appears as an operand of those two statements and of the
+    // products after the wait (LDS reads complete in order, so lgkmcnt(2 + JT) retires all but the newest set;
+    // the build's asm check walks the generated code for any other touch of such a register).
+    pf_u32x4 F0[2 + JT], F1[2 + JT];
+#define PF_READ(F, KK)                                                                                            \
+    do {                                                                                                          \
+        if constexpr (JT == 2)                                                                                    \
+            asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"  \
+                         : "=&v"(F[0]), "=&v"(F[1]), "=&v"(F[2]), "=&v"(F[3])                                     \
+                         : "v"(sb + aw[0][KK]), "v"(sb + aw[1][KK]), "v"(sb + ax[0][KK]), "v"(sb + ax[1][KK])     \
+                         : "memory");                                                                             \
+        else                                                                                                      \
+            asm volatile("ds_read_b128 %0, %6\n\tds_read_b128 %1, %7\n\tds_read_b128 %2, %8\n\tds_read_b128 %3, %9"  \
+                         "\n\tds_read_b128 %4, %10\n\tds_read_b128 %5, %11"                                       \
+                         : "=&v"(F[0]), "=&v"(F[1]), "=&v"(F[2]), "=&v"(F[3]), "=&v"(F[4]), "=&v"(F[5])           \
+                         : "v"(sb + aw[0][KK]), "v"(sb + aw[1][KK]), "v"(sb + ax[0][KK]), "v"(sb + ax[1][KK]),    \
+                           "v"(sb + ax[JT - 2][KK]), "v"(sb + ax[JT - 1][KK])                                     \
+                         : "memory");                                                                             \
+    } while (0)
+    // LAST: nothing newer is in flight
+#define PF_WAIT(F, LAST)                                                                                          \
+    do {                                                                                                          \
+        if constexpr (JT == 2) {                                                                                  \
+            if (LAST)                                                                                             \
+                asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(F[0]), "+v"(F[1]), "+v"(F[2]), "+v"(F[3])::"memory");  \
+            else                                                                                                  \
+                asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(F[0]), "+v"(F[1]), "+v"(F[2]), "+v"(F[3])::"memory");  \
+        } else {                                                                                                  \
+            if (LAST)                                                                                             \
+                asm volatile("s_waitcnt lgkmcnt(0)"                                                               \
+                             : "+v"(F[0]), "+v"(F[1]), "+v"(F[2]), "+v"(F[3]), "+v"(F[JT]), "+v"(F[JT + 1])::"memory"); \
+            else                                                                                                  \
+                asm volatile("s_waitcnt lgkmcnt(6)"                                                               \
+                             : "+v"(F[0]), "+v"(F[1]), "+v"(F[2]), "+v"(F[3]), "+v"(F[JT]), "+v"(F[JT + 1])::"memory"); \
+        }                                                                                                         \
+    } while (0)
+#define PF_PRODUCTS(F)                                                                                            \
+    do {                                                                                                          \
+        const bf16x8 W0 = __builtin_bit_cast(bf16x8, F[0]), W1 = __builtin_bit_cast(bf16x8, F[1]);                \
+        _Pragma("unroll") for (int j = 0; j < JT; j++) {                                                          \
+            const bf16x8 P = __builtin_bit_cast(bf16x8, F[2 + j]);                                                \
+            acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(W0, P, acc[0][j], 0, 0, 0);                       \
+            acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(W1, P, acc[1][j], 0, 0, 0);                       \
+        }                                                                                                         \
+    } while (0)
 
     issue(0);
     for (int64_t kt = 0; kt < nk; kt++) {
         const int stage = (int)(kt & 1);
         // this wavefront's loads of the stage have landed; the barrier says the same of the others' and that
-        // everyone is done reading the other stage (its reads were complete when their statements returned),
-        // which the next loads then overwrite
+        // everyone is done reading the other stage (its last PF_WAIT retired every read), which the next loads
+        // then overwrite
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __builtin_amdgcn_s_barrier();
         if (kt + 1 < nk) issue(stage ^ 1);
         const unsigned sb = lds0 + (unsigned)(stage * STAGE);
-#pragma unroll
-        for (int kk = 0; kk < 4; kk++) slice(sb, kk);
+        PF_READ(F0, 0);
+        PF_READ(F1, 1);
+        PF_WAIT(F0, false);
+        PF_PRODUCTS(F0);
+        PF_READ(F0, 2);
+        PF_WAIT(F1, false);
+        PF_PRODUCTS(F1);
+        PF_READ(F1, 3);
+        PF_WAIT(F0, false);
+        PF_PRODUCTS(F0);
+        PF_WAIT(F1, true);
+        PF_PRODUCTS(F1);
     }
+#undef PF_PRODUCTS
+#undef PF_WAIT
+#undef PF_READ
     pf_epilogue<EPI, JT>(a, acc, n0, m0, wn, wm, lane);
 }
 
