@@ -444,55 +444,11 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 #define PF_AS1 __attribute__((address_space(1)))
 #define PF_AS3 __attribute__((address_space(3)))
 
-// Results of a workgroup tile of pf_gemm_bf16_kernel, which multiplies with the positions as the A operand:
-// a lane holds logical weight row n0 + 64 wn + 32 i + lane%32 and, in register r of tile (j, i), position
-// m0 + 32 JT wm + 32 j + 8 (r/4) + 4 (lane/32) + r%4.  The outputs are contiguous along the weight rows, so a
-// store of one register covers two runs of 32 consecutive elements.
-template <int EPI, int JT>
-__device__ __forceinline__ void pf_epilogue_rows(const PfGemmArgs &a, f32x16 (&acc)[JT][2], int64_t n0, int m0, int wn,
-                                                 int wm, int lane) {
-#pragma unroll
-    for (int j = 0; j < JT; j++)
-#pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const int64_t L = n0 + 64 * wn + 32 * i + (lane & 31);
-            const bool lvalid = L < a.n_rows;
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int m = m0 + 32 * JT * wm + 32 * j + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                const float v = acc[j][i][r];
-                if (EPI == PF_SWIGLU) {
-                    // (w1 row u, w3 row u) = logical rows (2u, 2u+1) (src/inference.jl:295-299) sit in lanes 2u, 2u+1;
-                    // lane 4k then stores columns 2k, 2k+1 of hb as one word
-                    const float other = __shfl_xor(v, 1, WAVE);
-                    const float h = swiglu_val(v, other);  // meaningful in even lanes
-                    const float h2 = __shfl_xor(h, 2, WAVE);
-                    if (m < a.M && lvalid && !(lane & 1)) {
-                        uint16_t *o = a.out_bf + (int64_t)m * a.ldb + (L >> 1);
-                        if (L + 3 < a.n_rows) {
-                            if (!(lane & 2)) *(uint32_t *)o = pack_bf16(h, h2);  // L/2 is even and ldb is even: aligned
-                        } else {
-                            ((__bf16 *)o)[0] = (__bf16)h;
-                        }
-                    }
-                } else if (m < a.M && lvalid) {
-                    float *o = a.out + (int64_t)m * a.ldo + a.out_col0 + L;
-                    if (EPI == PF_RESID)
-                        *o += v;  // x .+= ... (src/inference.jl:284,305)
-                    else
-                        *o = v;
-                }
-            }
-        }
-}
-
 // The same product from weights expanded beforehand (pf_expand_kernel): no arithmetic on the operands.
-// What bounds such a product on this chip is the path from L2 into the CU (64 bytes per clock): a 128 x 128
-// tile fetches 32 KB per 64 inputs and keeps that path busier than the matrix cores.  So the tile is 256
-// weight rows x 64 JT positions (JT = 4: 256, half the bytes per product; JT = 2: 128, for matrices with
-// too few rows to give every CU a 256 x 256 tile), worked on by 8 wavefronts, 4 row groups x 2 position
-// groups, each 64 rows x 32 JT positions (the positions are the A operand of the matrix instructions, so
-// that a lane ends up with one weight row and the stores run along the outputs' contiguous dimension).  Both operand tiles of a K step travel from global memory
+// The tile is 256 weight rows x 64 JT positions (JT = 4: 256 positions, 64 KB fetched per 64 inputs, half
+// the bytes per product of a 128 x 128 tile; JT = 2: 128 positions, for matrices with too few rows to give
+// every CU a 256 x 256 tile), worked on by 8 wavefronts, 4 row groups x 2 position groups, each 64 rows x
+// 32 JT positions.  Both operand tiles of a K step travel from global memory
 // straight into LDS (16 bytes per lane and load, a wavefront's load filling 1 KB in lane order): the weight
 // tile is a linear copy of its 32 KB image, the position tile gets the c ^ pf_swz(r) placement by the choice
 // of the address each lane reads.  Two LDS stages: the loads of step kt + 1 are in flight during the products
