@@ -76,7 +76,7 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 = skip)")
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py: this build runs on exactly one GPU (batch-1 decode does not shard; see DESIGN.md); "
+        log("bench.py: this build runs on exactly one GPU (batch-1 decode of one sequence is not sharded here); "
             "--gpus %d is not supported" % args.gpus)
         sys.exit(2)
 
