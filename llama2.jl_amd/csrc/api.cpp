@@ -215,7 +215,6 @@ struct l2h_model {
     DecodeCtl *ctl = nullptr;
     int32_t *prompt_dev = nullptr, *out_tokens = nullptr;
     int64_t *argmax_partial = nullptr;
-    unsigned int *att_counter = nullptr;  // arrivals per head group of the long-cache value kernel (zero between launches)
     int max_out = 0;
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
@@ -791,7 +790,7 @@ static hipError_t enqueue_token(l2h_model *m) {
         if (c.seq_len <= 1024)
             CK(k_attention_fused(s, m->q, m->xb, kc, vc, m->ctl, m->hs, c.n_heads, c.n_kv_heads, c.seq_len));
         else
-            CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->att_counter, m->ctl, m->hs, c.n_heads, c.n_kv_heads,
+            CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->ctl, m->hs, c.n_heads, c.n_kv_heads,
                            c.seq_len));
         CK(launch_wo(m, l));
         CK(launch_w13(m, l));
@@ -837,7 +836,6 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     m->cache_layer_elems = (int64_t)c.seq_len * m->kv_dim;
     DA(m->kc, m->cache_layer_elems * c.n_layers, true);
     DA(m->vc, m->cache_layer_elems * c.n_layers, true);
-    DA(m->att_counter, c.n_heads, true);
     DA(m->ctl, 1, true);
     DA(m->prompt_dev, c.seq_len, true);
     m->max_out = c.seq_len;
@@ -1434,9 +1432,7 @@ extern "C" int l2h_attention(l2h_ctx *ctx, float *out, const float *q, const flo
     const int seq_len = ((np + L2H_ATT_TILE - 1) / L2H_ATT_TILE) * L2H_ATT_TILE;
     const int dim = head_size * n_heads, kv_dim = head_size * n_kv_heads;
     const int ntiles = seq_len / L2H_ATT_TILE;
-    DevBuf dq, dqd, dkl, dvl, dkc, dvc, datt, dpd, dpart, dout, dctl, dcnt;
-    HIPCHK(ctx, dcnt.alloc((size_t)n_heads * 4));
-    HIPCHK(ctx, hipMemset(dcnt.p, 0, (size_t)n_heads * 4));
+    DevBuf dq, dqd, dkl, dvl, dkc, dvc, datt, dpd, dpart, dout, dctl;
     HIPCHK(ctx, dq.alloc((size_t)dim * 4));
     HIPCHK(ctx, dqd.alloc((size_t)dim * 8));
     HIPCHK(ctx, dkl.alloc((size_t)np * kv_dim * 4));
@@ -1458,8 +1454,7 @@ extern "C" int l2h_attention(l2h_ctx *ctx, float *out, const float *q, const flo
     HIPCHK(ctx, k_kv_layout(ctx->stream, dkc.as<float>(), dvc.as<float>(), dkl.as<float>(), dvl.as<float>(), 0, np,
                             head_size, n_kv_heads, seq_len, true));
     HIPCHK(ctx, k_attention(ctx->stream, dqd.as<double>(), dkc.as<float>(), dvc.as<float>(), datt.as<float>(),
-                            dpd.as<double>(), dpart.as<double>(), dout.as<float>(), (unsigned int *)dcnt.p,
-                            (const DecodeCtl *)dctl.p,
+                            dpd.as<double>(), dpart.as<double>(), dout.as<float>(), (const DecodeCtl *)dctl.p,
                             head_size, n_heads, n_kv_heads, seq_len));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(out, dout.p, (size_t)dim * 4, hipMemcpyDeviceToHost));

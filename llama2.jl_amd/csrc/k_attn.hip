@@ -266,7 +266,7 @@ hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const flo
 
 template <int GH>
 static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att,
-                              double *pd, double *part, float *out, unsigned int *counter, const DecodeCtl *ctl, int hs,
+                              double *pd, double *part, float *out, const DecodeCtl *ctl, int hs,
                               int n_heads, int n_kv_heads, int seq_len) {
     const int ntiles = (seq_len + L2H_ATT_TILE - 1) / L2H_ATT_TILE;
     if (hs <= 128 && hs % 16 == 0 && L2H_ATT_TILE == 64) {
@@ -305,10 +305,10 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
 }
 
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
-                       double *part, float *out, unsigned int *counter, const DecodeCtl *ctl, int head_size, int n_heads,
+                       double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads,
                        int n_kv_heads, int seq_len) {
     const int G = n_heads / n_kv_heads;
-    if (G % 4 == 0) return launch_attn<4>(s, qd, kc, vc, att, pd, part, out, counter, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    if (G % 2 == 0) return launch_attn<2>(s, qd, kc, vc, att, pd, part, out, counter, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    return launch_attn<1>(s, qd, kc, vc, att, pd, part, out, counter, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    if (G % 4 == 0) return launch_attn<4>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    if (G % 2 == 0) return launch_attn<2>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
+    return launch_attn<1>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
 }

@@ -458,14 +458,15 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 
 template <int EPI, int JT>
-__global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned n_mt, unsigned n_tiles, unsigned per) {
+__global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned nt0, unsigned n_mt, unsigned n_tiles,
+                                                           unsigned per) {
     constexpr int MT = 64 * JT;                   // positions per workgroup
     constexpr int STAGE = 32768 + MT * 128;       // bytes: weight tile, then position tile
     extern __shared__ uint4 s_all[];              // two stages
     const unsigned tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
     if (tile >= n_tiles) return;
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wn = wave & 3, wm = wave >> 2;
-    const unsigned mt = tile % n_mt, nt = tile / n_mt;
+    const unsigned mt = tile % n_mt, nt = nt0 + tile / n_mt;  // this launch covers row groups nt0 ..
     const int64_t n0 = (int64_t)nt * 256;
     const int m0 = (int)mt * MT;
     const int64_t K = a.K, nk = K >> 6;
@@ -884,13 +885,16 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
     a.out_bf = out_bf;
     a.ldb = ldb;
     if (wbf) {
-        // 256 x 256 tiles when they give every CU work (n_cu = 256), else 256 rows x 128 positions
-        const unsigned n_nt = (unsigned)((rows + 255) / 256);
-        const int jt = n_nt * (unsigned)((M + 255) / 256) >= 256 ? 4 : 2;
-        const unsigned n_mt = (unsigned)((M + 64 * jt - 1) / (64 * jt)), n_tiles = n_mt * n_nt;
-        const unsigned per = (n_tiles + 7) / 8;
-        const dim3 grid(8 * per);
-        const size_t lds = 2 * (size_t)(32768 + 64 * jt * 128);
+        // 256 x 256 tiles (JT = 4) for as many row groups as fill whole rounds of the 256 CUs; what is left, or
+        // a matrix too small for one such round, goes in 256 x 128 tiles (JT = 2), which spread it over twice
+        // as many workgroups
+        const unsigned n_nt = (unsigned)((rows + 255) / 256), n_mt4 = (unsigned)((M + 255) / 256);
+        const unsigned nt4 = (n_nt * n_mt4 / 256) * 256 / n_mt4;  // row groups in whole rounds of 256 x 256 tiles
+        auto launch = [&](int jt, unsigned nt0, unsigned nnt) -> hipError_t {
+            const unsigned n_mt = (unsigned)((M + 64 * jt - 1) / (64 * jt)), n_tiles = n_mt * nnt;
+            const unsigned per = (n_tiles + 7) / 8;
+            const dim3 grid(8 * per);
+            const size_t lds = 2 * (size_t)(32768 + 64 * jt * 128);
 #define GO(E, J)                                                                                              \
     do {                                                                                                      \
         static bool attr_set = false;                                                                         \
@@ -900,25 +904,31 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
             if (e != hipSuccess) return e;                                                                    \
             attr_set = true;                                                                                  \
         }                                                                                                     \
-        hipLaunchKernelGGL((pf_gemm_bf16_kernel<E, J>), grid, dim3(512), lds, s, a, n_mt, n_tiles, per);      \
+        hipLaunchKernelGGL((pf_gemm_bf16_kernel<E, J>), grid, dim3(512), lds, s, a, nt0, n_mt, n_tiles, per); \
     } while (0)
-        if (jt == 4) {
-            switch (epi) {
-            case PF_STORE: GO(PF_STORE, 4); break;
-            case PF_RESID: GO(PF_RESID, 4); break;
-            case PF_SWIGLU: GO(PF_SWIGLU, 4); break;
-            default: return hipErrorInvalidValue;
+            if (jt == 4) {
+                switch (epi) {
+                case PF_STORE: GO(PF_STORE, 4); break;
+                case PF_RESID: GO(PF_RESID, 4); break;
+                case PF_SWIGLU: GO(PF_SWIGLU, 4); break;
+                default: return hipErrorInvalidValue;
+                }
+            } else {
+                switch (epi) {
+                case PF_STORE: GO(PF_STORE, 2); break;
+                case PF_RESID: GO(PF_RESID, 2); break;
+                case PF_SWIGLU: GO(PF_SWIGLU, 2); break;
+                default: return hipErrorInvalidValue;
+                }
             }
-        } else {
-            switch (epi) {
-            case PF_STORE: GO(PF_STORE, 2); break;
-            case PF_RESID: GO(PF_RESID, 2); break;
-            case PF_SWIGLU: GO(PF_SWIGLU, 2); break;
-            default: return hipErrorInvalidValue;
-            }
-        }
 #undef GO
-        return hipGetLastError();
+            return hipGetLastError();
+        };
+        if (nt4 > 0) {
+            const hipError_t e = launch(4, 0, nt4);
+            if (e != hipSuccess) return e;
+        }
+        return nt4 < n_nt ? launch(2, nt4, n_nt - nt4) : hipSuccess;
     }
     // (a 256-position tile, JT = 4, was measured slower: its 272 registers leave one wavefront per SIMD)
     switch (w[0].type) {

@@ -189,7 +189,7 @@ hipError_t k_mega_launch(hipStream_t s, const MegaArgs &g, int t_qkv, int t_wo, 
 hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64_t n, int pro, Q8Dev q8_out, float *f32_out);
 hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
-                       double *part, float *out, unsigned int *counter, const DecodeCtl *ctl, int head_size, int n_heads,
+                       double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads,
                        int n_kv_heads, int seq_len);
 // one launch for scores + softmax + values; needs head_size*8 + seq_len*12 + 8 KiB of LDS <= 64 KiB
 hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const float *kc, const float *vc,
