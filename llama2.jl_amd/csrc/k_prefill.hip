@@ -690,14 +690,24 @@ __device__ __forceinline__ void pf_lds_read(pf_u32x4 (&o)[4], unsigned addr) {
 
 template <int HS>
 __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles,
-                                                      int n_tiles_max, int M, int qpos0, int n_heads, int n_kv, int dim) {
+                                                      int n_tiles_max, int M, int qpos0, int n_heads, int n_kv, int dim,
+                                                      unsigned n_qb, unsigned n_items, unsigned per) {
     typedef PfKvTile<HS> T;
     constexpr int KSTEPS = HS / 16, DT = HS / 32, KH = KSTEPS / 2;
     // two stages: the copy of tile kt + 1 is in flight during the products of tile kt, one barrier per tile
     __shared__ __align__(16) unsigned char s_t[2 * T::BYTES];
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), g = lane >> 5, ql = lane & 31;
-    const int h = blockIdx.y, kvh = h / (n_heads / n_kv);
-    const int q0 = blockIdx.x * 128;
+    // Workgroups are dealt to the 8 XCDs in turn: workgroup w takes item (w % 8) * per + w / 8 of the list
+    // (head, query block), so an XCD works through a few heads (the heads of a KV group share its L2).  A
+    // block's work grows with its index (causal); two workgroups share a CU, the second of them from the
+    // later half of the XCD's run, so the heads that start in that half take their query blocks in reverse
+    // order and a long block meets a short one.
+    const unsigned item = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+    if (item >= n_items) return;
+    const int h = (int)(item / n_qb), u = (int)(item % n_qb);
+    const int kvh = h / (n_heads / n_kv);
+    const int qb = ((unsigned)h * n_qb) % per >= (per + 1) / 2 ? (int)n_qb - 1 - u : u;
+    const int q0 = qb * 128;
     const int myq = q0 + 32 * wave + ql;
     const bool qvalid = myq < M;
     bf16x8 qf[KSTEPS];
@@ -998,8 +1008,10 @@ hipError_t k_pf_kv_tiles(hipStream_t s, const float *kc, const float *vc, unsign
 hipError_t k_pf_attention(hipStream_t s, const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles, int n_tiles_max,
                           int M, int qpos0, int hs, int n_heads, int n_kv, int dim) {
     if ((qpos0 + M + 31) / 32 > n_tiles_max) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)((M + 127) / 128), (unsigned)n_heads);
-#define GO(HS) hipLaunchKernelGGL((pf_attn_kernel<HS>), grid, dim3(256), 0, s, Qb, Att, tiles, n_tiles_max, M, qpos0, n_heads, n_kv, dim)
+    const unsigned n_qb = (unsigned)((M + 127) / 128), n_items = n_qb * (unsigned)n_heads, per = (n_items + 7) / 8;
+    const dim3 grid(8 * per);
+#define GO(HS) \
+    hipLaunchKernelGGL((pf_attn_kernel<HS>), grid, dim3(256), 0, s, Qb, Att, tiles, n_tiles_max, M, qpos0, n_heads, n_kv, dim, n_qb, n_items, per)
     switch (hs) {
     case 32: GO(32); break;
     case 64: GO(64); break;
