@@ -457,16 +457,12 @@ __global__ __launch_bounds__(256) void pf_gemm_kernel(PfGemmArgs a) {
 // workgroups that share a weight tile share an L2.
 typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 
+// the tile (row group nt, position block mt) of one workgroup; s_all: two stages of LDS
 template <int EPI, int JT>
-__global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned nt0, unsigned n_mt, unsigned n_tiles,
-                                                           unsigned per) {
+__device__ __forceinline__ void pf_gemm_bf16_tile(const PfGemmArgs &a, unsigned nt, unsigned mt, uint4 *s_all) {
     constexpr int MT = 64 * JT;                   // positions per workgroup
     constexpr int STAGE = 32768 + MT * 128;       // bytes: weight tile, then position tile
-    extern __shared__ uint4 s_all[];              // two stages
-    const unsigned tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
-    if (tile >= n_tiles) return;
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6), wn = wave & 3, wm = wave >> 2;
-    const unsigned mt = tile % n_mt, nt = nt0 + tile / n_mt;  // this launch covers row groups nt0 ..
     const int64_t n0 = (int64_t)nt * 256;
     const int m0 = (int)mt * MT;
     const int64_t K = a.K, nk = K >> 6;
@@ -601,6 +597,37 @@ __global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigne
 #undef PF_WAIT
 #undef PF_READ
     pf_epilogue<EPI, JT>(a, acc, n0, m0, wn, wm, lane);
+}
+
+// row groups nt0 .. in tiles of 64 JT positions
+template <int EPI, int JT>
+__global__ __launch_bounds__(512) void pf_gemm_bf16_kernel(PfGemmArgs a, unsigned nt0, unsigned n_mt, unsigned n_tiles,
+                                                           unsigned per) {
+    extern __shared__ uint4 s_all[];
+    const unsigned tile = (blockIdx.x & 7u) * per + (blockIdx.x >> 3);
+    if (tile >= n_tiles) return;
+    pf_gemm_bf16_tile<EPI, JT>(a, nt0 + tile / n_mt, tile % n_mt, s_all);
+}
+
+// One round of the CUs over a matrix that would need between one and two rounds of 256 x 128 tiles: the
+// first nt4 row groups in 256 x 256 tiles, the others in 256 x 128 tiles, sized by the caller so that every
+// CU gets one workgroup (each XCD takes per4 of the large and then per2 of the small tiles, again as
+// contiguous runs, positions fastest).
+template <int EPI>
+__global__ __launch_bounds__(512) void pf_gemm_bf16_mixed_kernel(PfGemmArgs a, unsigned nt4, unsigned n_mt4, unsigned n_mt2,
+                                                                 unsigned n_tiles4, unsigned n_tiles2, unsigned per4,
+                                                                 unsigned per2) {
+    extern __shared__ uint4 s_all[];
+    const unsigned xcd = blockIdx.x & 7u, k = blockIdx.x >> 3;
+    if (k < per4) {
+        const unsigned tile = xcd * per4 + k;
+        if (tile >= n_tiles4) return;
+        pf_gemm_bf16_tile<EPI, 4>(a, tile / n_mt4, tile % n_mt4, s_all);
+    } else {
+        const unsigned tile = xcd * per2 + (k - per4);
+        if (tile >= n_tiles2) return;
+        pf_gemm_bf16_tile<EPI, 2>(a, nt4 + tile / n_mt2, tile % n_mt2, s_all);
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -934,6 +961,36 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
 #undef GO
             return hipGetLastError();
         };
+        const unsigned n_mt2 = (unsigned)((M + 127) / 128);
+        if (nt4 == 0 && n_nt * n_mt2 > 256 && n_mt2 > n_mt4) {
+            // more than one round of 256 x 128 tiles, less than one of 256 x 256: mix the two so that the work
+            // fits one round, na row groups in large tiles
+            const unsigned na = (n_nt * n_mt2 - 256 + (n_mt2 - n_mt4) - 1) / (n_mt2 - n_mt4);
+            if (na <= n_nt) {
+                const unsigned t4 = na * n_mt4, t2 = (n_nt - na) * n_mt2, per4 = (t4 + 7) / 8, per2 = (t2 + 7) / 8;
+                const dim3 grid(8 * (per4 + per2));
+                const size_t lds = 2 * (size_t)(32768 + 256 * 128);
+#define GO(E)                                                                                                       \
+    do {                                                                                                            \
+        static bool attr_set = false;                                                                               \
+        if (!attr_set) {                                                                                            \
+            const hipError_t e = hipFuncSetAttribute((const void *)pf_gemm_bf16_mixed_kernel<E>,                    \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);         \
+            if (e != hipSuccess) return e;                                                                          \
+            attr_set = true;                                                                                        \
+        }                                                                                                           \
+        hipLaunchKernelGGL((pf_gemm_bf16_mixed_kernel<E>), grid, dim3(512), lds, s, a, na, n_mt4, n_mt2, t4, t2, per4, per2); \
+    } while (0)
+                switch (epi) {
+                case PF_STORE: GO(PF_STORE); break;
+                case PF_RESID: GO(PF_RESID); break;
+                case PF_SWIGLU: GO(PF_SWIGLU); break;
+                default: return hipErrorInvalidValue;
+                }
+#undef GO
+                return hipGetLastError();
+            }
+        }
         if (nt4 > 0) {
             const hipError_t e = launch(4, 0, nt4);
             if (e != hipSuccess) return e;

@@ -77,13 +77,19 @@ WIDE = ("PLAN_Q5_K_M", dict(dim=512, hidden_dim=1536, n_layers=2, n_heads=8, n_k
                             rope_freq_base=10000.0, rope_is_neox=False))
 
 
-@pytest.mark.parametrize("case", sorted(CASES) + ["wide"])
+# w1|w3 with 86 groups of 256 rows at 300 positions: more than one round of 256 x 128 tiles on 256 CUs, less than
+# one of 256 x 256 ones, which is where the product kernel mixes the two tile shapes in one launch
+MIXED = ("PLAN_F32", dict(dim=64, hidden_dim=11008, n_layers=1, n_heads=2, n_kv_heads=2, vocab_size=512, seq_len=303,
+                          rope_freq_base=10000.0, rope_is_neox=False))
+
+
+@pytest.mark.parametrize("case", sorted(CASES) + ["wide", "mixed"])
 def test_prefill_weight_copy_changes_nothing(pkg, case):
     """l2h_prefill multiplies from a resident bf16 copy of the weights (default) or expands the quantized
     blocks inside the product kernel (l2h_model_set_prefill_copy(m, 0)): the same bf16 values either way,
     so logits and cache are equal bit for bit."""
     from llama2_jl_amd import synth
-    plan, kw = WIDE if case == "wide" else CASES[case]
+    plan, kw = WIDE if case == "wide" else MIXED if case == "mixed" else CASES[case]
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
     n = cfg.seq_len - 3
