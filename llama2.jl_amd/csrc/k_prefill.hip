@@ -47,18 +47,46 @@ __global__ __launch_bounds__(64) void pf_rope_table_kernel(float *cs, int pos0, 
 __global__ __launch_bounds__(256) void pf_rmsnorm_kernel(const float *X, const float *w, uint16_t *out, int64_t K) {
     __shared__ double red[16];
     const float *x = X + (int64_t)blockIdx.x * K;
+    __bf16 *o = (__bf16 *)out + (int64_t)blockIdx.x * K;
+    if (K % 4 == 0 && K <= 256 * 4 * 8) {  // the row stays in registers: 16 bytes per lane and load, one pass
+        float4 v[8];
+        double acc = 0.0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int64_t i = 4 * (threadIdx.x + 256 * j);
+            v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (i < K) v[j] = *(const float4 *)(x + i);
+            acc = fma((double)v[j].x, (double)v[j].x, acc);
+            acc = fma((double)v[j].y, (double)v[j].y, acc);
+            acc = fma((double)v[j].z, (double)v[j].z, acc);
+            acc = fma((double)v[j].w, (double)v[j].w, acc);
+        }
+        float ss = (float)block_sum_f64(acc, red);
+        ss /= (float)K;
+        ss += 1e-5f;
+        ss = 1.0f / sqrtf(ss);
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int64_t i = 4 * (threadIdx.x + 256 * j);
+            if (i < K) {
+                const float4 g = *(const float4 *)(w + i);
+                uint2 pk;
+                pk.x = pack_bf16(g.x * (ss * v[j].x), g.y * (ss * v[j].y));
+                pk.y = pack_bf16(g.z * (ss * v[j].z), g.w * (ss * v[j].w));
+                *(uint2 *)(o + i) = pk;
+            }
+        }
+        return;
+    }
     double acc = 0.0;
     for (int64_t i = threadIdx.x; i < K; i += blockDim.x) acc = fma((double)x[i], (double)x[i], acc);
     float ss = (float)block_sum_f64(acc, red);
     ss /= (float)K;
     ss += 1e-5f;
     ss = 1.0f / sqrtf(ss);
-    __bf16 *o = (__bf16 *)out + (int64_t)blockIdx.x * K;
     for (int64_t i = threadIdx.x; i < K; i += blockDim.x) o[i] = (__bf16)(w[i] * (ss * x[i]));
 }
 
-// rope! of q and k (src/inference.jl:112-157), cache append (:259-260): raw[m] = (q | k | v) fp32 ->
-// Qb bf16 [M][dim], K cache [n_kv][hs/4][seq_len][4], V cache [n_kv][seq_len][hs]
 __global__ __launch_bounds__(256) void pf_rope_scatter_kernel(const float *raw, const float *cs, uint16_t *Qb,
                                                               float *kc, float *vc, int M, int pos0, int dim,
                                                               int kv_dim, int hs, int seq_len, int neox) {
@@ -66,28 +94,42 @@ __global__ __launch_bounds__(256) void pf_rope_scatter_kernel(const float *raw, 
     if (m >= M) return;
     const float *r = raw + (int64_t)m * (dim + 2 * kv_dim);
     const int half = hs >> 1, pos = pos0 + m;
-    const int npairs = (dim + kv_dim) >> 1;
-    for (int p = threadIdx.x; p < npairs; p += blockDim.x) {
-        const bool is_q = p < (dim >> 1);
-        const int pp = is_q ? p : p - (dim >> 1);
-        const int h = pp / half, i = pp % half;
-        const int e0 = neox ? i : 2 * i, e1 = neox ? i + half : 2 * i + 1;
+    // a thread turns 4 consecutive pairs of one head: rotation indices i0 .. i0+3, whose 8 elements are two
+    // runs of 4 (interleaved pairs: 2 i0 .. and 2 i0 + 4 ..; half-split pairs: i0 .. and i0 + half ..)
+    const int qpH = half >> 2, nquads = ((dim + kv_dim) / hs) * qpH;
+    for (int p = threadIdx.x; p < nquads; p += blockDim.x) {
+        const int hh = p / qpH, i0 = 4 * (p % qpH);
+        const bool is_q = hh < dim / hs;
+        const int h = is_q ? hh : hh - dim / hs;
         const float *src = r + (is_q ? 0 : dim) + h * hs;
-        const float re = src[e0], im = src[e1];
-        const float c = cs[((int64_t)m * half + i) * 2], s = cs[((int64_t)m * half + i) * 2 + 1];
-        const float o0 = (re * c) - (im * s), o1 = (re * s) + (im * c);
+        const int ea = neox ? i0 : 2 * i0, eb = neox ? i0 + half : 2 * i0 + 4;
+        const float4 a = *(const float4 *)(src + ea), b = *(const float4 *)(src + eb);
+        const float4 c0 = *(const float4 *)(cs + ((int64_t)m * half + i0) * 2);      // cos, sin of i0, i0+1
+        const float4 c1 = *(const float4 *)(cs + ((int64_t)m * half + i0 + 2) * 2);  // ... of i0+2, i0+3
+        float4 oa, ob;
+        if (neox) {  // pair k = (a[k], b[k])
+            oa.x = (a.x * c0.x) - (b.x * c0.y), ob.x = (a.x * c0.y) + (b.x * c0.x);
+            oa.y = (a.y * c0.z) - (b.y * c0.w), ob.y = (a.y * c0.w) + (b.y * c0.z);
+            oa.z = (a.z * c1.x) - (b.z * c1.y), ob.z = (a.z * c1.y) + (b.z * c1.x);
+            oa.w = (a.w * c1.z) - (b.w * c1.w), ob.w = (a.w * c1.w) + (b.w * c1.z);
+        } else {  // pairs (a.x, a.y), (a.z, a.w), (b.x, b.y), (b.z, b.w)
+            oa.x = (a.x * c0.x) - (a.y * c0.y), oa.y = (a.x * c0.y) + (a.y * c0.x);
+            oa.z = (a.z * c0.z) - (a.w * c0.w), oa.w = (a.z * c0.w) + (a.w * c0.z);
+            ob.x = (b.x * c1.x) - (b.y * c1.y), ob.y = (b.x * c1.y) + (b.y * c1.x);
+            ob.z = (b.z * c1.z) - (b.w * c1.w), ob.w = (b.z * c1.w) + (b.w * c1.z);
+        }
         if (is_q) {
-            __bf16 *q = (__bf16 *)Qb + (int64_t)m * dim + h * hs;
-            q[e0] = (__bf16)o0;
-            q[e1] = (__bf16)o1;
-        } else {
-            kc[(((int64_t)h * (hs >> 2) + (e0 >> 2)) * seq_len + pos) * 4 + (e0 & 3)] = o0;
-            kc[(((int64_t)h * (hs >> 2) + (e1 >> 2)) * seq_len + pos) * 4 + (e1 & 3)] = o1;
+            uint16_t *q = Qb + (int64_t)m * dim + h * hs;
+            *(uint2 *)(q + ea) = make_uint2(pack_bf16(oa.x, oa.y), pack_bf16(oa.z, oa.w));
+            *(uint2 *)(q + eb) = make_uint2(pack_bf16(ob.x, ob.y), pack_bf16(ob.z, ob.w));
+        } else {  // kv.key_cache[:, :, pos] = k (src/inference.jl:259), elements in groups of 4 per timestep
+            *(float4 *)(kc + (((int64_t)h * (hs >> 2) + (ea >> 2)) * seq_len + pos) * 4) = oa;
+            *(float4 *)(kc + (((int64_t)h * (hs >> 2) + (eb >> 2)) * seq_len + pos) * 4) = ob;
         }
     }
-    for (int e = threadIdx.x; e < kv_dim; e += blockDim.x) {
+    for (int e = 4 * threadIdx.x; e < kv_dim; e += 4 * blockDim.x) {  // kv.value_cache[pos, :, :] = v (:260)
         const int h = e / hs, d = e % hs;
-        vc[((int64_t)h * seq_len + pos) * hs + d] = r[dim + kv_dim + e];
+        *(float4 *)(vc + ((int64_t)h * seq_len + pos) * hs + d) = *(const float4 *)(r + dim + kv_dim + e);
     }
 }
 
