@@ -730,35 +730,46 @@ __global__ __launch_bounds__(256) void pf_kv_tiles_kernel(const float *kc, const
     for (int c = t; c < T::BYTES / 16; c += 256) dst[c] = ((const uint4 *)s_img)[c];
 }
 
-// N 16-byte LDS reads STRIDE bytes apart, complete on return: the reads and their wait are one statement, so
-// the compiler never sees a register of a read under way, and (being asm) the reads are not made to wait for
-// the tile copies in flight into the other stage
+// N 16-byte LDS reads STRIDE bytes apart, issued and not waited for: until pf_lds_retire has run for `o`
+// its registers hold nothing yet and must appear nowhere else (the asm check of the build walks the generated
+// code for that).  Being asm, the reads are not made to wait for the tile copies in flight into the other stage.
 template <int N, int STRIDE>
-__device__ __forceinline__ void pf_lds_read(pf_u32x4 (&o)[4], unsigned addr) {
+__device__ __forceinline__ void pf_lds_issue(pf_u32x4 (&o)[4], unsigned addr) {
     static_assert(N >= 1 && N <= 4 && 3 * STRIDE < 65536, "");
     if constexpr (N == 1)
-        asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(o[0]) : "v"(addr) : "memory");
+        asm volatile("ds_read_b128 %0, %1" : "=&v"(o[0]) : "v"(addr) : "memory");
     else if constexpr (N == 2)
-        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:%3\n\ts_waitcnt lgkmcnt(0)"
+        asm volatile("ds_read_b128 %0, %2\n\tds_read_b128 %1, %2 offset:%3"
                      : "=&v"(o[0]), "=&v"(o[1])
                      : "v"(addr), "n"(STRIDE)
                      : "memory");
     else if constexpr (N == 3)
-        asm volatile("ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:%4\n\tds_read_b128 %2, %3 offset:%5\n\t"
-                     "s_waitcnt lgkmcnt(0)"
+        asm volatile("ds_read_b128 %0, %3\n\tds_read_b128 %1, %3 offset:%4\n\tds_read_b128 %2, %3 offset:%5"
                      : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2])
                      : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE)
                      : "memory");
     else
         asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %4 offset:%5\n\tds_read_b128 %2, %4 offset:%6\n\t"
-                     "ds_read_b128 %3, %4 offset:%7\n\ts_waitcnt lgkmcnt(0)"
+                     "ds_read_b128 %3, %4 offset:%7"
                      : "=&v"(o[0]), "=&v"(o[1]), "=&v"(o[2]), "=&v"(o[3])
                      : "v"(addr), "n"(STRIDE), "n"(2 * STRIDE), "n"(3 * STRIDE)
                      : "memory");
 }
+// every LDS read issued so far is complete; from here on `o` holds its values
+template <int N>
+__device__ __forceinline__ void pf_lds_retire(pf_u32x4 (&o)[4]) {
+    if constexpr (N == 1)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o[0])::"memory");
+    else if constexpr (N == 2)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o[0]), "+v"(o[1])::"memory");
+    else if constexpr (N == 3)
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2])::"memory");
+    else
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3])::"memory");
+}
 
 template <int HS>
-__global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles,
                                                       int n_tiles_max, int M, int qpos0, int n_heads, int n_kv, int dim,
                                                       unsigned n_qb, unsigned n_items, unsigned per) {
     typedef PfKvTile<HS> T;
@@ -819,14 +830,22 @@ __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16
         f32x16 s;
 #pragma unroll
         for (int r = 0; r < 16; r++) s[r] = 0.0f;
+        {
+            pf_u32x4 ka[2][4];
+            pf_lds_issue<KH, 32>(ka[0], k_addr + so);
+            pf_lds_issue<KH, 32>(ka[1], k_addr + so + (unsigned)(32 * KH));
+            pf_lds_retire<KH>(ka[0]);
+            pf_lds_retire<KH>(ka[1]);
 #pragma unroll
-        for (int half = 0; half < 2; half++) {
-            pf_u32x4 ka[4];
-            pf_lds_read<KH, 32>(ka, k_addr + so + (unsigned)(32 * KH * half));
+            for (int half = 0; half < 2; half++)
 #pragma unroll
-            for (int i = 0; i < KH; i++)
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[i]), qf[KH * half + i], s, 0, 0, 0);
+                for (int i = 0; i < KH; i++)
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ka[half][i]), qf[KH * half + i], s, 0, 0, 0);
         }
+        // the V^T operands of the second product are asked for now and arrive during the softmax arithmetic
+        pf_u32x4 va[2][4];
+        pf_lds_issue<DT, 32 * T::VROW>(va[0], v_addr + so);
+        pf_lds_issue<DT, 32 * T::VROW>(va[1], v_addr + so + 32u);
         // scores in units of log2 e: softmax(s / sqrt(hs)) = 2^(c s - max) / sum with c = log2 e / sqrt(hs)
         // (att ./= sqrt(hs); softmax!, src/inference.jl:268-270); only a tile on the diagonal needs the mask
         float tmax = -INFINITY;
@@ -861,16 +880,16 @@ __global__ __launch_bounds__(256) void pf_attn_kernel(const uint16_t *Qb, uint16
 #pragma unroll
                 for (int r = 0; r < 16; r++) o[d][r] *= alpha;
         }
+        pf_lds_retire<DT>(va[0]);
+        pf_lds_retire<DT>(va[1]);
 #pragma unroll
         for (int st = 0; st < 2; st++) {
             const uint4 pb = make_uint4(pack_bf16(s[8 * st], s[8 * st + 1]), pack_bf16(s[8 * st + 2], s[8 * st + 3]),
                                         pack_bf16(s[8 * st + 4], s[8 * st + 5]), pack_bf16(s[8 * st + 6], s[8 * st + 7]));
             const bf16x8 B = as_bf16x8(pb);
-            pf_u32x4 va[4];
-            pf_lds_read<DT, 32 * T::VROW>(va, v_addr + so + (unsigned)(32 * st));
 #pragma unroll
             for (int d = 0; d < DT; d++)
-                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[d]), B, o[d], 0, 0, 0);
+                o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va[st][d]), B, o[d], 0, 0, 0);
         }
     }
     if (!qvalid) return;
