@@ -849,21 +849,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
         // scores in units of log2 e: softmax(s / sqrt(hs)) = 2^(c s - max) / sum with c = log2 e / sqrt(hs)
         // (att ./= sqrt(hs); softmax!, src/inference.jl:268-270); only a tile on the diagonal needs the mask
         float tmax = -INFINITY;
-        const bool diagonal = key0 + 31 > qpos0 + q0 + 32 * wave || !qvalid;
+        // (wavefront-uniform: the tile reaches past the first query of the wavefront, or some query is past M)
+        const bool diagonal = key0 + 31 > qpos0 + q0 + 32 * wave || q0 + 32 * wave + 31 >= M;
+        if (diagonal) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            float v = s[r] * c_log2;
-            if (diagonal) {
+            for (int r = 0; r < 16; r++) {
                 const int key = key0 + 8 * (r >> 2) + 4 * g + (r & 3);
+                float v = s[r] * c_log2;
                 if (!qvalid || key > qpos0 + myq) v = -INFINITY;
+                s[r] = v;
+                tmax = fmaxf(tmax, v);
             }
-            s[r] = v;
-            tmax = fmaxf(tmax, v);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                s[r] *= c_log2;
+                tmax = fmaxf(tmax, s[r]);
+            }
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
-        const float mnew = fmaxf(mrun, tmax);
-        const float msub = (mnew == -INFINITY) ? 0.0f : mnew;  // a row with nothing visible yet: all terms 0
-        const float alpha = __builtin_amdgcn_exp2f(mrun - msub);
+        // The reference point of a query's exponents (mrun) follows its maximum only when the maximum has grown
+        // by more than 8 (a factor 256) since the reference was set, or when there was none: terms stay below
+        // 2^8, far inside fp32 and bf16 range, and the sums are rescaled on few tiles instead of on most (some
+        // query of the 64 in a wavefront meets a new maximum in nearly every tile).  The quotient sum / total at
+        // the end is the same softmax.
+        const bool move = tmax > mrun + 8.0f || (mrun == -INFINITY && tmax != -INFINITY);
+        if (__any(move)) {
+            const float mnew = fmaxf(mrun, tmax);
+            const float alpha = (mnew == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(mrun - mnew);
+            lrun *= alpha;
+            mrun = mnew;
+#pragma unroll
+            for (int d = 0; d < DT; d++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+        }
+        const float msub = (mrun == -INFINITY) ? 0.0f : mrun;  // a row with nothing visible yet: all terms 0
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 16; r++) {
@@ -872,14 +893,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
             psum += pv;
         }
         psum += __shfl_xor(psum, 32, WAVE);
-        lrun = lrun * alpha + psum;
-        mrun = mnew;
-        if (__any(alpha != 1.0f)) {  // the running maximum moved for some query of the wavefront
-#pragma unroll
-            for (int d = 0; d < DT; d++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[d][r] *= alpha;
-        }
+        lrun += psum;
         pf_lds_retire<DT>(va[0]);
         pf_lds_retire<DT>(va[1]);
 #pragma unroll
