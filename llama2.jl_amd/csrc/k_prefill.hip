@@ -768,6 +768,14 @@ __device__ __forceinline__ void pf_lds_retire(pf_u32x4 (&o)[4]) {
         asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(o[0]), "+v"(o[1]), "+v"(o[2]), "+v"(o[3])::"memory");
 }
 
+// the value of the lane 32 further on (or back): the two halves of the wavefront exchanged in one instruction
+__device__ __forceinline__ float pf_other_half(float x) {
+    typedef unsigned pf_u32x2 __attribute__((ext_vector_type(2)));
+    const pf_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    // r[0] = {low half, low half}, r[1] = {high half, high half}
+    return (threadIdx.x & 32) ? __uint_as_float(r[0]) : __uint_as_float(r[1]);
+}
+
 template <int HS>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void pf_attn_kernel(const uint16_t *Qb, uint16_t *Att, const unsigned char *tiles,
                                                       int n_tiles_max, int M, int qpos0, int n_heads, int n_kv, int dim,
@@ -867,7 +875,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
                 tmax = fmaxf(tmax, s[r]);
             }
         }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+        tmax = fmaxf(tmax, pf_other_half(tmax));
         // The reference point of a query's exponents (mrun) follows its maximum only when the maximum has grown
         // by more than 8 (a factor 256) since the reference was set, or when there was none: terms stay below
         // 2^8, far inside fp32 and bf16 range, and the sums are rescaled on few tiles instead of on most (some
@@ -892,7 +900,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void p
             s[r] = pv;
             psum += pv;
         }
-        psum += __shfl_xor(psum, 32, WAVE);
+        psum += pf_other_half(psum);
         lrun += psum;
         pf_lds_retire<DT>(va[0]);
         pf_lds_retire<DT>(va[1]);
