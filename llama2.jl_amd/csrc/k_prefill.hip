@@ -980,6 +980,8 @@ static hipError_t pf_weight_args(PfGemmArgs &a, const DevTensor *w, int nseg, in
     return hipSuccess;
 }
 
+#define PF_MAX_DEVICES 64
+
 // w: nseg tensors of one type sharing the input, or (wbf != nullptr) n_rows_bf rows expanded by
 // k_pf_expand; see PfGemmArgs for the outputs
 hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *wbf, int64_t n_rows_bf,
@@ -1005,6 +1007,12 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
     a.out_bf = out_bf;
     a.ldb = ldb;
     if (wbf) {
+        int dev = 0;
+        {
+            const hipError_t e = hipGetDevice(&dev);
+            if (e != hipSuccess) return e;
+            if (dev < 0 || dev >= PF_MAX_DEVICES) return hipErrorInvalidDevice;
+        }
         // 256 x 256 tiles (JT = 4) for as many row groups as fill whole rounds of the 256 CUs; what is left, or
         // a matrix too small for one such round, goes in 256 x 128 tiles (JT = 2), which spread it over twice
         // as many workgroups
@@ -1017,12 +1025,12 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
             const size_t lds = 2 * (size_t)(32768 + 64 * jt * 128);
 #define GO(E, J)                                                                                              \
     do {                                                                                                      \
-        static bool attr_set = false;                                                                         \
-        if (!attr_set) {                                                                                      \
+        static bool attr_set[PF_MAX_DEVICES] = {}; /* the attribute is kept per device */                     \
+        if (!attr_set[dev]) {                                                                                 \
             const hipError_t e = hipFuncSetAttribute((const void *)pf_gemm_bf16_kernel<E, J>,                 \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);   \
             if (e != hipSuccess) return e;                                                                    \
-            attr_set = true;                                                                                  \
+            attr_set[dev] = true;                                                                             \
         }                                                                                                     \
         hipLaunchKernelGGL((pf_gemm_bf16_kernel<E, J>), grid, dim3(512), lds, s, a, nt0, n_mt, n_tiles, per); \
     } while (0)
@@ -1055,12 +1063,12 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
                 const size_t lds = 2 * (size_t)(32768 + 256 * 128);
 #define GO(E)                                                                                                       \
     do {                                                                                                            \
-        static bool attr_set = false;                                                                               \
-        if (!attr_set) {                                                                                            \
+        static bool attr_set[PF_MAX_DEVICES] = {};                                                                  \
+        if (!attr_set[dev]) {                                                                                       \
             const hipError_t e = hipFuncSetAttribute((const void *)pf_gemm_bf16_mixed_kernel<E>,                    \
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);         \
             if (e != hipSuccess) return e;                                                                          \
-            attr_set = true;                                                                                        \
+            attr_set[dev] = true;                                                                                   \
         }                                                                                                           \
         hipLaunchKernelGGL((pf_gemm_bf16_mixed_kernel<E>), grid, dim3(512), lds, s, a, na, n_mt4, n_mt2, t4, t2, per4, per2); \
     } while (0)
