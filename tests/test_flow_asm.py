@@ -1,7 +1,9 @@
 """The streaming kernel polls activations with loads it issues from inline asm.  The compiler believes
 an asm statement's outputs valid as soon as the statement ends, so a load and the wait for it must be
 one statement; this test compiles k_flow.hip to assembly and checks that no register that such a load
-targets is read or written before the wait that follows it."""
+targets is read or written while the load can still be under way (loads complete in order: an asm-issued
+`s_waitcnt vmcnt(N)` leaves at most the N youngest; a variant with two polls under way, whose younger
+registers the compiler did read in a loop, was caught by this check)."""
 import os
 import re
 import shutil
@@ -24,13 +26,13 @@ def _regs(text):
 
 def _violations(path):
     """Linear scan: registers written by the asm-issued coherent 16-byte loads (`... sc1`) stay untouched
-    until an asm-issued s_waitcnt vmcnt."""
-    bad, fn, pending, in_asm, n_loads = [], None, {}, False, 0
+    until an asm-issued s_waitcnt vmcnt has retired the load."""
+    bad, fn, pending, in_asm, n_loads = [], None, [], False, 0   # pending: [(line, regs)], oldest first
     for ln, line in enumerate(open(path), 1):
         t = line.strip()
         m = re.match(r"^(_Z\w+):", t)
         if m:
-            fn, pending = m.group(1), {}
+            fn, pending = m.group(1), []
         if t.startswith(";;#ASMSTART"):
             in_asm = True
             continue
@@ -39,15 +41,21 @@ def _violations(path):
             continue
         if not t or t[0] in ";.":
             continue
-        if in_asm and "s_waitcnt vmcnt" in t:
-            pending = {}
+        m = re.search(r"s_waitcnt vmcnt\((\d+)\)", t)
+        if in_asm and m:
+            n = int(m.group(1))
+            pending = pending[len(pending) - n:] if n else []
             continue
+        live = set().union(*[r for _, r in pending]) if pending else set()
         if in_asm and t.startswith("global_load_dwordx4") and t.endswith("sc1"):
             n_loads += 1
-            for r in _regs(t.split(",")[0]):
-                pending[r] = ln
+            ops = t.split(None, 1)[1].split(",")
+            hit = _regs(",".join(ops[1:])) & live   # (asking again into a register whose load is under way is fine)
+            if hit:
+                bad.append((fn, ln, t, sorted(hit)))
+            pending.append((ln, _regs(ops[0])))
             continue
-        hit = _regs(t) & set(pending)
+        hit = _regs(t) & live
         if hit:
             bad.append((fn, ln, t, sorted(hit)))
     return bad, n_loads
