@@ -25,7 +25,7 @@ import __graft_entry__ as entry  # noqa: E402
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
 # (workload, launch path) -> bytes; path 1: per matvec launch, 31.23 MB read + 0.04 MB written
 # path 3: per token launch, 4474.4 MB read + 9.5 MB written (profiles/pmc_fetch_write_bench_8b-q4ks_streaming.md)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4505800000}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4505400000}
 
 WORKLOADS = {
     # name: (plan, config kwargs, prompt length)
