@@ -300,3 +300,37 @@ def test_temperature_sampling_on_device(pkg, rng):
         dev.sample_token(0.0, 0.5)
     with pytest.raises(pkg.L2HError):
         dev.sample_token(1.0, 1.0)
+
+
+def test_full_size_model_launch_paths_agree(pkg):
+    """The benchmark's model at its full size (Llama-3-8B shape: 32 layers, vocabulary 128256, q4_K layers, q6_K
+    output), too large for the CPU oracle to follow in a test: the two launch paths that share no kernel
+    code beyond the arithmetic helpers must give the same 128 greedy tokens and bit-identical final logits,
+    and the prompt pass must leave the same logits and cache with and without its bf16 weight copy."""
+    from llama2_jl_amd import synth
+    kw = dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8, vocab_size=128256, seq_len=512,
+              rope_freq_base=500000.0, rope_is_neox=False)
+    prompt = synth.seeded_prompt(7, 32, kw["vocab_size"])
+    got = {}
+    for path in (1, 3):
+        lm = _model(pkg, "PLAN_Q4_K_S", **kw)
+        dev = lm.device(path=path)
+        assert dev.path == path
+        ids, logits = dev.generate_greedy(prompt, 128, want_logits=True)
+        got[path] = (np.asarray(ids), logits.copy())
+        if path == 1:
+            long_prompt = synth.seeded_prompt(8, 300, kw["vocab_size"])
+            pf = []
+            for on in (True, False):
+                dev.set_prefill_copy(on)
+                dev.reset()
+                pl, nxt = dev.prefill(long_prompt, 0)
+                k, v = dev.kv_read(31, 0, 300)
+                pf.append((pl.copy(), nxt, k.copy(), v.copy()))
+            assert pf[0][1] == pf[1][1]
+            assert np.array_equal(pf[0][0], pf[1][0])
+            assert np.array_equal(pf[0][2], pf[1][2]) and np.array_equal(pf[0][3], pf[1][3])
+        dev.close()
+        del dev, lm
+    assert got[1][0].tolist() == got[3][0].tolist()
+    assert np.array_equal(got[1][1], got[3][1])
