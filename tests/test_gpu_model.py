@@ -313,19 +313,21 @@ def test_full_size_model_launch_paths_agree(pkg):
     prompt = synth.seeded_prompt(7, 32, kw["vocab_size"])
     got = {}
     for path in (1, 3):
-        lm = _model(pkg, "PLAN_Q4_K_S", **kw)
+        # (the streaming kernel takes short caches only; the prompt pass below needs room for 2048 positions)
+        lm = _model(pkg, "PLAN_Q4_K_S", **dict(kw, seq_len=512 if path == 3 else 2112))
         dev = lm.device(path=path)
         assert dev.path == path
         ids, logits = dev.generate_greedy(prompt, 128, want_logits=True)
         got[path] = (np.asarray(ids), logits.copy())
         if path == 1:
-            long_prompt = synth.seeded_prompt(8, 300, kw["vocab_size"])
+            # 2048 positions: the shapes at which the product kernels split a matrix over two tile sizes
+            long_prompt = synth.seeded_prompt(8, 2048, kw["vocab_size"])
             pf = []
             for on in (True, False):
                 dev.set_prefill_copy(on)
                 dev.reset()
                 pl, nxt = dev.prefill(long_prompt, 0)
-                k, v = dev.kv_read(31, 0, 300)
+                k, v = dev.kv_read(31, 0, 2048)
                 pf.append((pl.copy(), nxt, k.copy(), v.copy()))
             assert pf[0][1] == pf[1][1]
             assert np.array_equal(pf[0][0], pf[1][0])
