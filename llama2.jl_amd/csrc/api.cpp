@@ -729,6 +729,9 @@ static int flow_setup(l2h_model *m) {
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: %s", why.c_str()) : L2H_OK;
     if (m->L(0, L2H_RMS_ATT).layer_stride != m->L(0, L2H_RMS_FFN).layer_stride)
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ") : L2H_OK;
+    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount))
+        return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: its workgroups do not fit the device at once")
+                        : L2H_OK;
     std::vector<int64_t> off;
     const int64_t total = k_flow_offsets(a, cls_type, grid, off);
     unsigned char *stream = nullptr;

@@ -1553,9 +1553,23 @@ hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a) {
     return hipStreamSynchronize(s);
 }
 
+// Whether `grid` workgroups of the kernel can be resident at once on a device of n_cu CUs that runs nothing
+// else.  The kernel has no grid-wide barrier and every wait in it is bounded, so residency is what makes it
+// fast, not what makes it correct: workgroups that had to wait for a CU would let the others run into their
+// wait limit, and the launch would end with the error that l2h_model_set_wait_limit describes.
+bool k_flow_fits(int cls_type, int grid, int n_cu) {
+    const void *fn = cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K>
+                                               : (const void *)flow_token_kernel<L2H_TYPE_Q4_K>;
+    int per_cu = 0;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 1024, 0) != hipSuccess) return false;
+    return per_cu >= 1 && (int64_t)per_cu * n_cu >= grid;
+}
+
+// A plain launch: a cooperative one costs about 20 µs more per token on this stack, and all it would add is the
+// residency check that k_flow_fits makes once.
 hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid) {
     void *args[] = {&gen0};
     const void *fn = cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K>
                                                : (const void *)flow_token_kernel<L2H_TYPE_Q4_K>;
-    return hipLaunchCooperativeKernel(fn, dim3(grid), dim3(1024), args, 0, s);
+    return hipLaunchKernel(fn, dim3(grid), dim3(1024), args, 0, s);
 }

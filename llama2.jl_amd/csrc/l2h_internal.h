@@ -168,6 +168,7 @@ hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream
                          int layer, const DevTensor *w, int nw, int grid, int cls_type);
 hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a);
 hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid);
+bool k_flow_fits(int cls_type, int grid, int n_cu);
 
 // ---- launchers (kernel files) ----------------------------------------------------------------
 // Each returns hipGetLastError() of its launch.
