@@ -17,6 +17,8 @@
 //    marked empty again) only two or more phases after its last read, and reaching a phase requires every
 //    workgroup to have finished the phase before the previous one, so a word is never overwritten while
 //    somebody may still want its old value.
+//    The caller puts all these words into uncached device memory: a store there reaches a poller on another
+//    XCD sooner than through the L2s.
 //
 //  Besides: a few pieces per phase travel through registers, requested while the phase waits for its
 //  input (see flow_reg_pieces), and the attention is built for low latency (flow_attention_short).
