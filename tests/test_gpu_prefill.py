@@ -139,3 +139,7 @@ def test_prefill_argument_checks(pkg):
         dev.prefill([1, 2, 3], lm.config.seq_len - 2)
     with pytest.raises(pkg.L2HError):
         dev.prefill([lm.config.vocab_size], 0)
+    # l2h_model_set_prefill_copy takes 0 or 1
+    from llama2_jl_amd import _lib
+    assert _lib.lib().l2h_model_set_prefill_copy(dev.handle, 2) != 0
+    assert _lib.lib().l2h_model_set_prefill_copy(dev.handle, 1) == 0
