@@ -117,9 +117,10 @@ __host__ __device__ inline int flow_wave_start(const FlowGeom &g, int wg, int wa
 // of that wait a wavefront therefore requests the last FLOW_R pieces of its run for the phase into
 // registers; the ring's stream passes over them (they sit in a part of the wavefront's stream of their
 // own).  That moves their share of the HBM time out of the loops; the price is that the wait's first poll
-// returns after them (loads return in order), which is why there are only a few.
+// returns after them (loads return in order), which is why there are only a few: one is the best count now,
+// two were while the waits themselves took longer.
 #ifndef FLOW_R
-#define FLOW_R 2
+#define FLOW_R 1
 #endif
 __host__ __device__ inline int flow_reg_pieces(const FlowGeom &g, int wg, int wave) {
     const int cnt = flow_wave_pieces(g, wg, wave);
