@@ -172,6 +172,23 @@ def test_attention(pkg, orc, ctx, rng, hs, n_heads, n_kv, pos):
     assert _rel(out, want) <= 2e-6
 
 
+@pytest.mark.parametrize("hs,n_heads,n_kv,pos", [(96, 32, 32, 2047), (96, 32, 32, 2113), (96, 32, 32, 4000),
+                                                 (128, 32, 8, 4000), (64, 6, 2, 1500), (128, 4, 2, 700)])
+def test_attention_long_cache(pkg, orc, ctx, rng, hs, n_heads, n_kv, pos):
+    """Caches of many 64-timestep tiles per head (scores, softmax and value sums in separate launches, the
+    value sums split over the tiles); one row with scores far above the others'."""
+    from llama2_jl_amd import _lib
+    q = rng.standard_normal(hs * n_heads).astype(np.float32)
+    kc = rng.standard_normal((pos + 1, hs * n_kv)).astype(np.float32)
+    vc = rng.standard_normal((pos + 1, hs * n_kv)).astype(np.float32)
+    kc[pos // 3] *= 3.0
+    out = np.empty(hs * n_heads, np.float32)
+    ctx.check(_lib.lib().l2h_attention(ctx.handle, _lib.ptr(out), _lib.ptr(q), _lib.ptr(kc), _lib.ptr(vc), hs, n_heads,
+                                       n_kv, pos))
+    want, _ = orc.attention(q, kc, vc, hs, n_heads, n_kv, pos, orc.GPU_SPEC)
+    assert _rel(out, want) <= 2e-6
+
+
 def test_swiglu(pkg, orc, ctx, rng):
     from llama2_jl_amd import _lib
     n = 1376
