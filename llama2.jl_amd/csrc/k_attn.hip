@@ -103,12 +103,12 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(const double *part, fl
     out[e] = (float)acc;
 }
 
-// ---- long caches: three launches sized to fill the chip --------------------------------------
+// ---- long caches: launches sized to fill the chip (scores, exponentials, values, final sum) ----
 // Scores: a workgroup = 64 timesteps of GH heads that share a KV head; wavefront w takes quarter w
 // of the head dimension (all of its 16-byte loads in flight at once), the quarters are added in
 // fixed order through LDS.
 template <int GH>
-__global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, const float *kc, float *att,
+__global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, const float *kc, float *att, float *tmax,
                                                            const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
                                                            int seq_len) {
     __shared__ double s_q[GH * 128];
@@ -148,27 +148,66 @@ __global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, con
     for (int g = 0; g < GH; g++) s_part[part][g][lane] = acc[g];
     __syncthreads();
     const float scale = sqrtf((float)hs);
-    for (int i = threadIdx.x; i < GH * 64; i += 256) {
-        const int g = i >> 6, l = i & 63;
-        if (t0 + l > pos) continue;
+    if (threadIdx.x < GH * 64) {  // wavefront g: the 64 scores of head h0 + g, and the largest of them
+        const int g = part, l = lane;
+        const bool there = t0 + l <= pos;
         const double v = ((s_part[0][g][l] + s_part[1][g][l]) + s_part[2][g][l]) + s_part[3][g][l];
-        att[(int64_t)(h0 + g) * seq_len + t0 + l] = (float)v / scale;
+        const float sc = (float)v / scale;
+        if (there) att[(int64_t)(h0 + g) * seq_len + t0 + l] = sc;
+        const float m = wave_max_f32(there ? sc : -INFINITY);
+        if (l == 0) tmax[(int64_t)(h0 + g) * gridDim.x + blockIdx.x] = m;
     }
 }
 
+// Softmax over a long cache, first half: a workgroup takes 1024 timesteps of one head.  The head's
+// maximum comes from the tiles' maxima; e = fp32(exp(score - max)) replaces the score, the fp64 sum of the
+// workgroup's e goes to psum[head][workgroup].  The division by the total is left to the value pass.
+__global__ __launch_bounds__(256) void attn_exp_kernel(float *att, const float *tmax, double *psum, const DecodeCtl *ctl,
+                                                       int seq_len, int ntiles) {
+    __shared__ double redd[4];
+    __shared__ float redf[4];
+    const int pos = ctl->pos, h = blockIdx.y, c0 = blockIdx.x * 1024;
+    if (c0 > pos) return;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i <= pos / 64; i += 256) mx = fmaxf(mx, tmax[(int64_t)h * ntiles + i]);
+    mx = block_max_f32(mx, redf);
+    float *x = att + (int64_t)h * seq_len;
+    double acc = 0.0;
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int t = c0 + threadIdx.x + 256 * k;
+        if (t <= pos) {
+            const float e = (float)exp((double)(x[t] - mx));
+            x[t] = e;
+            acc += (double)e;
+        }
+    }
+    acc = block_sum_f64(acc, redd);
+    if (threadIdx.x == 0) psum[(int64_t)h * gridDim.x + blockIdx.x] = acc;
+}
+
 // Values: a workgroup = `chunk` (a multiple of 64) timesteps of GH heads sharing a KV head; thread =
-// (16-byte group of the head dimension, timestep group), eight loads in flight per round; fp64
+// (16-byte group of the head dimension, timestep group), eight loads in flight per round; the
+// probabilities p = e / total are formed here (fp32 division, as softmax! does), widened to fp64; fp64
 // partial sums per workgroup go to `part`, which attn_reduce4_kernel adds in block order.
 template <int GH>
-__global__ __launch_bounds__(256) void attn_av4_kernel(const double *pd, const float *vc, double *part,
-                                                       const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
-                                                       int seq_len, int chunk) {
+__global__ __launch_bounds__(256) void attn_av4_kernel(const float *att, const double *psum, int npsum, const float *vc,
+                                                       double *part, const DecodeCtl *ctl, int hs, int n_heads,
+                                                       int n_kv_heads, int seq_len, int chunk) {
     __shared__ double s_p[GH][64];
     __shared__ double s_red[8][GH][128];
     const int pos = ctl->pos;
     const int split = blockIdx.x, c0 = split * chunk;
     if (c0 > pos) return;
     const int h0 = blockIdx.y * GH, kvh = h0 / (n_heads / n_kv_heads);
+    // the heads' totals: the sums of attn_exp_kernel's workgroups in their order, rounded to fp32 (softmax!'s sum)
+    float sf[GH];
+#pragma unroll
+    for (int g = 0; g < GH; g++) {
+        double t = 0.0;
+        for (int c = 0; c <= pos / 1024; c++) t += psum[(int64_t)(h0 + g) * npsum + c];
+        sf[g] = (float)t;
+    }
     const int n4 = hs >> 2, ngrp = min(8, 256 / n4);  // hs <= 128
     const int i4 = threadIdx.x % n4, tg = threadIdx.x / n4;
     const bool active = tg < ngrp;
@@ -180,7 +219,10 @@ __global__ __launch_bounds__(256) void attn_av4_kernel(const double *pd, const f
         __syncthreads();
         for (int i = threadIdx.x; i < GH * 64; i += 256) {
             const int g = i >> 6, l = i & 63;
-            s_p[g][l] = l < nt ? pd[(int64_t)(h0 + g) * seq_len + t0 + l] : 0.0;
+            float sg = sf[0];
+#pragma unroll
+            for (int k = 1; k < GH; k++) sg = g == k ? sf[k] : sg;
+            s_p[g][l] = l < nt ? (double)(att[(int64_t)(h0 + g) * seq_len + t0 + l] / sg) : 0.0;
         }
         float4 v[8];
         if (active) {
@@ -270,18 +312,22 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
                               int n_heads, int n_kv_heads, int seq_len) {
     const int ntiles = (seq_len + L2H_ATT_TILE - 1) / L2H_ATT_TILE;
     if (hs <= 128 && hs % 16 == 0 && L2H_ATT_TILE == 64) {
-        hipLaunchKernelGGL((attn_scores4_kernel<GH>), dim3(ntiles, n_heads / GH), dim3(256), 0, s, qd, kc, att, ctl, hs,
-                           n_heads, n_kv_heads, seq_len);
+        // (pd, seq_len doubles per head, holds the softmax workgroups' sums and after them the tiles' maxima)
+        const int npsum = (seq_len + 1023) / 1024;
+        double *psum = pd;
+        float *tmax = (float *)(pd + (int64_t)n_heads * npsum);
+        hipLaunchKernelGGL((attn_scores4_kernel<GH>), dim3(ntiles, n_heads / GH), dim3(256), 0, s, qd, kc, att, tmax, ctl,
+                           hs, n_heads, n_kv_heads, seq_len);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(attn_softmax_kernel, dim3(n_heads), dim3(1024), 0, s, att, pd, ctl, seq_len);
+        hipLaunchKernelGGL(attn_exp_kernel, dim3(npsum, n_heads), dim3(256), 0, s, att, tmax, psum, ctl, seq_len, ntiles);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         // timesteps per value workgroup: as large as still leaves about 512 workgroups over a full cache
         int chunk = 64;
         while (chunk < 512 && (int64_t)(seq_len / (2 * chunk)) * (n_heads / GH) >= 512) chunk *= 2;
-        hipLaunchKernelGGL((attn_av4_kernel<GH>), dim3((seq_len + chunk - 1) / chunk, n_heads / GH), dim3(256), 0, s, pd,
-                           vc, part, ctl, hs, n_heads, n_kv_heads, seq_len, chunk);
+        hipLaunchKernelGGL((attn_av4_kernel<GH>), dim3((seq_len + chunk - 1) / chunk, n_heads / GH), dim3(256), 0, s, att,
+                           psum, npsum, vc, part, ctl, hs, n_heads, n_kv_heads, seq_len, chunk);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
         const int dim = hs * n_heads;
