@@ -173,4 +173,59 @@ function sample(m::DeviceModel, model::LanguageModel, prompt::String = ""; tempe
     return nothing
 end
 
+# ---- the single operators (each one seam of src/inference.jl / src/matmul.jl; host arrays in, host arrays out) ----
+
+"`matmul!(y, A, x)` (src/matmul.jl:3-23) on the GPU: A is `(in, out)` of Float32 or `(in ÷ 256, out)` of k-quant blocks."
+function matmul!(ctx::Context, y::Vector{Float32}, A::AbstractMatrix, x::Vector{Float32})
+    host = A isa Array ? A : collect(A)
+    ne0, ne1 = in_out(host)
+    @assert length(x) == ne0 && length(y) == ne1
+    GC.@preserve host check(ctx.handle, ccall((:l2h_matmul, lib), Cint,
+        (Ptr{Cvoid}, Cint, Ptr{Cvoid}, Int64, Int64, Ptr{Float32}, Ptr{Float32}, Ptr{Int32}, Ptr{Int32}),
+        ctx.handle, ggml_type(host), pointer(host), ne0, ne1, x, y, C_NULL, C_NULL))
+    return y
+end
+
+"`dequantize!(y, x)` (src/kquants.jl:70-125, 186-251, 322-363) of a vector of k-quant blocks."
+function dequantize!(ctx::Context, y::Vector{Float32}, x::Vector{T}) where {T <: Union{block_q4_K, block_q5_K, block_q6_K}}
+    @assert length(y) == 256 * length(x)
+    check(ctx.handle, ccall((:l2h_dequantize, lib), Cint, (Ptr{Cvoid}, Cint, Ptr{Cvoid}, Int64, Ptr{Float32}),
+                            ctx.handle, ggml_type(x), x, length(x), y))
+    return y
+end
+
+"`rmsnorm!(o, x, weight)` (src/inference.jl:102-110); `o` may be `x`."
+function rmsnorm!(ctx::Context, o::Vector{Float32}, x::Vector{Float32}, weight::Vector{Float32})
+    check(ctx.handle, ccall((:l2h_rmsnorm, lib), Cint, (Ptr{Cvoid}, Ptr{Float32}, Ptr{Float32}, Ptr{Float32}, Int64),
+                            ctx.handle, o, x, weight, length(x)))
+    return o
+end
+
+"`rope!(x, pos, config)` (src/inference.jl:112-167) on `x` of `(head_size, n_heads)`; `pos` is 1-based."
+function rope!(ctx::Context, x::Matrix{Float32}, pos::Int, config::ModelConfig)
+    check(ctx.handle, ccall((:l2h_rope, lib), Cint, (Ptr{Cvoid}, Ptr{Float32}, Cint, Cint, Cint, Cfloat, Cint),
+                            ctx.handle, x, size(x, 1), size(x, 2), pos - 1, config.rope_freq_base, config.rope_is_neox ? 1 : 0))
+    return x
+end
+
+"`softmax!(x)` (src/inference.jl:169-174)."
+function softmax!(ctx::Context, x::Vector{Float32})
+    check(ctx.handle, ccall((:l2h_softmax, lib), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int64), ctx.handle, x, length(x)))
+    return x
+end
+
+"First index of the largest element, 1-based, as `argmax(logits)` in `sample` (src/inference.jl:360)."
+function argmax_first(ctx::Context, x::Vector{Float32})
+    out = Ref{Int32}(0)
+    check(ctx.handle, ccall((:l2h_argmax, lib), Cint, (Ptr{Cvoid}, Ptr{Float32}, Int64, Ref{Int32}), ctx.handle, x, length(x), out))
+    return Int(out[]) + 1
+end
+
+"Rows `pos .. pos+n-1` (1-based) of a layer's K and V cache, each `(kv_dim, n)` on this side (src/inference.jl:259-260)."
+function kv_write!(m::DeviceModel, layer::Int, pos::Int, k::Matrix{Float32}, v::Matrix{Float32})
+    @assert size(k) == size(v)
+    check(m.ctx.handle, ccall((:l2h_kv_write, lib), Cint, (Ptr{Cvoid}, Cint, Cint, Cint, Ptr{Float32}, Ptr{Float32}),
+                              m.handle, layer - 1, pos - 1, size(k, 2), k, v))
+end
+
 end # module
