@@ -189,6 +189,21 @@ def test_attention_long_cache(pkg, orc, ctx, rng, hs, n_heads, n_kv, pos):
     assert _rel(out, want) <= 2e-6
 
 
+@pytest.mark.parametrize("hs,n_heads,n_kv,pos", [(72, 4, 2, 300), (40, 6, 3, 70), (256, 2, 1, 100), (8, 3, 3, 0)])
+def test_attention_other_head_sizes(pkg, orc, ctx, rng, hs, n_heads, n_kv, pos):
+    """Head sizes that are not a multiple of 16, or above 128: the general kernels (one lane per timestep
+    for the scores, one thread per feature for the values)."""
+    from llama2_jl_amd import _lib
+    q = rng.standard_normal(hs * n_heads).astype(np.float32)
+    kc = rng.standard_normal((pos + 1, hs * n_kv)).astype(np.float32)
+    vc = rng.standard_normal((pos + 1, hs * n_kv)).astype(np.float32)
+    out = np.empty(hs * n_heads, np.float32)
+    ctx.check(_lib.lib().l2h_attention(ctx.handle, _lib.ptr(out), _lib.ptr(q), _lib.ptr(kc), _lib.ptr(vc), hs, n_heads,
+                                       n_kv, pos))
+    want, _ = orc.attention(q, kc, vc, hs, n_heads, n_kv, pos, orc.GPU_SPEC)
+    assert _rel(out, want) <= 2e-6
+
+
 def test_swiglu(pkg, orc, ctx, rng):
     from llama2_jl_amd import _lib
     n = 1376
