@@ -8,6 +8,10 @@
 // contiguous 16-byte pieces); V cache: [n_kv_heads][seq_len][hs] (a lane per feature).
 #include "matvec_dev.h"
 
+#ifndef L2H_AV_MIN_WGS
+#define L2H_AV_MIN_WGS 1024  // the value pass splits a full cache over at least this many workgroups (512: 0.5 % slower, 2048: 2 %)
+#endif
+
 // One wavefront: 64 consecutive timesteps of GH query heads that share one KV head.
 template <int GH>
 __global__ __launch_bounds__(256) void attn_scores_kernel(const double *qd, const float *kc, float *att,
@@ -323,9 +327,9 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
         hipLaunchKernelGGL(attn_exp_kernel, dim3(npsum, n_heads), dim3(256), 0, s, att, tmax, psum, ctl, seq_len, ntiles);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
-        // timesteps per value workgroup: as large as still leaves about 512 workgroups over a full cache
+        // timesteps per value workgroup: as large as still leaves L2H_AV_MIN_WGS workgroups over a full cache
         int chunk = 64;
-        while (chunk < 512 && (int64_t)(seq_len / (2 * chunk)) * (n_heads / GH) >= 512) chunk *= 2;
+        while (chunk < 512 && (int64_t)(seq_len / (2 * chunk)) * (n_heads / GH) >= L2H_AV_MIN_WGS) chunk *= 2;
         hipLaunchKernelGGL((attn_av4_kernel<GH>), dim3((seq_len + chunk - 1) / chunk, n_heads / GH), dim3(256), 0, s, att,
                            psum, npsum, vc, part, ctl, hs, n_heads, n_kv_heads, seq_len, chunk);
         e = hipGetLastError();
