@@ -112,10 +112,6 @@ function generate(m::DeviceModel, prompt::Vector{Int}, n_new::Int; pos::Int = 1)
     return Int.(out) .+ 1
 end
 
-"""
-    sample(m::DeviceModel, model::LanguageModel, prompt=""; temperature=0.9f0, stop_on_special_token=true,
-           max_seq_len=typemax(Int), bos_token=true)
-
 # Whole prompt in one pass on the matrix cores (no counterpart in Llama2.jl, which feeds the prompt token
 # by token): fills the cache for positions pos .. pos+length(prompt)-1 and returns the next token (1-based).
 function prefill!(m::DeviceModel, prompt::Vector{Int}; pos::Int = 1)
@@ -136,7 +132,23 @@ function sample_token(m::DeviceModel, temperature::Float32; u::Float32 = min(ran
     return Int(tok[]) + 1
 end
 
-Same behaviour and output as `Llama2.sample` (src/inference.jl:317-395).
+# One step without copying the logits back: returns the argmax (1-based); the logits stay on the device
+# for sample_token.
+function step!(m::DeviceModel, token::Int, pos::Int)
+    am = Ref{Int32}(0)
+    check(m.ctx.handle, ccall((:l2h_forward, lib), Cint, (Ptr{Cvoid}, Cint, Cint, Ptr{Float32}, Ref{Int32}),
+                              m.handle, token - 1, pos - 1, C_NULL, am))
+    return Int(am[]) + 1
+end
+
+"""
+    sample(m::DeviceModel, model::LanguageModel, prompt=""; temperature=0.9f0, stop_on_special_token=true,
+           max_seq_len=typemax(Int), bos_token=true)
+
+Same behaviour and output as `Llama2.sample` (src/inference.jl:317-395): the prompt is encoded with the
+model's tokenizer, BOS is pushed in front (:338-340), tokens are printed as they are chosen, generation
+stops at BOS/EOS (:371-373) and the tok/s line closes the output (:392).  The forward pass, the argmax
+and the temperature draw run on the device; the uniform number of the draw comes from Julia's RNG.
 """
 function sample(m::DeviceModel, model::LanguageModel, prompt::String = ""; temperature::Float32 = 0.9f0,
                 stop_on_special_token = true, max_seq_len = typemax(Int), bos_token = true)
@@ -144,23 +156,20 @@ function sample(m::DeviceModel, model::LanguageModel, prompt::String = ""; tempe
     config, tokenizer = model.config, model.tokenizer
     prompt_tokens = encode(prompt, tokenizer)
     reset!(m)
-    logits = Vector{Float32}(undef, config.vocab_size)
     time_start = time_ns()
     bos_token && pushfirst!(prompt_tokens, tokenizer.bos_token_id)
     !bos_token && print(tokenizer.id_to_token[prompt_tokens[1]])
     token = prompt_tokens[1]
     generated_seq_len = 0
     for pos in 1:min(config.seq_len, max_seq_len)
-        am = transformer!(logits, m, token, pos)
+        am = step!(m, token, pos)
         generated_seq_len += 1
         if pos + 1 <= length(prompt_tokens)
             next = prompt_tokens[pos + 1]
         elseif temperature == 0f0
             next = am
         else
-            logits ./= temperature
-            Llama2.softmax!(logits)
-            next = Llama2.wsample(1:config.vocab_size, logits)
+            next = sample_token(m, temperature)
         end
         if stop_on_special_token && (next == tokenizer.bos_token_id || next == tokenizer.eos_token_id)
             break

@@ -2,8 +2,9 @@
 
 The oracle runs in the mode the HIP path implements (q8_K activations for k-quant weights,
 fp64-accumulated sums): logits within 1e-3 relative max-abs (the stated bar; the observed
-difference is ~1e-6) and identical greedy token sequences.  The deviation from the reference's
-float-activation arithmetic (oracle mode 0) is printed as information.
+difference is ~1e-6) and identical greedy token sequences.  The distance to the reference's
+float-activation arithmetic (oracle mode 0) is measured teacher-forced, position by position, in
+test_distance_to_reference_float_arithmetic.
 """
 import numpy as np
 import pytest
@@ -73,13 +74,53 @@ def test_forward_and_greedy(pkg, orc, case, path):
     ids, logits = dev.generate_greedy(prompt, n_new, want_logits=True)
     ref_ids, ref_logits = om.generate_greedy(prompt, n_new, orc.GPU_SPEC)
     err = _rel(logits, ref_logits)
-    om.reset()
-    f_ids, f_logits = om.generate_greedy(prompt, n_new, orc.REFERENCE)
-    agree = int(np.argmax(np.append(ids != f_ids, True)))
-    print("\n[%s path %d] logits rel err vs oracle(q8k,fp64 sums) %.3g; vs reference float path: %d/%d tokens agree, "
-          "final-logit rel diff %.3g" % (case, path, err, agree, n_new, _rel(logits, f_logits)))
+    print("\n[%s path %d] logits rel err vs oracle(q8k,fp64 sums) %.3g" % (case, path, err))
     assert ids.tolist() == ref_ids.tolist(), case
     assert err <= 1e-3, case
+
+
+HEADLINE_2L = ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=32000,
+                                   seq_len=192, rope_freq_base=500000.0, rope_is_neox=False))
+
+
+@pytest.mark.parametrize("case", sorted(CASES) + ["headline_widths"])
+def test_distance_to_reference_float_arithmetic(pkg, orc, case):
+    """How far the device path (q8_K activations, integer dot products) is from the reference's own
+    arithmetic (float activations times dequantized weights, reference src/kquants.jl:127-184), measured
+    teacher-forced: the oracle in mode 0 generates greedily, and the token it fed at every position is
+    fed to the device too, so both sides see the same history and the per-position difference is the
+    error of one forward pass, not the divergence of two sequences.  Reported per case: the largest and
+    the median relative max-abs logit difference over the positions, and how often the two agree on the
+    most likely token.  F32 models take no q8_K step: they must agree to round-off."""
+    from llama2_jl_amd import synth
+    plan, kw = HEADLINE_2L if case == "headline_widths" else CASES[case]
+    lm = _model(pkg, plan, **kw)
+    cfg = lm.config
+    prompt = synth.seeded_prompt(5, 6, cfg.vocab_size)
+    n_new = min(40, cfg.seq_len - len(prompt))
+    om = orc.model_from_language_model(lm, nthreads=16)
+    f_ids, _ = om.generate_greedy(prompt, n_new, orc.REFERENCE)
+    fed = list(prompt) + [int(t) for t in f_ids[:-1]]
+    dev = lm.device()
+    dev.reset()
+    om.reset()
+    errs, agree = [], 0
+    for pos, tok in enumerate(fed):
+        logits, am = dev.forward(int(tok), pos)
+        ref = om.forward(int(tok), pos, orc.REFERENCE)
+        errs.append(_rel(logits, ref))
+        agree += int(am == orc.argmax(ref))
+    errs = np.array(errs)
+    print("\n[%s, launch path %d] teacher-forced against the reference's float arithmetic, %d positions: logit rel "
+          "diff max %.3g median %.3g; same top-1 token at %d/%d positions"
+          % (case, dev.path, len(fed), errs.max(), float(np.median(errs)), agree, len(fed)))
+    if plan == "PLAN_F32":
+        assert errs.max() <= 1e-5 and agree == len(fed)
+    else:
+        # the q8_K step: 8 bits per activation, about 0.7 % RMS per matvec
+        assert errs.max() <= 0.15
+    dev.close()
+    om.close()
 
 
 def test_headline_shape_128_greedy_tokens(pkg, orc):

@@ -23,6 +23,93 @@ def test_library_exports_every_declared_symbol(pkg):
     assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
 
 
+def _c_prototypes():
+    """name -> list of C parameter types, from include/l2h.h"""
+    header = open(os.path.join(ROOT, "include", "l2h.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    protos = {}
+    for m in re.finditer(r"\b(?:int|void|const char \*)\s*\*?\s*(l2h_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", header, flags=re.S):
+        params = [a.strip() for a in m.group(2).split(",")]
+        protos[m.group(1)] = [] if params == ["void"] else params
+    return protos
+
+
+def _julia_class(t):
+    """coarse class of a Julia ccall argument type"""
+    t = t.strip()
+    if t in ("Cint", "Int32", "UInt32", "Cuint"):
+        return "i32"
+    if t in ("Int64", "UInt64"):
+        return "i64"
+    if t in ("Cfloat", "Float32"):
+        return "f32"
+    if t.startswith("Ptr{") or t.startswith("Ref{") or t == "Cstring":
+        return "ptr"
+    raise AssertionError("unclassified Julia type " + t)
+
+
+def _c_class(p):
+    if "*" in p:
+        return "ptr"
+    base = " ".join(p.split()[:-1]) if len(p.split()) > 1 else p
+    if base in ("int", "int32_t", "unsigned int", "uint32_t"):
+        return "i32"
+    if base in ("int64_t", "uint64_t"):
+        return "i64"
+    if base == "float":
+        return "f32"
+    raise AssertionError("unclassified C parameter " + p)
+
+
+def test_julia_binding_matches_the_header():
+    """Nobody can run Julia where this library is built, so the binding is checked as text: every ccall in
+    llama2.jl_amd/julia/Llama2HIP.jl names a function the header declares, passes as many arguments as its
+    prototype has, of the same class (32-bit integer, 64-bit integer, float, pointer) in the same order;
+    and the functions the integration notes promise are defined at top level, outside any string."""
+    src = open(os.path.join(ROOT, "llama2.jl_amd", "julia", "Llama2HIP.jl")).read()
+    assert src.count('"""') % 2 == 0
+    code = re.sub(r'""".*?"""', "", src, flags=re.S)      # docstrings out
+    code = re.sub(r"(?m)#.*$", "", code)                   # comments out
+    protos = _c_prototypes()
+    assert len(protos) >= 30
+    calls = list(re.finditer(r"ccall\(\(:(l2h_[a-z0-9_]+),\s*lib\),\s*(\w+),\s*\(([^()]*?)\),", code, flags=re.S))
+    assert len(calls) >= 15
+    for m in calls:
+        name, ret, types = m.group(1), m.group(2), m.group(3)
+        assert name in protos, name + " is not declared in include/l2h.h"
+        jl = [t for t in (x.strip() for x in types.split(",")) if t]
+        want = protos[name]
+        assert len(jl) == len(want), "%s: %d ccall argument types, prototype has %d" % (name, len(jl), len(want))
+        for i, (a, b) in enumerate(zip(jl, want)):
+            assert _julia_class(a) == _c_class(b), "%s argument %d: Julia %s vs C %s" % (name, i, a, b)
+        # the values passed: as many as the types (counted up to the call's closing parenthesis)
+        depth, j = 1, m.end()
+        args, cur = [], ""
+        while depth > 0:
+            ch = code[j]
+            if ch in "([{":
+                depth += 1
+            elif ch in ")]}":
+                depth -= 1
+                if depth == 0:
+                    break
+            if ch == "," and depth == 1:
+                args.append(cur)
+                cur = ""
+            else:
+                cur += ch
+            j += 1
+        args.append(cur)
+        args = [a for a in (x.strip() for x in args) if a]
+        assert len(args) == len(jl), "%s: %d values for %d argument types" % (name, len(args), len(jl))
+        assert ret in ("Cint", "Cvoid", "Cstring")
+    defined = set(re.findall(r"(?m)^function\s+([A-Za-z_!0-9]+)\s*\(", code)) | \
+        set(re.findall(r"(?m)^([A-Za-z_!0-9]+)\([^\n]*\)\s*=", code))
+    for fn in ("Context", "DeviceModel", "set_tensor!", "reset!", "transformer!", "generate", "prefill!", "sample_token",
+               "sample", "matmul!", "dequantize!", "rmsnorm!", "rope!", "softmax!", "argmax_first", "kv_write!"):
+        assert fn in defined, "Llama2HIP.%s is not defined" % fn
+
+
 def test_no_device_is_an_error_not_a_fallback(pkg):
     """Without a GPU the context cannot be created; nothing computes on the CPU instead."""
     import ctypes

@@ -231,3 +231,97 @@ def test_transformer_against_float64(orc, rng, neox, n_kv):
     for _ in range(4):
         seq = seq + [int(np.argmax(np_ref.transformer_f32(cfg, W, seq)[-1]))]
     assert ids.tolist() == seq[3:]
+
+
+def test_q8k_half_way_cases_round_to_even(orc):
+    """Round-half-to-even in l2c_quantize_q8_K, with expected bytes written by hand.  The block's extreme is
+    -127, so iscale = -127 / -127 = 1 exactly and every other element x maps to rne(x): halves go to the
+    even neighbour (0.5 -> 0, 1.5 -> 2, 2.5 -> 2, -0.5 -> 0, -1.5 -> -2, -2.5 -> -2, 126.5 -> 126), where
+    round-half-away-from-zero would give 1, 2, 3, -1, -2, -3, 127.  With +127 as the extreme iscale is -1 and
+    the signs flip; a value whose product lies just beside a half rounds to the nearer integer."""
+    x = np.zeros(512, np.float32)
+    vals = [-127.0, 0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, -3.5, 126.5, -126.5, 0.49999997, 0.50000006, 1.0, -1.0, 63.5]
+    want = [-127, 0, 2, 2, 4, 0, -2, -2, -4, 126, -126, 0, 1, 1, -1, 64]
+    x[:16] = vals
+    x[256:256 + 16] = [-v for v in vals]  # extreme +127: iscale = -1, q = rne(-x) = the same integers
+    q = orc.quantize_q8_K(x)
+    assert q[0]["qs"][:16].tolist() == want
+    assert q[1]["qs"][:16].tolist() == want
+    assert q[0]["d"] == 1.0 and q[1]["d"] == -1.0
+    assert q[0]["bsums"][0] == sum(want) and not q[0]["qs"][16:].any()
+    # the clamp: a product that rounds to 128 cannot occur (|x| <= |max|), but +127.5-like cases stay at 127
+    y = np.zeros(256, np.float32)
+    y[0], y[1] = -254.0, 253.5   # iscale = 0.5: 253.5 * 0.5 = 126.75 -> 127
+    y[2] = 253.0                 # 126.5 -> 126 (half to even)
+    y[3] = 251.0                 # 125.5 -> 126
+    q = orc.quantize_q8_K(y)
+    assert q[0]["qs"][:4].tolist() == [-127, 127, 126, 126]
+
+
+def _quant_model(orc, rng, cfg, typ_layers, typ_out):
+    """a small k-quant model: random blocks (valid by construction), returned as oracle tensors and as the
+    float64-exact dequantized matrices of the same blocks"""
+    dim, hid, L, V = cfg["dim"], cfg["hidden_dim"], cfg["n_layers"], cfg["vocab_size"]
+    kv_dim = dim // cfg["n_heads"] * cfg["n_kv_heads"]
+    T, W = {}, dict(rms_final=rng.uniform(0.8, 1.2, dim).astype(np.float32))
+
+    def qmat(typ, rows, cols):
+        raw = rand_blocks(rng, typ, rows * (cols // 256))
+        return raw, np_ref.DEQUANT[typ](raw).reshape(rows, cols).astype(np.float32)
+
+    def put(role, layer, typ, raw, ne0, ne1):
+        T[(role, layer)] = (typ, raw, ne0, ne1)
+
+    raw, W["emb"] = qmat(Q4, V, dim)
+    put(orc.TOK_EMB, 0, Q4, raw, dim, V)
+    raw, W["output"] = qmat(typ_out, V, dim)
+    put(orc.OUTPUT, 0, typ_out, raw, dim, V)
+    T[(orc.RMS_FINAL, 0)] = (F32, W["rms_final"], dim, 1)
+    for name in ("rms_att", "rms_ffn", "wq", "wk", "wv", "wo", "w1", "w2", "w3"):
+        W[name] = []
+    shapes = dict(wq=(dim, dim), wk=(kv_dim, dim), wv=(kv_dim, dim), wo=(dim, dim), w1=(hid, dim), w2=(dim, hid),
+                  w3=(hid, dim))
+    roles = dict(wq=orc.WQ, wk=orc.WK, wv=orc.WV, wo=orc.WO, w1=orc.W1, w2=orc.W2, w3=orc.W3)
+    for l in range(L):
+        for name, role in (("rms_att", orc.RMS_ATT), ("rms_ffn", orc.RMS_FFN)):
+            w = rng.uniform(0.8, 1.2, dim).astype(np.float32)
+            W[name].append(w)
+            T[(role, l)] = (F32, w, dim, 1)
+        for name, (rows, cols) in shapes.items():
+            raw, deq = qmat(typ_layers[name], rows, cols)
+            W[name].append(deq)
+            put(roles[name], l, typ_layers[name], raw, cols, rows)
+    return T, W
+
+
+@pytest.mark.parametrize("plan", ["q4", "q5_q6"])
+def test_transformer_kquant_model_all_modes(orc, rng, plan):
+    """l2c_forward on a k-quant model (the wiring of the quantized matvecs, and the embedding row of a token
+    other than 0) against the float64 numpy transformer run on the dequantized matrices.  Mode 0 (float
+    activations) must agree to fp32 round-off; modes 1 and 3 (q8_K activations) differ from it by the
+    activation quantization step only, checked here as a bound far below what a wiring mistake (a swapped
+    matrix, a wrong row offset, a missing residual) would cause."""
+    cfg = dict(dim=256, hidden_dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=40, seq_len=8,
+               rope_freq_base=10000.0, rope_is_neox=False)
+    typ = dict.fromkeys(["wq", "wk", "wv", "wo", "w1", "w2", "w3"], Q4)
+    out = Q4
+    if plan == "q5_q6":
+        typ = dict(typ, **dict.fromkeys(["wq", "wk", "wv", "wo", "w1", "w3"], Q5), w2=Q6)
+        out = Q6
+    T, W = _quant_model(orc, rng, cfg, typ, out)
+    m = orc.Model(cfg, T)
+    tokens = [7, 39, 1, 7]
+    want = np_ref.transformer_f32(cfg, W, tokens)
+    for mode, tol in ((0, 5e-6), (2, 1e-6), (1, 5e-2), (3, 5e-2)):  # observed 1.2e-6, 1e-7, 1e-2 to 3e-2; a wrong embedding row: 1.2e-1
+        m.reset()
+        for pos, tok in enumerate(tokens):
+            got = m.forward(tok, pos, mode)
+            assert rel(got, want[pos]) < tol, (plan, mode, pos, rel(got, want[pos]))
+    # random blocks have scales of every size: the logits are large and structured, so a wiring mistake is
+    # an O(1) difference; the q8_K modes stay within a few per cent of the float path and of each other
+    m.reset()
+    a = [m.forward(t, p, 1) for p, t in enumerate(tokens)]
+    m.reset()
+    b = [m.forward(t, p, 3) for p, t in enumerate(tokens)]
+    for p in range(len(tokens)):
+        assert rel(a[p], b[p]) < 1e-4  # fp32 against fp64 sums of the same integer dot products
