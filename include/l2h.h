@@ -80,7 +80,8 @@ void l2h_model_destroy(l2h_model *m);
 /* Stands in for storing a host array in a TransformerWeights field: `host` holds ne1
  * output rows of ne0 input features, row-contiguous, as GGUF stores them and as
  * `view(A, :, i)` hands them to vecdot (src/matmul.jl:19).  k-quant types need
- * ne0 % 256 == 0 (src/load_gguf.jl:141).  Repacks into the device layout and uploads.
+ * ne0 % 256 == 0 (src/load_gguf.jl:141) and ne0 <= 16384 (the longest activation vector the
+ * matvec kernels stage; L2H_EINVAL beyond it).  Repacks into the device layout and uploads.
  * layer is ignored for the three per-model roles. */
 int l2h_model_set_tensor(l2h_model *m, int role, int layer, int ggml_type, const void *host, int64_t ne0,
                          int64_t ne1);
@@ -160,7 +161,7 @@ int l2h_dequantize(l2h_ctx *ctx, int ggml_type, const void *blocks, int64_t nb, 
 /* matmul!(y, A, x) (src/matmul.jl:3-23): uploads A (ne0 x ne1, as set_tensor), runs the
  * same matvec kernel the model uses (k-quant: on q8_K-quantized x; F32: on x), y[ne1].
  * I_sc / I_min (may be NULL; k-quant only) receive, per (row, super-block), the integer
- * sums the kernel formed: [ne1][ne0/256] int32 each. */
+ * sums the kernel formed: [ne1][ne0/256] int32 each.  k-quant: ne0 <= 16384. */
 int l2h_matmul(l2h_ctx *ctx, int ggml_type, const void *A, int64_t ne0, int64_t ne1, const float *x, float *y,
                int32_t *I_sc, int32_t *I_min);
 /* rmsnorm!(o, x, weight) (src/inference.jl:102-110). o may alias x. n <= 15360. */
@@ -186,7 +187,10 @@ int l2h_argmax(l2h_ctx *ctx, const float *x, int64_t n, int32_t *out);
 /* Launches the model's matvec for `role` on every layer in turn, `iters` times over,
  * between two HIP events on the context's stream; *avg_us = mean time of one launch,
  * *bytes = weight bytes one launch streams (GGUF block bytes x blocks).  role = L2H_W1
- * times the fused w1+w3 launch, L2H_WQ the fused q/k/v launch. */
+ * times the fused w1+w3 launch, L2H_WQ the fused q/k/v launch.
+ * The launches are the model's own and write where a decode step writes: the call leaves the
+ * RunState (residual stream, position, cache row 0 of every layer) in an undefined state.  Call
+ * l2h_state_reset and feed the prompt again before decoding on. */
 int l2h_profile_matvec(l2h_model *m, int role, int iters, float *avg_us, int64_t *bytes);
 /* plain device-to-device read of n bytes, timed with HIP events: the measured streaming
  * ceiling the roofline fractions can be restated against. */

@@ -48,6 +48,9 @@ static bool is_kquant(int type) {
     return type == L2H_TYPE_Q4_K || type == L2H_TYPE_Q5_K || type == L2H_TYPE_Q6_K;
 }
 static bool type_ok(int type) { return type == L2H_TYPE_F32 || is_kquant(type); }
+// longest input vector of a k-quant matvec: the activation staging of the kernels holds
+// STAGE_MAX_ROUNDS (4) q8_K blocks per wavefront, 16 wavefronts
+#define L2H_MAX_KQ_INPUT 16384
 
 static int64_t align256(int64_t v) { return (v + 255) & ~(int64_t)255; }
 
@@ -359,6 +362,9 @@ extern "C" int l2h_model_set_tensor(l2h_model *m, int role, int layer, int type,
         return set_err(ctx, L2H_ETYPE, "%s must be F32", role_name(role));
     if (is_kquant(type) && ne0 % QK_K != 0)
         return set_err(ctx, L2H_EINVAL, "%s: ne0 = %lld is not a multiple of 256", role_name(role), (long long)ne0);
+    if (is_kquant(type) && ne0 > L2H_MAX_KQ_INPUT)
+        return set_err(ctx, L2H_EINVAL, "%s: a k-quant matrix takes at most %d input features, got %lld", role_name(role),
+                       L2H_MAX_KQ_INPUT, (long long)ne0);
     HIPCHK(ctx, hipSetDevice(ctx->device));
     DevTensor &slot = role < 3 ? m->glob[role] : m->L(layer, role);
     dev_tensor_free(&slot);
@@ -1017,6 +1023,7 @@ static int generate_impl(l2h_model *m, const int32_t *prompt, int n_prompt, int 
     if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
     if (!prompt || n_prompt < 1) return set_err(ctx, L2H_EINVAL, "prompt cannot be empty");  // inference.jl:326-328
     if (n_new < 0 || pos0 < 0) return set_err(ctx, L2H_EINVAL, "negative count");
+    if (n_prompt > m->c.seq_len) return set_err(ctx, L2H_EINVAL, "prompt of %d tokens exceeds seq_len %d", n_prompt, m->c.seq_len);
     const int total = n_prompt - 1 + n_new;
     if (pos0 + total > m->c.seq_len)
         return set_err(ctx, L2H_EINVAL, "pos0 %d + %d steps exceeds seq_len %d", pos0, total, m->c.seq_len);
@@ -1037,17 +1044,20 @@ static int generate_impl(l2h_model *m, const int32_t *prompt, int n_prompt, int 
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     int rc;
     if (decode_ms) {
-        hipEvent_t e0, e1;
+        hipEvent_t e0 = nullptr, e1 = nullptr;
         HIPCHK(ctx, hipEventCreate(&e0));
-        HIPCHK(ctx, hipEventCreate(&e1));
-        if ((rc = run_steps(m, total - n_new))) return rc;
-        HIPCHK(ctx, hipEventRecord(e0, ctx->stream));
-        if ((rc = run_steps(m, n_new))) return rc;
-        HIPCHK(ctx, hipEventRecord(e1, ctx->stream));
-        HIPCHK(ctx, hipEventSynchronize(e1));
-        HIPCHK(ctx, hipEventElapsedTime(decode_ms, e0, e1));
+        hipError_t he = hipEventCreate(&e1);
+        rc = L2H_OK;
+        if (he == hipSuccess) rc = run_steps(m, total - n_new);
+        if (he == hipSuccess && rc == L2H_OK) he = hipEventRecord(e0, ctx->stream);
+        if (he == hipSuccess && rc == L2H_OK) rc = run_steps(m, n_new);
+        if (he == hipSuccess && rc == L2H_OK) he = hipEventRecord(e1, ctx->stream);
+        if (he == hipSuccess && rc == L2H_OK) he = hipEventSynchronize(e1);
+        if (he == hipSuccess && rc == L2H_OK) he = hipEventElapsedTime(decode_ms, e0, e1);
         (void)hipEventDestroy(e0);
-        (void)hipEventDestroy(e1);
+        if (e1) (void)hipEventDestroy(e1);
+        if (rc) return rc;
+        if (he != hipSuccess) return set_err(ctx, L2H_EHIP, "timing the decode steps failed: %s", hipGetErrorString(he));
     } else {
         if ((rc = run_steps(m, total))) return rc;
     }
@@ -1366,6 +1376,9 @@ extern "C" int l2h_matmul(l2h_ctx *ctx, int type, const void *A, int64_t ne0, in
     if (ne0 <= 0 || ne1 < 0) return set_err(ctx, L2H_EINVAL, "bad shape");
     if (is_kquant(type) && ne0 % QK_K != 0)
         return set_err(ctx, L2H_EINVAL, "ne0 = %lld is not a multiple of 256", (long long)ne0);
+    if (is_kquant(type) && ne0 > L2H_MAX_KQ_INPUT)
+        return set_err(ctx, L2H_EINVAL, "a k-quant matrix takes at most %d input features, got %lld", L2H_MAX_KQ_INPUT,
+                       (long long)ne0);
     if ((I_sc == nullptr) != (I_min == nullptr)) return set_err(ctx, L2H_EINVAL, "I_sc and I_min go together");
     if (I_sc && !is_kquant(type)) return set_err(ctx, L2H_EINVAL, "integer sums exist for k-quant types only");
     if (ne1 == 0) return L2H_OK;

@@ -197,8 +197,9 @@ class LanguageModel:  # src/inference.jl:50-54
         self._device = None
 
     def device(self, ctx=None, path=0):
-        """Upload once; later calls reuse the resident copy.  path: see l2h_model_set_path."""
-        if self._device is None:
+        """Upload once; later calls reuse the resident copy (a closed one is replaced).  path: see
+        l2h_model_set_path; it takes effect when the copy is made."""
+        if self._device is None or not self._device.handle:
             self._device = DeviceModel(self.config, self.weights, ctx, path)
         return self._device
 

@@ -310,6 +310,32 @@ def test_generate_argument_checks(pkg):
     with pytest.raises(pkg.L2HError):  # token outside the vocabulary
         dev.generate_greedy([lm.config.vocab_size], 1)
     dev.generate_greedy([1, 2, 3], lm.config.seq_len - 2)  # exactly fills the cache
+    with pytest.raises(pkg.L2HError):  # a prompt longer than the cache, nothing to generate
+        dev.generate_greedy(np.ones(lm.config.seq_len + 1, np.int32), 0)
+
+
+def test_kquant_input_length_limit(pkg, ctx):
+    """A k-quant matrix with more than 16384 input features (64 q8_K blocks, what the kernels' activation
+    staging holds) is refused with an error instead of being multiplied wrongly: by l2h_matmul and by
+    l2h_model_set_tensor (w2 of a model whose hidden_dim is 16640)."""
+    from llama2_jl_amd import kquants, synth
+    ne0 = 16384 + 256
+    A = kquants.QuantMatrix(12, np.zeros(2 * (ne0 // 256) * 144, np.uint8), ne0, 2)
+    with pytest.raises(pkg.L2HError):
+        kquants.matmul(A, np.zeros(ne0, np.float32), ctx=ctx)
+    kw = dict(dim=256, hidden_dim=ne0, n_layers=1, n_heads=2, n_kv_heads=2, vocab_size=300, seq_len=16,
+              rope_freq_base=10000.0, rope_is_neox=False)
+    with pytest.raises(pkg.L2HError) as ei:
+        _model(pkg, "PLAN_Q4_K", **kw).device()
+    assert "16384" in str(ei.value)
+    # the longest length that is taken: exact integer sums against numpy
+    ne0 = 16384
+    rng = np.random.default_rng(3)
+    W = kquants.quantize_weights(rng.standard_normal((2, ne0)).astype(np.float32) * 0.02, 12)
+    x = rng.standard_normal(ne0).astype(np.float32)
+    y = kquants.matmul(W, x, ctx=ctx)
+    ref = kquants.dequantize(W, ctx=ctx).reshape(2, ne0).astype(np.float64) @ x.astype(np.float64)
+    assert np.max(np.abs(y - ref)) <= 2e-2 * np.max(np.abs(ref))
 
 
 def test_temperature_sampling_on_device(pkg, rng):
