@@ -183,6 +183,16 @@ int l2h_swiglu(l2h_ctx *ctx, float *hb, const float *hb2, int64_t n);
 /* argmax(logits), first maximal index, 0-based (src/inference.jl:360) */
 int l2h_argmax(l2h_ctx *ctx, const float *x, int64_t n, int32_t *out);
 
+/* The same argmax for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  x_dev (n floats) and out_dev (one
+ * int32) are DEVICE pointers owned by the caller; the call allocates nothing, enqueues its two kernels on
+ * the context's stream and returns without waiting (l2h_sync waits).  The kernels' intermediate keys live
+ * in a 2 KiB array inside the library's device image, one copy per GPU, held until the process ends:
+ * calls that overlap on one GPU (two contexts on one device) race on it.  n above
+ * L2H_ARGMAX_NOALLOC_MAX_N is L2H_EINVAL. */
+#define L2H_ARGMAX_NOALLOC_MAX_N ((int64_t)1 << 30)
+int l2h_argmax_noalloc(l2h_ctx *ctx, const float *x_dev, int64_t n, int32_t *out_dev);
+
 /* ---- measurement -------------------------------------------------------------------- */
 /* Launches the model's matvec for `role` on every layer in turn, `iters` times over,
  * between two HIP events on the context's stream; *avg_us = mean time of one launch,

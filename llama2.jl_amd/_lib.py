@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libl2hip.so")
+# L2H_LIB names another build of the same library (e.g. the profiling build libl2hip_tl.so)
+LIB_PATH = os.environ.get("L2H_LIB") or os.path.join(HERE, "libl2hip.so")
 
 # error codes / enums of include/l2h.h
 OK, EINVAL, ETYPE, ESTATE, EHIP, ENOMEM, ENODEV = 0, -1, -2, -3, -4, -5, -6
@@ -69,6 +70,7 @@ SIGNATURES = {
     "l2h_attention": (_I, [_P, _P, _P, _P, _P, _I, _I, _I, _I]),
     "l2h_swiglu": (_I, [_P, _P, _P, _I64]),
     "l2h_argmax": (_I, [_P, _P, _I64, _PI32]),
+    "l2h_argmax_noalloc": (_I, [_P, _P, _I64, _P]),
     "l2h_profile_matvec": (_I, [_P, _I, _I, _PF, C.POINTER(_I64)]),
     "l2h_profile_stream_read": (_I, [_P, _I64, _I, _PF]),
     "l2h_synth_normal": (_I, [C.c_uint64, C.c_uint64, _I64, _I64, _F, _P, _I]),

@@ -153,6 +153,7 @@ extern "C" int l2h_ctx_create(int device, l2h_ctx **out) {
     e = hipSetDevice(device);
     if (e == hipSuccess) e = hipGetDeviceProperties(&ctx->prop, device);
     if (e == hipSuccess) e = hipStreamCreate(&ctx->stream);
+    if (e == hipSuccess) e = k_noalloc_init(device);  // address of this device's copy of the no-allocation scratch array
     if (e != hipSuccess) {
         set_err(nullptr, L2H_EHIP, "context setup failed: %s", hipGetErrorString(e));
         delete ctx;
@@ -1562,6 +1563,18 @@ extern "C" int l2h_argmax(l2h_ctx *ctx, const float *x, int64_t n, int32_t *out)
     HIPCHK(ctx, k_argmax(ctx->stream, dx.as<float>(), n, dp.as<int64_t>(), (DecodeCtl *)dctl.p, dout.as<int32_t>(), 1));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(out, dout.p, 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
+// l2h_argmax on device memory, without a single allocation: the keys of the first stage live in a static device
+// array whose address on this context's device was looked up at l2h_ctx_create.
+extern "C" int l2h_argmax_noalloc(l2h_ctx *ctx, const float *x_dev, int64_t n, int32_t *out_dev) {
+    if (!ctx || !x_dev || !out_dev) return set_err(ctx, L2H_EINVAL, "l2h_argmax_noalloc: NULL argument");
+    if (n <= 0 || n > L2H_ARGMAX_NOALLOC_MAX_N)
+        return set_err(ctx, L2H_EINVAL, "l2h_argmax_noalloc: n = %lld outside 1..%lld", (long long)n,
+                       (long long)L2H_ARGMAX_NOALLOC_MAX_N);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    HIPCHK(ctx, k_argmax_noalloc(ctx->stream, ctx->device, x_dev, n, out_dev));
     return L2H_OK;
 }
 

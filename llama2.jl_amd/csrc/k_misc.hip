@@ -1,5 +1,7 @@
 // Small per-token kernels: weight repack, embedding lookup, rmsnorm + q8_K quantize,
 // SwiGLU + quantize, RoPE + KV append, argmax, layout helpers.
+#include <mutex>
+
 #include "dev_common.h"
 
 // ------------------------------------------------------------------------------------------
@@ -257,6 +259,56 @@ hipError_t k_argmax(hipStream_t s, const float *x, int64_t n, int64_t *partial, 
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(argmax_stage2_kernel, dim3(1), dim3(256), 0, s, (const unsigned long long *)partial,
                        L2H_ARGMAX_BLOCKS, ctl, out_tokens, max_out);
+    return hipGetLastError();
+}
+
+// ------------------------------------------------------------------------------------------
+// argmax for callers that cannot allocate (code under stream capture, serving loops, harnesses that forbid
+// hipMalloc): the same two stages, with the per-workgroup keys of stage 1 in a file-scope device array
+// instead of an allocation.  Every GPU the library runs on holds its own copy of the array (2 KiB) until
+// the process ends; calls that overlap on one GPU would share it and race.
+// ------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned long long scratch[L2H_ARGMAX_BLOCKS];
+
+// In host code `scratch` is a stand-in, not a device address: each device's address is asked for once, with
+// that device current, and kept.
+#define L2H_MAX_DEVICES 64
+static unsigned long long *g_scratch_ptr[L2H_MAX_DEVICES];
+
+static std::mutex g_scratch_mu;
+
+hipError_t k_noalloc_init(int device) {
+    if (device < 0 || device >= L2H_MAX_DEVICES) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (g_scratch_ptr[device]) return hipSuccess;
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return e;
+    if (!p) return hipErrorInvalidSymbol;
+    g_scratch_ptr[device] = (unsigned long long *)p;
+    return hipSuccess;
+}
+
+__global__ __launch_bounds__(256) void argmax_stage2_plain_kernel(const unsigned long long *partial, int nparts,
+                                                                  int32_t *out) {
+    __shared__ unsigned long long red[4];
+    unsigned long long best = 0;
+    for (int i = threadIdx.x; i < nparts; i += blockDim.x) best = partial[i] > best ? partial[i] : best;
+    best = block_max_u64(best, red);
+    if (threadIdx.x == 0) *out = (int32_t)(0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFull));
+}
+
+// x and out are device pointers; nothing is allocated, nothing is waited for.  Stage 1 writes every one of
+// the L2H_ARGMAX_BLOCKS keys on every call (a workgroup without elements writes the smallest key), so what
+// the previous call left in the array is never read.
+hipError_t k_argmax_noalloc(hipStream_t s, int device, const float *x, int64_t n, int32_t *out) {
+    if (device < 0 || device >= L2H_MAX_DEVICES || !g_scratch_ptr[device]) return hipErrorNotInitialized;
+    unsigned long long *partial = g_scratch_ptr[device];
+    hipLaunchKernelGGL(argmax_stage1_kernel, dim3(L2H_ARGMAX_BLOCKS), dim3(256), 0, s, x, n, partial);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    hipLaunchKernelGGL(argmax_stage2_plain_kernel, dim3(1), dim3(256), 0, s, (const unsigned long long *)partial,
+                       L2H_ARGMAX_BLOCKS, out);
     return hipGetLastError();
 }
 

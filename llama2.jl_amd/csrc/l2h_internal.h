@@ -198,6 +198,9 @@ hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const flo
 hipError_t k_softmax(hipStream_t s, float *x, int64_t n);
 hipError_t k_argmax(hipStream_t s, const float *x, int64_t n, int64_t *partial, DecodeCtl *ctl, int32_t *out_tokens,
                     int max_out);
+// argmax without allocations: k_noalloc_init once per device (that device current), then k_argmax_noalloc
+hipError_t k_noalloc_init(int device);
+hipError_t k_argmax_noalloc(hipStream_t s, int device, const float *x_dev, int64_t n, int32_t *out_dev);
 hipError_t k_sample(hipStream_t s, const float *logits, int n, float temperature, float u, float *p, int32_t *out);
 hipError_t k_kv_layout(hipStream_t s, float *kc, float *vc, float *k_lin, float *v_lin, int pos0, int n, int head_size,
                        int n_kv_heads, int seq_len, bool to_cache);
