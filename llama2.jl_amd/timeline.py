@@ -1,0 +1,75 @@
+"""Where the time of one token goes inside the streaming decode kernel (launch path 3).
+
+    python llama2.jl_amd/build.py --timeline          # builds llama2.jl_amd/libl2hip_tl.so (-DL2H_TIMELINE)
+    python llama2.jl_amd/timeline.py [n_layers]       # on the GPU; prints the table
+
+In the profiling build thread 0 of every workgroup stamps the 100 MHz wall clock at the phase boundaries
+of the first layers of a launch (after staging a phase's input, after the wait for the ring's pieces, at
+the end of its own streaming loop, when the whole workgroup has finished it, after the epilogue).  The
+script decodes a few tokens of a model with the benchmark's widths, reads the stamps of the last launch
+and prints, per boundary, the minimum / median / maximum over the workgroups, the step from the previous
+boundary (median), and a one-line summary of a steady-state layer.  Numbers are microseconds since the
+first workgroup started."""
+import ctypes
+import importlib.util
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+PHASES = ("qkv", "wo", "w13", "w2")
+STAMPS = ("staged", "drained", "looped", "alldone", "fin")
+
+
+def main():
+    os.environ.setdefault("L2H_LIB", os.path.join(HERE, "libl2hip_tl.so"))
+    spec = importlib.util.spec_from_file_location("llama2_jl_amd", os.path.join(HERE, "__init__.py"),
+                                                  submodule_search_locations=[HERE])
+    pkg = importlib.util.module_from_spec(spec)
+    sys.modules["llama2_jl_amd"] = pkg
+    spec.loader.exec_module(pkg)
+    from llama2_jl_amd import _lib, synth
+    n_layers = int(sys.argv[1]) if len(sys.argv) > 1 else 4
+    cfg = pkg.ModelConfig(dim=4096, hidden_dim=14336, n_layers=n_layers, n_heads=32, n_kv_heads=8, vocab_size=128256,
+                          seq_len=512, rope_freq_base=500000.0)
+    lm = synth.synthetic_model(cfg, synth.PLAN_Q4_K_S, seed=1)
+    dev = lm.device(path=3)
+    dev.generate_greedy(synth.seeded_prompt(1, 32, cfg.vocab_size), 8)
+    lib = _lib.lib()
+    if not hasattr(lib, "l2h_debug_timeline"):
+        sys.exit("this library was built without -DL2H_TIMELINE: python llama2.jl_amd/build.py --timeline")
+    lib.l2h_debug_timeline.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int]
+    n_wg = dev.ctx.device_info()["n_cu"] if isinstance(dev.ctx.device_info(), dict) else 256
+    buf = np.zeros(n_wg * 64 + 1024, np.int64)
+    assert lib.l2h_debug_timeline(dev.handle, buf.ctypes.data_as(ctypes.c_void_p), n_wg) == 0
+    tl = buf[:n_wg * 64].reshape(n_wg, 64)
+    us = (tl - tl[:, 0].min()) * 0.01
+    # the workgroups that run a head's attention have one more stamp per layer than the others
+    stride = n_wg // cfg.n_heads
+    att = np.array([(w // stride < cfg.n_heads) and (w % stride == (w // stride) % stride) for w in range(n_wg)])
+    names = ["start"]
+    for l in range(3):
+        for ph in PHASES:
+            if ph == "wo":
+                names.append("att done l%d" % l)
+            names += ["%s %s l%d" % (ph, st, l) for st in STAMPS]
+    prev = None
+    for i, nm in enumerate(names[:60]):
+        col = us[~att, i]
+        med = float(np.median(col))
+        print("%-18s min %7.2f  med %7.2f  max %7.2f  step %5.2f | attention workgroups: med %7.2f"
+              % (nm, col.min(), med, col.max(), med - prev if prev is not None else 0.0, float(np.median(us[att, i]))))
+        prev = med
+    med = np.median(us[~att], axis=0)
+    per = len(PHASES) * len(STAMPS) + 1
+    i0 = 1 + per  # layer 1: steady state
+    if n_layers >= 3:
+        d = np.diff(med[i0 - 1:i0 + per])
+        print("layer 1: %.2f us = " % (med[i0 + per - 1] - med[i0 - 1]) +
+              " ".join("%s:%.2f" % (names[i0 + k].rsplit(" ", 1)[0].replace(" ", "/"), d[k]) for k in range(per)))
+    dev.close()
+
+
+if __name__ == "__main__":
+    main()
