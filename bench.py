@@ -74,6 +74,8 @@ def main():
     ap.add_argument("--repeats", type=int, default=3, help="timed regions; the median is reported")
     ap.add_argument("--path", type=int, default=0, help="0 auto, 1 kernel per phase, 2 persistent kernel, 3 streaming kernel")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 = skip)")
+    ap.add_argument("--kv", default="fp32", choices=["fp32", "fp16"],
+                    help="element type of the KV cache: fp32 as the reference's, or the fp16 option (launch path 1)")
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on exactly one GPU (batch-1 decode of one sequence is not sharded here); "
@@ -97,7 +99,7 @@ def main():
                                share_classifier=(plan_name == "PLAN_F32"))
     log("model generated + quantized on %d host threads in %.1f s" % (synth._threads(), time.time() - t0))
     t0 = time.time()
-    dev = lm.device(path=args.path)
+    dev = lm.device(path=args.path, kv_fp16=(args.kv == "fp16"))
     ctx.sync()
     log("uploaded in %.1f s; launch path %d (1 = kernel per phase, 2 = persistent kernel, 3 = streaming kernel)" % (time.time() - t0, dev.path))
 
@@ -164,12 +166,19 @@ def main():
     dt = float(np.median(times))
     tok_s = K / dt
     # positions read by the timed steps: pos0 .. pos0+K-1, each reads pos+1 cache rows
-    kv_bytes = 2 * cfg.n_layers * kv_dim * 4 * (pos0 + 1 + (K - 1) / 2.0)
+    kv_bytes = 2 * cfg.n_layers * kv_dim * (2 if args.kv == "fp16" else 4) * (pos0 + 1 + (K - 1) / 2.0)
     bytes_per_token = w_bytes + kv_bytes
     roofline_tok_s = HBM_PEAK_GBS * 1e9 / bytes_per_token
 
-    # ---- dominant kernel: the k-quant (or fp32) matvec, timed with HIP events on the library's
-    # stream, every layer's tensor in turn so that nothing is cache-resident ----------------------
+    # ---- dominant kernel -----------------------------------------------------------------------------
+    # launch path 3: one launch per token does everything; its duration comes from HIP events around K launches on
+    # the library's stream (taken first: the per-phase timing below overwrites the decode state), its algorithmic
+    # bytes are the token's
+    ev_ms = None
+    if dev.path == 3:
+        _, ev_ms = dev.generate_greedy([first], K, pos0=pos0, timed=True)
+    # the k-quant (or fp32) matvec of every phase, timed with HIP events on the library's stream, every layer's
+    # tensor in turn so that nothing is cache-resident
     roles = [("qkv", _lib.WQ), ("wo", _lib.WO), ("w1w3", _lib.W1), ("w2", _lib.W2), ("output", _lib.OUTPUT)]
     per_kernel, tot_us, tot_b, n_launch = {}, 0.0, 0, 0
     dominant_type = lm.weights.layers[0].w1.type if hasattr(lm.weights.layers[0].w1, "type") else 0
@@ -187,9 +196,6 @@ def main():
     kernel_name = "matvec_kq_kernel (k-quant x q8_K dequant-matvec)"
     bytes_per_launch, launches, avg_launch_us = int(tot_b / max(1, n_launch)), n_launch, tot_us / max(1, n_launch)
     if dev.path == 3:
-        # the streaming kernel: one launch per token does everything; its duration comes from HIP events
-        # around the K launches on the library's stream, its algorithmic bytes are the token's
-        _, ev_ms = dev.generate_greedy([first], K, pos0=pos0, timed=True)
         kernel_name = "flow_token_kernel (whole token: q4_K/q6_K x q8_K matvecs, attention, argmax)"
         bytes_per_launch, launches, avg_launch_us = int(bytes_per_token), 1, ev_ms * 1e3 / K
         achieved = bytes_per_launch / avg_launch_us / 1e3
@@ -233,6 +239,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "shape": kw, "plan": plan_name, "prompt_tokens": n_prompt,
                    "decode_positions": [pos0, pos0 + K - 1], "repeats": args.repeats, "launch_path": dev.path,
+                   "kv_cache": args.kv,
                    "bytes_per_token": int(bytes_per_token), "weight_bytes_per_token": int(w_bytes),
                    "roofline_tok_s_at_8TBs": round(roofline_tok_s, 1),
                    "frac_of_roofline": round(tok_s / roofline_tok_s, 4),

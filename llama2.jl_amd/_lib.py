@@ -46,6 +46,7 @@ SIGNATURES = {
     "l2h_model_destroy": (None, [_P]),
     "l2h_model_set_tensor": (_I, [_P, _I, _I, _I, _P, _I64, _I64]),
     "l2h_model_get_tensor": (_I, [_P, _I, _I, _P, _I64]),
+    "l2h_model_set_kv_type": (_I, [_P, _I]),
     "l2h_model_set_path": (_I, [_P, _I]),
     "l2h_model_set_wait_limit": (_I, [_P, C.c_uint]),
     "l2h_model_set_prefill_copy": (_I, [_P, _I]),

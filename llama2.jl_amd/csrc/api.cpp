@@ -224,6 +224,7 @@ struct l2h_model {
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     // persistent decode kernel
+    int kv16 = 0;          // 1: the KV cache holds fp16 elements (l2h_model_set_kv_type)
     int path_request = 0;  // 0 auto, 1 one kernel per phase, 2 persistent kernel, 3 streaming kernel (2, 3: required)
     bool mega = false;
     PhaseArgs mega_ph[5];  // q/k/v, wo, w1+w3, w2 of layer 0 and the classifier, planned for the persistent grid
@@ -391,6 +392,14 @@ extern "C" int l2h_model_set_prefill_copy(l2h_model *m, int on) {
     return L2H_OK;
 }
 
+extern "C" int l2h_model_set_kv_type(l2h_model *m, int kv_type) {
+    if (!m) return L2H_EINVAL;
+    if (m->finalized) return set_err(m->ctx, L2H_ESTATE, "model already finalized");
+    if (kv_type != L2H_KV_F32 && kv_type != L2H_KV_F16) return set_err(m->ctx, L2H_EINVAL, "kv_type must be L2H_KV_F32 or L2H_KV_F16");
+    m->kv16 = kv_type == L2H_KV_F16;
+    return L2H_OK;
+}
+
 extern "C" int l2h_model_set_path(l2h_model *m, int path) {
     if (!m) return L2H_EINVAL;
     if (m->finalized) return set_err(m->ctx, L2H_ESTATE, "model already finalized");
@@ -465,6 +474,10 @@ static int dalloc(l2h_model *m, T **p, int64_t n, bool zero) {
     return L2H_OK;
 }
 
+// the caches of layer l (fp32 or fp16 elements: addressed in bytes)
+static float *layer_kc(l2h_model *m, int l) { return (float *)((char *)m->kc + (int64_t)l * m->cache_layer_elems * (m->kv16 ? 2 : 4)); }
+static float *layer_vc(l2h_model *m, int l) { return (float *)((char *)m->vc + (int64_t)l * m->cache_layer_elems * (m->kv16 ? 2 : 4)); }
+
 // ---- the per-token launch sequence: transformer! (reference src/inference.jl:222-315) ----------
 static PhaseArgs base_args(l2h_model *m) {
     PhaseArgs a{};
@@ -476,7 +489,8 @@ static PhaseArgs base_args(l2h_model *m) {
     a.rope_cs = m->rope_cs;
     a.qd = m->qd;
     a.normw_stride = m->L(0, L2H_RMS_ATT).layer_stride;
-    a.cache_stride = m->cache_layer_elems * 4;
+    a.cache_stride = m->cache_layer_elems * (m->kv16 ? 2 : 4);
+    a.kv16 = m->kv16;
     return a;
 }
 
@@ -488,8 +502,8 @@ static PhaseArgs make_qkv(l2h_model *m, int l, int first, int last) {
     PhaseArgs a = base_args(m);
     a.xf = m->x;
     a.normw = m->L(l, L2H_RMS_ATT).f32;
-    a.kc = m->kc + (int64_t)l * m->cache_layer_elems;
-    a.vc = m->vc + (int64_t)l * m->cache_layer_elems;
+    a.kc = layer_kc(m, l);
+    a.vc = layer_vc(m, l);
     a.nseg = last - first;
     a.seg_roles = 0;
     for (int k = first; k < last; k++) {
@@ -847,15 +861,15 @@ static hipError_t enqueue_token(l2h_model *m) {
     // token embedding (:236) and this position's RoPE table
     CK(k_embed(s, m->glob[L2H_TOK_EMB], m->ctl, m->prompt_dev, m->x, m->rope_cs, m->hs, m->theta_scale));
     for (int l = 0; l < c.n_layers; l++) {
-        float *kc = m->kc + (int64_t)l * m->cache_layer_elems;
-        float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
+        float *kc = layer_kc(m, l), *vc = layer_vc(m, l);
         CK(launch_qkv(m, l));
         // attention (:263-278) -> xb: one launch while the sequence fits one workgroup's LDS, else split over time
-        if (c.seq_len <= 1024)
+        // (an fp16 cache is read by the split kernels only)
+        if (c.seq_len <= 1024 && !m->kv16)
             CK(k_attention_fused(s, m->q, m->xb, kc, vc, m->ctl, m->hs, c.n_heads, c.n_kv_heads, c.seq_len));
         else
             CK(k_attention(s, m->qd, kc, vc, m->att, m->pd, m->part, m->xb, m->ctl, m->hs, c.n_heads, c.n_kv_heads,
-                           c.seq_len));
+                           c.seq_len, m->kv16));
         CK(launch_wo(m, l));
         CK(launch_w13(m, l));
         CK(launch_w2(m, l));
@@ -898,8 +912,16 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     const int ntiles = (c.seq_len + L2H_ATT_TILE - 1) / L2H_ATT_TILE;
     DA(m->part, (int64_t)ntiles * c.dim, true);
     m->cache_layer_elems = (int64_t)c.seq_len * m->kv_dim;
-    DA(m->kc, m->cache_layer_elems * c.n_layers, true);
-    DA(m->vc, m->cache_layer_elems * c.n_layers, true);
+    if (m->kv16) {
+        if (m->hs > 128 || m->hs % 16 != 0)
+            return set_err(ctx, L2H_EINVAL, "an fp16 KV cache needs a head size that is a multiple of 16, at most 128");
+        if (m->path_request == 2 || m->path_request == 3)
+            return set_err(ctx, L2H_EINVAL, "an fp16 KV cache runs on launch path 1 only");
+        m->path_request = 1;
+    }
+    // (an fp16 cache takes half the floats)
+    DA(m->kc, m->cache_layer_elems * c.n_layers / (m->kv16 ? 2 : 1) + 1, true);
+    DA(m->vc, m->cache_layer_elems * c.n_layers / (m->kv16 ? 2 : 1) + 1, true);
     DA(m->ctl, 1, true);
     DA(m->prompt_dev, c.seq_len, true);
     m->max_out = c.seq_len;
@@ -974,7 +996,7 @@ static int mega_check(l2h_model *m) {
 extern "C" int l2h_state_reset(l2h_model *m) {
     if (!m) return L2H_EINVAL;
     if (!m->finalized) return set_err(m->ctx, L2H_ESTATE, "model not finalized");
-    const size_t bytes = (size_t)m->cache_layer_elems * m->c.n_layers * 4;
+    const size_t bytes = (size_t)m->cache_layer_elems * m->c.n_layers * (m->kv16 ? 2 : 4);
     HIPCHK(m->ctx, hipMemsetAsync(m->kc, 0, bytes, m->ctx->stream));
     HIPCHK(m->ctx, hipMemsetAsync(m->vc, 0, bytes, m->ctx->stream));
     HIPCHK(m->ctx, hipStreamSynchronize(m->ctx->stream));
@@ -997,8 +1019,8 @@ static int kv_xfer(l2h_model *m, int layer, int pos0, int n, float *k, float *v,
         if (e == hipSuccess) e = hipMemcpy(dv, v, bytes, hipMemcpyHostToDevice);
     }
     if (e == hipSuccess)
-        e = k_kv_layout(ctx->stream, m->kc + layer * m->cache_layer_elems, m->vc + layer * m->cache_layer_elems, dk, dv,
-                        pos0, n, m->hs, m->c.n_kv_heads, m->c.seq_len, to_cache);
+        e = k_kv_layout(ctx->stream, layer_kc(m, layer), layer_vc(m, layer), dk, dv, pos0, n, m->hs, m->c.n_kv_heads,
+                        m->c.seq_len, to_cache, m->kv16);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
     if (e == hipSuccess && !to_cache) {
         e = hipMemcpy(k, dk, bytes, hipMemcpyDeviceToHost);
@@ -1198,6 +1220,7 @@ extern "C" int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0,
     for (int i = 0; i < n; i++)
         if (tokens[i] < 0 || tokens[i] >= m->c.vocab_size)
             return set_err(ctx, L2H_EINVAL, "tokens[%d] = %d outside vocabulary", i, tokens[i]);
+    if (m->kv16) return set_err(ctx, L2H_ESTATE, "the batched prompt pass writes an fp32 cache only (this model's is fp16)");
     if (!k_pf_attention_supported(m->hs))
         return set_err(ctx, L2H_EINVAL, "batched prompt pass needs a head size of 32, 64, 96 or 128 (have %d)", m->hs);
     if (m->c.dim % 8 != 0 || m->c.hidden_dim % 8 != 0)
@@ -1523,10 +1546,10 @@ extern "C" int l2h_attention(l2h_ctx *ctx, float *out, const float *q, const flo
     HIPCHK(ctx, hipMemcpy(dvl.p, vc, (size_t)np * kv_dim * 4, hipMemcpyHostToDevice));
     HIPCHK(ctx, k_f32_to_f64(ctx->stream, dq.as<float>(), dqd.as<double>(), dim));
     HIPCHK(ctx, k_kv_layout(ctx->stream, dkc.as<float>(), dvc.as<float>(), dkl.as<float>(), dvl.as<float>(), 0, np,
-                            head_size, n_kv_heads, seq_len, true));
+                            head_size, n_kv_heads, seq_len, true, 0));
     HIPCHK(ctx, k_attention(ctx->stream, dqd.as<double>(), dkc.as<float>(), dvc.as<float>(), datt.as<float>(),
                             dpd.as<double>(), dpart.as<double>(), dout.as<float>(), (const DecodeCtl *)dctl.p,
-                            head_size, n_heads, n_kv_heads, seq_len));
+                            head_size, n_heads, n_kv_heads, seq_len, 0));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     HIPCHK(ctx, hipMemcpy(out, dout.p, (size_t)dim * 4, hipMemcpyDeviceToHost));
     return L2H_OK;

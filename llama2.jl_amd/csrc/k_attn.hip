@@ -111,7 +111,7 @@ __global__ __launch_bounds__(256) void attn_reduce_kernel(const double *part, fl
 // Scores: a workgroup = 64 timesteps of GH heads that share a KV head; wavefront w takes quarter w
 // of the head dimension (all of its 16-byte loads in flight at once), the quarters are added in
 // fixed order through LDS.
-template <int GH>
+template <int GH, bool H16>
 __global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, const float *kc, float *att, float *tmax,
                                                            const DecodeCtl *ctl, int hs, int n_heads, int n_kv_heads,
                                                            int seq_len) {
@@ -125,11 +125,11 @@ __global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, con
     for (int i = threadIdx.x; i < GH * hs; i += 256) s_q[(i / hs) * 128 + i % hs] = qd[(int64_t)h0 * hs + i];
     const int per = hs >> 4;  // 16-byte groups per quarter (hs <= 128: at most 8)
     const int t = min(t0 + lane, pos);
-    const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
+    const int64_t kg = ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;  // group of four elements
     float4 kv[8];
 #pragma unroll
     for (int u = 0; u < 8; u++)
-        if (u < per) kv[u] = ldg_nt_f4(kp + (int64_t)u * seq_len);
+        if (u < per) kv[u] = ldg_nt_kv4<H16>(kc, kg + (int64_t)u * seq_len);
     __syncthreads();
     double acc[GH];
 #pragma unroll
@@ -194,7 +194,7 @@ __global__ __launch_bounds__(256) void attn_exp_kernel(float *att, const float *
 // (16-byte group of the head dimension, timestep group), eight loads in flight per round; the
 // probabilities p = e / total are formed here (fp32 division, as softmax! does), widened to fp64; fp64
 // partial sums per workgroup go to `part`, which attn_reduce4_kernel adds in block order.
-template <int GH>
+template <int GH, bool H16>
 __global__ __launch_bounds__(256) void attn_av4_kernel(const float *att, const double *psum, int npsum, const float *vc,
                                                        double *part, const DecodeCtl *ctl, int hs, int n_heads,
                                                        int n_kv_heads, int seq_len, int chunk) {
@@ -230,12 +230,12 @@ __global__ __launch_bounds__(256) void attn_av4_kernel(const float *att, const d
         }
         float4 v[8];
         if (active) {
-            const float4 *vp = (const float4 *)(vc + ((int64_t)kvh * seq_len + t0) * hs) + i4;
+            const int64_t vg = ((int64_t)kvh * seq_len + t0) * n4 + i4;  // group of four elements
 #pragma unroll
             for (int u = 0; u < 8; u++) {
                 const int l = tg + ngrp * u;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (l < nt) v[u] = ldg_nt_f4(vp + (int64_t)l * n4);
+                if (l < nt) v[u] = ldg_nt_kv4<H16>(vc, vg + (int64_t)l * n4);
             }
         }
         __syncthreads();
@@ -310,7 +310,7 @@ hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const flo
     return hipGetLastError();
 }
 
-template <int GH>
+template <int GH, bool H16>
 static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att,
                               double *pd, double *part, float *out, const DecodeCtl *ctl, int hs,
                               int n_heads, int n_kv_heads, int seq_len) {
@@ -320,7 +320,7 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
         const int npsum = (seq_len + 1023) / 1024;
         double *psum = pd;
         float *tmax = (float *)(pd + (int64_t)n_heads * npsum);
-        hipLaunchKernelGGL((attn_scores4_kernel<GH>), dim3(ntiles, n_heads / GH), dim3(256), 0, s, qd, kc, att, tmax, ctl,
+        hipLaunchKernelGGL((attn_scores4_kernel<GH, H16>), dim3(ntiles, n_heads / GH), dim3(256), 0, s, qd, kc, att, tmax, ctl,
                            hs, n_heads, n_kv_heads, seq_len);
         hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -330,7 +330,7 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
         // timesteps per value workgroup: as large as still leaves L2H_AV_MIN_WGS workgroups over a full cache
         int chunk = 64;
         while (chunk < 512 && (int64_t)(seq_len / (2 * chunk)) * (n_heads / GH) >= L2H_AV_MIN_WGS) chunk *= 2;
-        hipLaunchKernelGGL((attn_av4_kernel<GH>), dim3((seq_len + chunk - 1) / chunk, n_heads / GH), dim3(256), 0, s, att,
+        hipLaunchKernelGGL((attn_av4_kernel<GH, H16>), dim3((seq_len + chunk - 1) / chunk, n_heads / GH), dim3(256), 0, s, att,
                            psum, npsum, vc, part, ctl, hs, n_heads, n_kv_heads, seq_len, chunk);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -338,6 +338,7 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
         hipLaunchKernelGGL(attn_reduce4_kernel, dim3((dim + 63) / 64), dim3(256), 0, s, part, out, ctl, dim, chunk);
         return hipGetLastError();
     }
+    if (H16) return hipErrorInvalidValue;  // (the general kernels below read fp32 caches only)
     hipLaunchKernelGGL((attn_scores_kernel<GH>), dim3((ntiles + 3) / 4, n_heads / GH), dim3(256), 0, s, qd, kc, att,
                        ctl, hs, n_heads, n_kv_heads, seq_len);
     hipError_t e = hipGetLastError();
@@ -356,9 +357,13 @@ static hipError_t launch_attn(hipStream_t s, const double *qd, const float *kc, 
 
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
                        double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads,
-                       int n_kv_heads, int seq_len) {
+                       int n_kv_heads, int seq_len, int kv16) {
     const int G = n_heads / n_kv_heads;
-    if (G % 4 == 0) return launch_attn<4>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    if (G % 2 == 0) return launch_attn<2>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
-    return launch_attn<1>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len);
+#define GO(GH_)                                                                                                          \
+    return kv16 ? launch_attn<GH_, true>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len) \
+                : launch_attn<GH_, false>(s, qd, kc, vc, att, pd, part, out, ctl, head_size, n_heads, n_kv_heads, seq_len)
+    if (G % 4 == 0) GO(4);
+    if (G % 2 == 0) GO(2);
+    GO(1);
+#undef GO
 }

@@ -1,5 +1,6 @@
 // Small per-token kernels: weight repack, embedding lookup, rmsnorm + q8_K quantize,
 // SwiGLU + quantize, RoPE + KV append, argmax, layout helpers.
+#include <hip/hip_fp16.h>
 #include <mutex>
 
 #include "dev_common.h"
@@ -171,7 +172,7 @@ hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int 
 
 // canonical [n][kv_dim] rows <-> cache layouts, positions pos0 .. pos0+n-1 of one layer
 __global__ __launch_bounds__(256) void kv_layout_kernel(float *kc, float *vc, float *k_lin, float *v_lin, int pos0,
-                                                        int n, int hs, int n_kv_heads, int seq_len, int to_cache) {
+                                                        int n, int hs, int n_kv_heads, int seq_len, int to_cache, int kv16) {
     const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int kv_dim = hs * n_kv_heads;
     if (gid >= (int64_t)n * kv_dim) return;
@@ -179,6 +180,17 @@ __global__ __launch_bounds__(256) void kv_layout_kernel(float *kc, float *vc, fl
     const int h = e / hs, i = e % hs, t = pos0 + r;
     const int64_t ki = kc_index(h, i, t, hs, seq_len);
     const int64_t vi = ((int64_t)h * seq_len + t) * hs + i;
+    if (kv16) {  // fp16 cache: rounded to nearest even on the way in, widened exactly on the way out
+        __half *kh = (__half *)kc, *vh = (__half *)vc;
+        if (to_cache) {
+            kh[ki] = __float2half_rn(k_lin[gid]);
+            vh[vi] = __float2half_rn(v_lin[gid]);
+        } else {
+            k_lin[gid] = __half2float(kh[ki]);
+            v_lin[gid] = __half2float(vh[vi]);
+        }
+        return;
+    }
     if (to_cache) {
         kc[ki] = k_lin[gid];
         vc[vi] = v_lin[gid];
@@ -189,10 +201,10 @@ __global__ __launch_bounds__(256) void kv_layout_kernel(float *kc, float *vc, fl
 }
 
 hipError_t k_kv_layout(hipStream_t s, float *kc, float *vc, float *k_lin, float *v_lin, int pos0, int n, int head_size,
-                       int n_kv_heads, int seq_len, bool to_cache) {
+                       int n_kv_heads, int seq_len, bool to_cache, int kv16) {
     const int64_t total = (int64_t)n * head_size * n_kv_heads;
     hipLaunchKernelGGL(kv_layout_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, kc, vc, k_lin, v_lin,
-                       pos0, n, head_size, n_kv_heads, seq_len, to_cache ? 1 : 0);
+                       pos0, n, head_size, n_kv_heads, seq_len, to_cache ? 1 : 0, kv16);
     return hipGetLastError();
 }
 

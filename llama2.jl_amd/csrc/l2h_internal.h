@@ -88,6 +88,7 @@ struct PhaseArgs {
     float *kc, *vc;        // this layer's caches
     const DecodeCtl *ctl;
     int hs, seq_len, neox;
+    int kv16;              // the caches hold fp16 elements (kc, vc are then byte addresses of such arrays)
     // debug: per (row, block) integer sums (EPI_STORE only), or nullptr
     int32_t *dbg_isc, *dbg_imin;
     int64_t dbg_row0[3];
@@ -189,9 +190,10 @@ hipError_t k_mega_launch(hipStream_t s, const MegaArgs &g, int t_qkv, int t_wo, 
                          size_t lds);
 hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64_t n, int pro, Q8Dev q8_out, float *f32_out);
 hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
+// kv16: the caches hold fp16 elements (needs head_size <= 128, a multiple of 16)
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
                        double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads,
-                       int n_kv_heads, int seq_len);
+                       int n_kv_heads, int seq_len, int kv16);
 // one launch for scores + softmax + values; needs head_size*8 + seq_len*12 + 8 KiB of LDS <= 64 KiB
 hipError_t k_attention_fused(hipStream_t s, const float *q, float *xb, const float *kc, const float *vc,
                              const DecodeCtl *ctl, int head_size, int n_heads, int n_kv_heads, int seq_len);
@@ -203,7 +205,7 @@ hipError_t k_noalloc_init(int device);
 hipError_t k_argmax_noalloc(hipStream_t s, int device, const float *x_dev, int64_t n, int32_t *out_dev);
 hipError_t k_sample(hipStream_t s, const float *logits, int n, float temperature, float u, float *p, int32_t *out);
 hipError_t k_kv_layout(hipStream_t s, float *kc, float *vc, float *k_lin, float *v_lin, int pos0, int n, int head_size,
-                       int n_kv_heads, int seq_len, bool to_cache);
+                       int n_kv_heads, int seq_len, bool to_cache, int kv16);
 hipError_t k_stream_read(hipStream_t s, const uint4 *p, int64_t n16, uint32_t *sink);
 hipError_t k_f32_to_f64(hipStream_t s, const float *x, double *y, int64_t n);
 

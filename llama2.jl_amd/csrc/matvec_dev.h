@@ -1,6 +1,8 @@
 // Device code of the k-quant / fp32 matvec phases, shared by the per-phase kernels and the
 // persistent decode kernel.
 #pragma once
+#include <hip/hip_fp16.h>
+
 #include "dev_common.h"
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -14,6 +16,23 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ float4 ldg_nt_f4(const float4 *p) {
     const f32x4v t = __builtin_nontemporal_load((const f32x4v *)p);
     return make_float4(t.x, t.y, t.z, t.w);
+}
+// The KV cache holds fp32 (the reference's, src/inference.jl:62-65) or, as an option, fp16 elements in the
+// same index layout.  Group g of four consecutive elements, widened to fp32 (exact):
+template <bool H16>
+__device__ __forceinline__ float4 ldg_nt_kv4(const void *base, int64_t g) {
+    if (!H16) return ldg_nt_f4((const float4 *)base + g);
+    typedef unsigned int u32x2v __attribute__((ext_vector_type(2)));
+    const u32x2v t = __builtin_nontemporal_load((const u32x2v *)base + g);
+    return make_float4(half_bits_to_float((uint16_t)(t.x & 0xFFFF)), half_bits_to_float((uint16_t)(t.x >> 16)),
+                       half_bits_to_float((uint16_t)(t.y & 0xFFFF)), half_bits_to_float((uint16_t)(t.y >> 16)));
+}
+// element i of a cache <- v (fp16: rounded to nearest even)
+__device__ __forceinline__ void st_kv(void *base, int64_t i, float v, bool h16) {
+    if (h16)
+        ((__half *)base)[i] = __float2half_rn(v);
+    else
+        ((float *)base)[i] = v;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -572,7 +591,10 @@ __device__ __forceinline__ void finish_row(const PhaseArgs &a, int layer, int64_
         const int pos = a.ctl->pos;
         const int h = (int)(rr.row / a.hs), e = (int)(rr.row % a.hs);
         if (role == SEG_V) {
-            st_f32<COH>(at_layer(a.vc, a.cache_stride, layer) + ((int64_t)h * a.seq_len + pos) * a.hs + e, val);
+            if (a.kv16)
+                st_kv(at_layer(a.vc, a.cache_stride, layer), ((int64_t)h * a.seq_len + pos) * a.hs + e, val, true);
+            else
+                st_f32<COH>(at_layer(a.vc, a.cache_stride, layer) + ((int64_t)h * a.seq_len + pos) * a.hs + e, val);
             return;
         }
         const int half = a.hs >> 1;
@@ -585,7 +607,11 @@ __device__ __forceinline__ void finish_row(const PhaseArgs &a, int layer, int64_
             st_f32<COH>(a.y[0] + rr.row, out);  // q is always the first segment of its launch
             st_f64<COH>(a.qd + rr.row, (double)out);
         } else {
-            st_f32<COH>(at_layer(a.kc, a.cache_stride, layer) + (((int64_t)h * (a.hs >> 2) + (e >> 2)) * a.seq_len + pos) * 4 + (e & 3), out);
+            const int64_t ki = (((int64_t)h * (a.hs >> 2) + (e >> 2)) * a.seq_len + pos) * 4 + (e & 3);
+            if (a.kv16)
+                st_kv(at_layer(a.kc, a.cache_stride, layer), ki, out, true);
+            else
+                st_f32<COH>(at_layer(a.kc, a.cache_stride, layer) + ki, out);
         }
     }
 }

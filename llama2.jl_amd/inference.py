@@ -64,7 +64,7 @@ _LAYER_ROLES = [("rms_att_weight", _lib.RMS_ATT), ("rms_ffn_weight", _lib.RMS_FF
 class DeviceModel:
     """l2h_model: the weights in HBM plus the RunState (activations, KV cache)."""
 
-    def __init__(self, config, weights, ctx=None, path=0):
+    def __init__(self, config, weights, ctx=None, path=0, kv_fp16=False):
         self.ctx = ctx or _lib.default_context()
         self.config = config
         cfg = _lib.Config(config.dim, config.hidden_dim, config.n_layers, config.n_heads, config.n_kv_heads,
@@ -81,6 +81,8 @@ class DeviceModel:
             for l, lw in enumerate(weights.layers):
                 for name, role in _LAYER_ROLES:
                     self._set(role, l, getattr(lw, name))
+            if kv_fp16:
+                self.ctx.check(_lib.lib().l2h_model_set_kv_type(self.handle, 1))
             self.ctx.check(_lib.lib().l2h_model_set_path(self.handle, path))
             self.ctx.check(_lib.lib().l2h_model_finalize(self.handle))
             self.path = _lib.lib().l2h_model_path(self.handle)  # 1 = kernel per phase, 2 = persistent kernel
@@ -196,11 +198,11 @@ class LanguageModel:  # src/inference.jl:50-54
         self.config, self.tokenizer, self.weights = config, tokenizer, weights
         self._device = None
 
-    def device(self, ctx=None, path=0):
+    def device(self, ctx=None, path=0, kv_fp16=False):
         """Upload once; later calls reuse the resident copy (a closed one is replaced).  path: see
-        l2h_model_set_path; it takes effect when the copy is made."""
+        l2h_model_set_path; kv_fp16: an fp16 KV cache (l2h_model_set_kv_type).  Both take effect when the copy is made."""
         if self._device is None or not self._device.handle:
-            self._device = DeviceModel(self.config, self.weights, ctx, path)
+            self._device = DeviceModel(self.config, self.weights, ctx, path, kv_fp16)
         return self._device
 
     def __str__(self):  # src/inference.jl:56-60

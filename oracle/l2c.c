@@ -24,6 +24,9 @@
  *                         summation order up to fp64 round-off, so a parallel
  *                         implementation reproduces it (almost always bit for bit).
  *   3 = both              the specification of the GPU path.
+ *   L2C_KV16     (4)      the rows appended to the KV cache are rounded to binary16 (round to
+ *                         nearest even) and read back widened: the device's optional fp16 cache.
+ *                         Not in the reference, whose cache is Float32 (src/inference.jl:62-65).
  *
  * What pins this file (the reference ships no tests, fixtures or golden vectors):
  *   codecs   hand-built blocks with by-hand expected values, per-field toggles of the
@@ -49,6 +52,7 @@
 
 #define L2C_ACT_Q8K 1
 #define L2C_CANON 2
+#define L2C_KV16 4
 
 enum { L2C_F32 = 0, L2C_Q4_K = 12, L2C_Q5_K = 13, L2C_Q6_K = 14 }; /* src/load_gguf.jl:26-42 */
 
@@ -90,6 +94,34 @@ int64_t l2c_block_bytes(int type) {
     case L2C_Q6_K: return 210;
     }
     return -1;
+}
+
+/* IEEE binary32 -> binary16, round to nearest even, overflow to infinity, subnormals kept (what
+ * Julia's Float16(::Float32) and numpy's astype(float16) do). */
+uint16_t l2c_fp32_to_fp16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t mag = x & 0x7FFFFFFFu;
+    if (mag >= 0x7F800000u) return (uint16_t)(sign | 0x7C00u | ((mag > 0x7F800000u) ? 0x200u : 0u)); /* inf / nan */
+    if (mag >= 0x477FF000u) return (uint16_t)(sign | 0x7C00u); /* >= 65520 rounds to infinity */
+    if (mag < 0x33000001u) return (uint16_t)sign;               /* <= 2^-25: rounds to zero (2^-25 itself ties to even 0) */
+    const int e = (int)(mag >> 23) - 127;
+    uint32_t man = (mag & 0x7FFFFFu) | 0x800000u; /* 24-bit significand */
+    int shift;                                      /* bits to drop */
+    uint32_t base;
+    if (e >= -14) { /* normal half: keep 11 bits */
+        shift = 13;
+        base = (uint32_t)(e + 15) << 10;
+        man &= 0x7FFFFFu; /* implicit bit goes into the exponent field */
+    } else {          /* subnormal half: value = man * 2^(e-23), unit 2^-24 */
+        shift = 13 + (-14 - e);
+        base = 0;
+    }
+    uint32_t q = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++; /* a carry runs into the exponent field: correct */
+    return (uint16_t)(sign | (base + q));
 }
 
 /* IEEE binary16 -> binary32, exact (Julia's Float32(::Float16), src/kquants.jl:74). */
@@ -730,6 +762,12 @@ int l2c_forward(l2c_model *m, int token, int pos0, int mode, float *logits_out) 
         mm(m, m->v, &w[L2C_WV], m->xb, mode);                               /* :249 */
         l2c_rope(m->q, hs, c->n_heads, pos0, theta_scale, c->rope_is_neox, mode);    /* :255 */
         l2c_rope(m->k, hs, c->n_kv_heads, pos0, theta_scale, c->rope_is_neox, mode); /* :256 */
+        if (mode & L2C_KV16) {
+            for (int i = 0; i < kv_dim; i++) {
+                m->k[i] = l2c_fp16_to_fp32(l2c_fp32_to_fp16(m->k[i]));
+                m->v[i] = l2c_fp16_to_fp32(l2c_fp32_to_fp16(m->v[i]));
+            }
+        }
         memcpy(kc + (size_t)pos0 * kv_dim, m->k, (size_t)kv_dim * 4); /* :259 */
         memcpy(vc + (size_t)pos0 * kv_dim, m->v, (size_t)kv_dim * 4); /* :260 */
         l2c_attention(m->xb, m->q, kc, vc, m->att, hs, c->n_heads, c->n_kv_heads, pos0, mode); /* :266-278 */

@@ -12,7 +12,7 @@ import numpy as np
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libl2c.so")
 
-ACT_Q8K, CANON = 1, 2
+ACT_Q8K, CANON, KV16 = 1, 2, 4
 GPU_SPEC = ACT_Q8K | CANON  # the mode the HIP path implements
 REFERENCE = 0               # float activations, fp32 sums in index order: the reference snapshot
 
@@ -48,6 +48,7 @@ def lib():
         sig = {
             "l2c_block_bytes": (_I64, [_I]),
             "l2c_fp16_to_fp32": (_F, [C.c_uint16]),
+            "l2c_fp32_to_fp16": (C.c_uint16, [_F]),
             "l2c_scale_min_k4": (None, [_P, _P, _P]),
             "l2c_dequantize": (_I, [_I, _P, _I64, _P]),
             "l2c_vecdot_f32act": (_F, [_I, _P, _I64, _P, _I]),

@@ -325,3 +325,22 @@ def test_transformer_kquant_model_all_modes(orc, rng, plan):
     b = [m.forward(t, p, 3) for p, t in enumerate(tokens)]
     for p in range(len(tokens)):
         assert rel(a[p], b[p]) < 1e-4  # fp32 against fp64 sums of the same integer dot products
+
+
+def test_fp32_to_fp16_matches_numpy(orc, rng):
+    """l2c_fp32_to_fp16 (the KV16 mode's rounding) against numpy's float16 conversion: random values over the
+    whole range, every half-way point between consecutive half values and its two neighbours (ties go to even),
+    the overflow threshold 65520, subnormals, zeros and infinities."""
+    L = orc.lib()
+    x = (rng.standard_normal(40000) * rng.choice([1e-8, 1e-5, 1e-3, 1, 100, 30000, 70000], 40000)).astype(np.float32)
+    h = np.arange(0, 0x7C00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    mid = ((h[:-1].astype(np.float64) + h[1:].astype(np.float64)) / 2).astype(np.float32)
+    edge = np.array([0, -0.0, 65504, 65519.996, 65520, 65536, 1e38, -1e38, np.inf, -np.inf, 2.0 ** -24, 2.0 ** -25,
+                     2.0 ** -25 * 1.0001, 2.0 ** -24 * 1.5, 2.0 ** -14, 2.0 ** -14 * (1 - 2.0 ** -11)], np.float32)
+    x = np.concatenate([x, mid, -mid, np.nextafter(mid, np.float32(np.inf)), np.nextafter(mid, np.float32(-np.inf)), edge])
+    got = np.array([L.l2c_fp32_to_fp16(float(v)) for v in x], np.uint16)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+    back = np.array([L.l2c_fp16_to_fp32(int(b)) for b in got[:2000]], np.float32)
+    assert np.array_equal(back, got[:2000].view(np.float16).astype(np.float32))
