@@ -23,9 +23,11 @@ sys.path.insert(0, ROOT)
 import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
-# (workload, launch path) -> bytes; path 1: per matvec launch, 31.23 MB read + 0.04 MB written
-# path 3: per token launch, 4474.4 MB read + 9.5 MB written (profiles/pmc_fetch_write_bench_8b-q4ks_streaming.md)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4505400000}
+# HBM traffic of the dominant kernel per launch, from rocprofv3 --pmc runs of this script (FETCH_SIZE x 2.000 KiB +
+# WRITE_SIZE x 1.000 KiB per unit, the factors a plain read of known size gave in the same runs):
+#   (workload, launch path 1): per matvec launch, 31.23 MB read + 0.04 MB written (profiles/pmc_fetch_write_bench_8b-q4ks.md)
+#   (workload, launch path 3): per token launch, 4489.4 MB read + 9.3 MB written (profiles/pmc_fetch_write_bench_8b-q4ks_streaming.md)
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4498700000}
 
 WORKLOADS = {
     # name: (plan, config kwargs, prompt length)
@@ -33,6 +35,10 @@ WORKLOADS = {
                                     vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
     "8b-q5km": ("PLAN_Q5_K_M", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
                                     vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
+    # the same shape with the tensor mix of a Q4_K_S file as llama.cpp is said to write it: attn_v and ffn_down of the
+    # first four layers q5_K (the streaming kernel takes all-q4_K layers only: this runs on launch path 1)
+    "8b-q4ks-file": ("plan_q4_k_s_file", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
+                                              vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
     "llama2c-f32": ("PLAN_F32", dict(dim=512, hidden_dim=1376, n_layers=8, n_heads=8, n_kv_heads=8, vocab_size=32000,
                                      seq_len=1024, rope_freq_base=10000.0, rope_is_neox=False), 16),
     # Phi-3-mini shape, no GQA, neox RoPE, 4096-long cache pre-filled with 3840 seeded rows: attention-dominated
@@ -95,13 +101,17 @@ def main():
     info = ctx.device_info()
     log("device:", info)
     t0 = time.time()
-    lm = synth.synthetic_model(cfg, getattr(synth, plan_name), seed=20240607,
+    plan = getattr(synth, plan_name)
+    if callable(plan):
+        plan = plan(cfg.n_layers)
+    lm = synth.synthetic_model(cfg, plan, seed=20240607,
                                share_classifier=(plan_name == "PLAN_F32"))
     log("model generated + quantized on %d host threads in %.1f s" % (synth._threads(), time.time() - t0))
     t0 = time.time()
     dev = lm.device(path=args.path, kv_fp16=(args.kv == "fp16"))
     ctx.sync()
-    log("uploaded in %.1f s; launch path %d (1 = kernel per phase, 2 = persistent kernel, 3 = streaming kernel)" % (time.time() - t0, dev.path))
+    log("uploaded in %.1f s; launch path %d (1 = kernel per phase, 2 = persistent kernel, 3 = streaming kernel)%s"
+        % (time.time() - t0, dev.path, "; not 3 because: " + dev.path_reason if dev.path_reason else ""))
 
     w_bytes = synth.weight_bytes_per_token(lm)
     kv_dim = cfg.dim // cfg.n_heads * cfg.n_kv_heads

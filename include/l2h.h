@@ -106,6 +106,10 @@ int l2h_model_set_kv_type(l2h_model *m, int kv_type);
  * the choice after finalize (1, 2 or 3). */
 int l2h_model_set_path(l2h_model *m, int path);
 int l2h_model_path(l2h_model *m);
+/* After finalize with the automatic choice: why the streaming kernel (path 3) was not taken, e.g. "layer matrices
+ * must be q4_K" for a file whose first layers hold q5_K attn_v / ffn_down tensors; "" when it was taken.  The
+ * string lives as long as the model. */
+const char *l2h_model_path_reason(l2h_model *m);
 /* Launch paths 2 and 3 wait on the device for other workgroups' results; every such wait gives up after
  * `spins` polls (default 2^20 on path 3, about a second), upon which all workgroups leave the kernel and
  * the call that launched it returns L2H_EHIP; the model stays usable (l2h_state_reset, then decode

@@ -47,6 +47,7 @@ SIGNATURES = {
     "l2h_model_set_tensor": (_I, [_P, _I, _I, _I, _P, _I64, _I64]),
     "l2h_model_get_tensor": (_I, [_P, _I, _I, _P, _I64]),
     "l2h_model_set_kv_type": (_I, [_P, _I]),
+    "l2h_model_path_reason": (C.c_char_p, [_P]),
     "l2h_model_set_path": (_I, [_P, _I]),
     "l2h_model_set_wait_limit": (_I, [_P, C.c_uint]),
     "l2h_model_set_prefill_copy": (_I, [_P, _I]),

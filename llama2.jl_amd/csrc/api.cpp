@@ -242,6 +242,7 @@ struct l2h_model {
     bool flow = false;
     FlowArgs flow_args{};
     int flow_grid = 0, flow_cls_type = 0;
+    std::string flow_why;  // why the streaming kernel was not chosen (empty if it was, or if it was not asked for)
     unsigned int flow_gen = 1;  // epoch of the next launch's input; 0 is what cleared memory holds
     // batched prompt pass: buffers for pf_cap positions, allocated at the first l2h_prefill
     int pf_cap = 0;
@@ -406,6 +407,12 @@ extern "C" int l2h_model_set_path(l2h_model *m, int path) {
     if (path < 0 || path > 3) return set_err(m->ctx, L2H_EINVAL, "path must be 0, 1, 2 or 3");
     m->path_request = path;
     return L2H_OK;
+}
+
+extern "C" const char *l2h_model_path_reason(l2h_model *m) {
+    if (!m || !m->finalized) return "";
+    if (m->kv16) return "an fp16 KV cache runs on launch path 1";
+    return m->flow_why.c_str();
 }
 
 extern "C" int l2h_model_path(l2h_model *m) { return (m && m->finalized) ? (m->flow ? 3 : (m->mega ? 2 : 1)) : 0; }
@@ -725,6 +732,7 @@ static int flow_setup(l2h_model *m) {
     l2h_ctx *ctx = m->ctx;
     const l2h_config &c = m->c;
     m->flow = false;
+    m->flow_why.clear();
     // automatic choice: this kernel where the model fits it (it is the fastest path), else one kernel per phase
     if (m->path_request != 3 && m->path_request != 0) return L2H_OK;
     const bool required = m->path_request == 3;
@@ -746,13 +754,19 @@ static int flow_setup(l2h_model *m) {
     const int grid = ctx->prop.multiProcessorCount;
     const int cls_type = m->glob[L2H_OUTPUT].type;
     std::string why;
-    if (!k_flow_plan(a, types.data(), (int)types.size(), cls_type, grid, &why))
+    if (!k_flow_plan(a, types.data(), (int)types.size(), cls_type, grid, &why)) {
+        m->flow_why = why;
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: %s", why.c_str()) : L2H_OK;
-    if (m->L(0, L2H_RMS_ATT).layer_stride != m->L(0, L2H_RMS_FFN).layer_stride)
+    }
+    if (m->L(0, L2H_RMS_ATT).layer_stride != m->L(0, L2H_RMS_FFN).layer_stride) {
+        m->flow_why = "norm weight slabs differ";
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ") : L2H_OK;
-    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount))
+    }
+    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount)) {
+        m->flow_why = "its workgroups do not fit the device at once";
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: its workgroups do not fit the device at once")
                         : L2H_OK;
+    }
     std::vector<int64_t> off;
     const int64_t total = k_flow_offsets(a, cls_type, grid, off);
     unsigned char *stream = nullptr;

@@ -85,7 +85,8 @@ class DeviceModel:
                 self.ctx.check(_lib.lib().l2h_model_set_kv_type(self.handle, 1))
             self.ctx.check(_lib.lib().l2h_model_set_path(self.handle, path))
             self.ctx.check(_lib.lib().l2h_model_finalize(self.handle))
-            self.path = _lib.lib().l2h_model_path(self.handle)  # 1 = kernel per phase, 2 = persistent kernel
+            self.path = _lib.lib().l2h_model_path(self.handle)  # 1 = kernel per phase, 2 = persistent kernel, 3 = streaming
+            self.path_reason = _lib.lib().l2h_model_path_reason(self.handle).decode()  # why not 3 ("" if 3)
         except Exception:
             self.close()
             raise

@@ -20,6 +20,15 @@ PLAN_Q5_K_M = dict(PLAN_F32, emb=TYPE_Q4_K, wq=TYPE_Q5_K, wk=TYPE_Q5_K, wv=TYPE_
 PLAN_Q4_K = dict(PLAN_F32, **dict.fromkeys(["emb", "output", "wq", "wk", "wv", "wo", "w1", "w2", "w3"], TYPE_Q4_K))
 
 
+def plan_q4_k_s_file(n_layers, n_first=None):
+    """The tensor mix llama.cpp's quantizer is said to give a Q4_K_S file (not checked against a real file here):
+    as PLAN_Q4_K_S, but attn_v and ffn_down of the first n_layers / 8 layers are q5_K.  A plan entry may be a
+    list with one type per layer."""
+    n_first = n_layers // 8 if n_first is None else n_first
+    per_layer = [TYPE_Q5_K if l < n_first else TYPE_Q4_K for l in range(n_layers)]
+    return dict(PLAN_Q4_K_S, wv=per_layer, w2=per_layer)
+
+
 def _threads():
     return max(1, min(16, os.cpu_count() or 1))
 
@@ -65,8 +74,9 @@ def synthetic_model(config, plan, seed=1234, sigma=0.02, share_classifier=False)
     hs = c.dim // c.n_heads
     kv_dim = hs * c.n_kv_heads
 
-    def mat(stream, ne1, ne0, role):
-        return make_matrix(seed, stream, ne1, ne0, plan[role], sigma)
+    def mat(stream, ne1, ne0, role, layer=0):
+        t = plan[role]
+        return make_matrix(seed, stream, ne1, ne0, t[layer] if isinstance(t, (list, tuple)) else t, sigma)
 
     emb = mat(1, c.vocab_size, c.dim, "emb")
     layers = []
@@ -74,9 +84,9 @@ def synthetic_model(config, plan, seed=1234, sigma=0.02, share_classifier=False)
         s = 100 + 16 * l
         layers.append(TransformerLayerWeights(
             rms_att_weight=np.ones(c.dim, np.float32), rms_ffn_weight=np.ones(c.dim, np.float32),
-            wq=mat(s + 0, c.dim, c.dim, "wq"), wk=mat(s + 1, kv_dim, c.dim, "wk"), wv=mat(s + 2, kv_dim, c.dim, "wv"),
-            wo=mat(s + 3, c.dim, c.dim, "wo"), w1=mat(s + 4, c.hidden_dim, c.dim, "w1"),
-            w2=mat(s + 5, c.dim, c.hidden_dim, "w2"), w3=mat(s + 6, c.hidden_dim, c.dim, "w3")))
+            wq=mat(s + 0, c.dim, c.dim, "wq", l), wk=mat(s + 1, kv_dim, c.dim, "wk", l), wv=mat(s + 2, kv_dim, c.dim, "wv", l),
+            wo=mat(s + 3, c.dim, c.dim, "wo", l), w1=mat(s + 4, c.hidden_dim, c.dim, "w1", l),
+            w2=mat(s + 5, c.dim, c.hidden_dim, "w2", l), w3=mat(s + 6, c.hidden_dim, c.dim, "w3", l)))
     output = emb if share_classifier else mat(2, c.vocab_size, c.dim, "output")
     weights = TransformerWeights(emb, layers, np.ones(c.dim, np.float32), output)
     return LanguageModel(c, dummy_tokenizer(c.vocab_size), weights)
