@@ -811,6 +811,10 @@ static int flow_setup(l2h_model *m) {
     TA(a.hbw, 2 * (int64_t)c.hidden_dim);
     HIPCHK(ctx, hipMemset(a.hbw, 0xFF, 2 * (size_t)c.hidden_dim * 4));
     TA(a.amax, 2 * grid);
+    {
+        const int64_t G = grid / c.n_heads;
+        TA(a.att_x, (int64_t)c.n_heads * G * 3 + (int64_t)c.n_heads * G * m->hs * 2);
+    }
     TA(a.abort_flag, 1);
 #undef TA
     a.kc = m->kc;

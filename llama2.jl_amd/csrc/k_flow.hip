@@ -1088,61 +1088,101 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
 }
 #undef ATL
 
-// longer caches: the same arithmetic with loops over the timesteps
-__device__ __noinline__ bool flow_attention_long(int layer, int h, int pos, unsigned e_in, unsigned e_out) {
-    layer = uni(layer), h = uni(h), pos = uni(pos), e_in = uni(e_in), e_out = uni(e_out);
+// Longer caches: the G = (workgroups / heads) workgroups h*G .. h*G + G-1 share head h, each taking a run of the
+// timesteps, so that the whole chip reads the cache.  The arithmetic is that of attention_head with the sums
+// regrouped: a member publishes its run's largest score, every member takes the largest of all; then e = fp32(exp(s -
+// max)) and the run's fp64 sum of e, published; every member adds the sums in member order and rounds (softmax!'s
+// sum); then p = e / sum (fp32) and the run's fp64 partial value sums, published; member j adds the partial sums of
+// its hs / G output elements in member order, rounds and stores them.  The exchanged numbers are {32 bits, epoch}
+// words like q, k, v (a double travels as two of them); every wait is bounded.
+__device__ __forceinline__ void tag_store_f64(u64 *p, double v, unsigned epoch) {
+    const unsigned long long b = (unsigned long long)__double_as_longlong(v);
+    tag_store(p, __uint_as_float((unsigned)b), epoch);
+    tag_store(p + 1, __uint_as_float((unsigned)(b >> 32)), epoch);
+}
+// waits for the two words of a double; ok is cleared if the wait gave up
+__device__ __forceinline__ double tag_wait_f64(const u64 *p, unsigned epoch, bool &ok) {
+    u64 lo = tag_load(p), hi = tag_load(p + 1);
+    unsigned spins = 0;
+    while (!(tag_is(lo, epoch) && tag_is(hi, epoch))) {
+        if (++spins > c_flow.spin_limit ||
+            ((spins & 63) == 0 && __hip_atomic_load(c_flow.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+            ok = false;
+            break;
+        }
+        lo = tag_load(p);
+        hi = tag_load(p + 1);
+    }
+    return __longlong_as_double((long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned long long)(unsigned)lo));
+}
+
+__device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e_in, unsigned e_out) {
+    layer = uni(layer), pos = uni(pos), e_in = uni(e_in), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
+    // head h runs on workgroups h * G .. h * G + G - 1 (workgroups beyond the last head's take no part)
+    const int G = (int)gridDim.x / a.n_heads, h = (int)blockIdx.x / G, j = (int)blockIdx.x - h * G;
+    if (h >= a.n_heads) return true;
     const int hs = a.hs, seq_len = a.seq_len, np = pos + 1;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
     const float *kc = a.kc + (int64_t)layer * a.cache_layer_elems;
     const float *vc = a.vc + (int64_t)layer * a.cache_layer_elems;
-    double *s_q = (double *)s_act;
-    double *s_p = s_q + hs;
-    double *s_r = s_p + ((seq_len + 1) & ~1);  // keeps the float areas behind it 16-byte aligned
-    float *s_att = (float *)(s_r + (FLOW_NW * hs > 1024 ? FLOW_NW * hs : 1024));
-    float *s_kcur = s_att + ((seq_len + 3) & ~3);
+    // this member's run of timesteps [lo, hi): runs are multiples of 64 long, the last members' may be empty
+    const int C = (((np + G - 1) / G) + 63) & ~63;
+    const int lo = min(np, j * C), hi = min(np, lo + C), nj = hi - lo;
+    double *s_q = (double *)s_act;                                        // [hs]
+    double *s_r = s_q + hs;                                               // [max(16 * hs, 1024)]
+    float *s_att = (float *)(s_r + (FLOW_NW * hs > 1024 ? FLOW_NW * hs : 1024));  // [C]: scores, then e
+    float *s_kcur = s_att + C;
     float *s_vcur = s_kcur + hs;
+    double *s_x = (double *)(s_vcur + hs);                                // [G]: the members' maxima / sums
+    u64 *x_max = a.att_x + (int64_t)h * G;
+    u64 *x_sum = a.att_x + (int64_t)a.n_heads * G + ((int64_t)h * G) * 2;
+    u64 *x_part = a.att_x + (int64_t)a.n_heads * G * 3 + ((int64_t)h * G) * hs * 2;
     const int tid = threadIdx.x;
     bool ok = true;
     __syncthreads();  // the activation area is free
     if (tid < 3 * hs) {
         const int which = tid / hs, i = tid % hs;
-        const u64 *p = which == 0 ? a.q + (int64_t)h * hs + i : (which == 1 ? a.kcur : a.vcur) + (int64_t)kvh * hs + i;
-        u64 w = tag_load(p);
-        unsigned spins = 0;
-        while (!tag_is(w, e_in)) {
-            if (++spins > a.spin_limit ||
-                ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-                ok = false;
-                break;
+        // (k and v of the current position are needed by the member whose run holds it)
+        if (which == 0 || (pos >= lo && pos < hi)) {
+            const u64 *p = which == 0 ? a.q + (int64_t)h * hs + i : (which == 1 ? a.kcur : a.vcur) + (int64_t)kvh * hs + i;
+            u64 w = tag_load(p);
+            unsigned spins = 0;
+            while (!tag_is(w, e_in)) {
+                if (++spins > a.spin_limit ||
+                    ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                    ok = false;
+                    break;
+                }
+                w = tag_load(p);
             }
-            w = tag_load(p);
+            if (which == 0)
+                s_q[i] = (double)tag_val(w);
+            else if (which == 1)
+                s_kcur[i] = tag_val(w);
+            else
+                s_vcur[i] = tag_val(w);
         }
-        if (which == 0)
-            s_q[i] = (double)tag_val(w);
-        else if (which == 1)
-            s_kcur[i] = tag_val(w);
-        else
-            s_vcur[i] = tag_val(w);
     }
     if (!ok) s_flag = 1;
     __syncthreads();
-    if (s_flag) {
-        if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return false;
+#define SPLIT_CHECK()                                                                                              \
+    if (s_flag) {                                                                                                  \
+        if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);             \
+        return false;                                                                                              \
     }
+    SPLIT_CHECK();
     const float scale = sqrtf((float)hs);
     float mx = -INFINITY;
-    // scores: thread = (timestep tl of a block of 256, quarter of the head dimension); the quarter's
-    // 16-byte loads are all in flight at once; quarters are added in order (fp64)
+    // scores: thread = (timestep tl of a block of 256, quarter of the head dimension); the quarter's 16-byte loads
+    // are all in flight at once; quarters are added in order (fp64)
     {
         const int tl = tid & 255, part = tid >> 8, per = hs >> 4;  // hs is a multiple of 16, at most 128
         double *s_sp = s_r;                                        // [4][256]
-        for (int t0 = 0; t0 < np; t0 += 256) {
+        for (int t0 = lo; t0 < hi; t0 += 256) {
             const int t = t0 + tl;
             double acc = 0.0;
-            if (t < np) {
-                // the current position's key is in LDS, the earlier ones in the cache: same code after the loads
+            if (t < hi) {
                 const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
                 const float4 *kl = (const float4 *)s_kcur + part * per;
                 float4 kv[8];
@@ -1161,47 +1201,72 @@ __device__ __noinline__ bool flow_attention_long(int layer, int h, int pos, unsi
             }
             s_sp[part * 256 + tl] = acc;
             __syncthreads();
-            if (part == 0 && t < np) {
+            if (part == 0 && t < hi) {
                 const double v = ((s_sp[tl] + s_sp[256 + tl]) + s_sp[512 + tl]) + s_sp[768 + tl];
                 const float sc = (float)v / scale;
-                s_att[t] = sc;
+                s_att[t - lo] = sc;
                 mx = fmaxf(mx, sc);
             }
             __syncthreads();
         }
     }
     mx = block_max_f32(mx, s_redf);
+    if (tid == 0) tag_store(x_max + j, mx, e_out);
+    if (tid < G) {  // the largest score of the head: every member's
+        const u64 *p = x_max + tid;
+        u64 w = tag_load(p);
+        unsigned spins = 0;
+        while (!tag_is(w, e_out)) {
+            if (++spins > a.spin_limit ||
+                ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                ok = false;
+                break;
+            }
+            w = tag_load(p);
+        }
+        s_x[tid] = (double)tag_val(w);
+    }
+    if (!ok) s_flag = 1;
+    __syncthreads();
+    SPLIT_CHECK();
+    float gmx = -INFINITY;
+    for (int k = 0; k < G; k++) gmx = fmaxf(gmx, (float)s_x[k]);
     double sum = 0.0;
-    for (int t = tid; t < np; t += blockDim.x) {
-        const float e = (float)exp((double)(s_att[t] - mx));
+    for (int t = tid; t < nj; t += blockDim.x) {
+        const float e = (float)exp((double)(s_att[t] - gmx));
         s_att[t] = e;
         sum += (double)e;
     }
-    const float sf = (float)block_sum_f64(sum, s_red);
-    for (int t = tid; t < np; t += blockDim.x) s_p[t] = (double)(s_att[t] / sf);
+    sum = block_sum_f64(sum, s_red);  // (ends with every thread past the reads of s_x above)
+    if (tid == 0) tag_store_f64(x_sum + 2 * j, sum, e_out);
+    if (tid < G) s_x[tid] = tag_wait_f64(x_sum + 2 * tid, e_out, ok);
+    if (!ok) s_flag = 1;
     __syncthreads();
-    // values: thread = (16-byte group i4 of the head dimension, timestep group), up to eight loads in
-    // flight; the groups of one wavefront are folded with lane exchanges, the rest through LDS
-    const int n4 = hs >> 2;         // a power of two (hs 32, 64, 128)
+    SPLIT_CHECK();
+    double tot = 0.0;
+    for (int k = 0; k < G; k++) tot += s_x[k];
+    const float sf = (float)tot;  // softmax!'s sum (reference src/inference.jl:169-174)
+    // values: thread = (16-byte group i4 of the head dimension, timestep group), up to eight loads in flight; the
+    // groups of one wavefront are folded with lane exchanges, the rest through LDS
+    const int n4 = hs >> 2;  // a power of two (hs 32, 64, 128)
     const int ngrp = blockDim.x / n4;
     {
         const int i4 = tid & (n4 - 1), grp = tid / n4;
         const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
         double acc[4] = {0.0, 0.0, 0.0, 0.0};
-        for (int t0 = grp; t0 < np; t0 += 8 * ngrp) {
+        for (int t0 = lo + grp; t0 < hi; t0 += 8 * ngrp) {
             float4 v[8];
 #pragma unroll
             for (int u = 0; u < 8; u++) {
                 const int t = t0 + u * ngrp;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (t < pos) v[u] = vp[(int64_t)t * n4];
-                else if (t == pos) v[u] = *(const float4 *)(s_vcur + 4 * i4);
+                if (t < hi) v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : vp[(int64_t)t * n4];
             }
 #pragma unroll
             for (int u = 0; u < 8; u++) {
                 const int t = t0 + u * ngrp;
-                if (t < np) {
-                    const double p = s_p[t];
+                if (t < hi) {
+                    const double p = (double)(s_att[t - lo] / sf);
                     acc[0] = fma(p, (double)v[u].x, acc[0]);
                     acc[1] = fma(p, (double)v[u].y, acc[1]);
                     acc[2] = fma(p, (double)v[u].z, acc[2]);
@@ -1222,8 +1287,26 @@ __device__ __noinline__ bool flow_attention_long(int layer, int h, int pos, unsi
     if (tid < hs) {
         double acc = 0.0;
         for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
-        bare_store(a.xo + (int64_t)(e_out & 1u) * a.dim + (int64_t)h * hs + tid, bare_of((float)acc));
-        bare_store(a.xo + (int64_t)((e_out & 1u) ^ 1u) * a.dim + (int64_t)h * hs + tid, FLOW_EMPTY);
+        tag_store_f64(x_part + ((int64_t)j * hs + tid) * 2, acc, e_out);
+    }
+    // member j finishes the hs / G output elements j * hs / G ...: thread (element, member) fetches one partial
+    // sum, thread (element, 0) adds them in member order
+    const int per_m = hs / G;
+    __syncthreads();  // (s_r is free)
+    if (tid < per_m * G) {
+        const int el = j * per_m + tid / G, m = tid % G;
+        s_r[tid] = tag_wait_f64(x_part + ((int64_t)m * hs + el) * 2, e_out, ok);
+    }
+    if (!ok) s_flag = 1;
+    __syncthreads();
+    SPLIT_CHECK();
+#undef SPLIT_CHECK
+    if (tid < per_m) {
+        double acc = 0.0;
+        for (int m = 0; m < G; m++) acc += s_r[tid * G + m];
+        const int el = j * per_m + tid;
+        bare_store(a.xo + (int64_t)(e_out & 1u) * a.dim + (int64_t)h * hs + el, bare_of((float)acc));
+        bare_store(a.xo + (int64_t)((e_out & 1u) ^ 1u) * a.dim + (int64_t)h * hs + el, FLOW_EMPTY);
     }
     __syncthreads();
     return true;
@@ -1322,8 +1405,9 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                 ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, a.dim, nw, tok)
                             : flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, nw, tok);
             } else if (kind == 1) {
-                if (is_att) {
-                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_long(l, att_h, pos, e_q, e_att)
+                // (a long cache is shared by all the workgroups of a head, a short one read by one of them)
+                if (is_att || pos >= FLOW_ATT_SHORT) {
+                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_split(l, pos, e_q, e_att)
                                       : a.hs == 128 ? flow_attention_short<128>(l, att_h, pos, e_q, e_att)
                                       : a.hs == 64  ? flow_attention_short<64>(l, att_h, pos, e_q, e_att)
                                                     : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
@@ -1348,7 +1432,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             flow_drain(r);
             flow_reg_arrived(rp);
             FTL();
-            if (kind == 0 && is_att) flow_touch_cache(l, att_h, pos);
+            if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
             flow_loop_q4<true, true>(g, r, ring_base, wg, rp, n_reg);
             FTL();
             FTLS();
@@ -1493,8 +1577,11 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     if (cls_type == L2H_TYPE_Q6_K && a.dim % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
     if (a.hidden > 14336 || a.dim > 4096) return no("dim above 4096 or hidden_dim above 14336");
     if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 128)) return no("head size must be 32, 64 or 128");
-    const size_t att = (size_t)a.hs * 8 + (size_t)((a.seq_len + 1) & ~1) * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 +
-                       (size_t)((a.seq_len + 3) & ~3) * 4 + (size_t)a.hs * 8;
+    // the split attention of long caches: q, the partial sums, one member's run of scores, k and v of the position, G numbers
+    const int G = grid / a.n_heads;
+    if (G < 1 || a.hs % G != 0 || G > 64) return no("head size must be a multiple of workgroups / heads");
+    const size_t run = (size_t)((((a.seq_len + G - 1) / G) + 63) & ~63);
+    const size_t att = (size_t)a.hs * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 + run * 4 + (size_t)a.hs * 8 + 64 * 8;
     if (att > FLOW_ACT_BYTES) return no("sequence too long for the attention area");
     a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim, L2H_TYPE_Q4_K, grid);
     a.wo = make_geom(a.dim, a.dim, L2H_TYPE_Q4_K, grid);

@@ -141,6 +141,9 @@ struct FlowArgs {
     const int64_t *wave_off;      // [grid * 16] byte offset of each wavefront's stream
     // activations as {fp32 value, epoch} words
     unsigned long long *q, *kcur, *vcur, *amax;
+    // long-cache attention: per head and member workgroup the run's largest score [heads][G], its sum of
+    // exponentials [heads][G][2], its partial value sums [heads][G][hs][2]
+    unsigned long long *att_x;
     // activations as bare fp32 words, 0xFFFFFFFF = not written yet: the residual stream in two buffers,
     // attention outputs [2][dim] and SwiGLU outputs [2][hidden] (the pairs alternate from layer to layer)
     unsigned int *x_a, *x_b, *xo, *hbw;

@@ -249,13 +249,17 @@ def test_kv_prefill_and_long_context(pkg, orc, rng, path, seq_len):
     assert _rel(logits, ref_logits) <= 1e-3
 
 
-@pytest.mark.parametrize("n_pre", [250, 300])
-def test_streaming_kernel_long_cache(pkg, orc, rng, n_pre):
+@pytest.mark.parametrize("case,n_pre,seq_len", [("all_q4", 250, 384), ("all_q4", 300, 384), ("all_q4", 1500, 1600),
+                                                ("all_q4_neox", 1000, 1100), ("q4ks_headline_widths", 2100, 4096),
+                                                ("q4ks_headline_widths", 4070, 4096)])
+def test_streaming_kernel_long_cache(pkg, orc, rng, case, n_pre, seq_len):
     """Path 3 decoding into a pre-filled cache: from 250 the run crosses position 256, where the kernel
-    changes from its short-cache attention to the one with loops over the timesteps; from 300 it is in
-    the latter throughout."""
-    plan, kw = FLOW_CASES["all_q4"]
-    kw = dict(kw, seq_len=384, n_layers=2)
+    changes from its short-cache attention (one workgroup per head) to the one in which all workgroups of a
+    head share the cache; the other cases are in the latter throughout: runs of one and of several tiles per
+    member workgroup, empty runs, 16 and 8 member workgroups, with and without GQA, up to the end of a
+    4096-long cache."""
+    plan, kw = FLOW_CASES[case]
+    kw = dict(kw, seq_len=seq_len, n_layers=2)
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
     dev = lm.device(path=3)
@@ -403,3 +407,27 @@ def test_full_size_model_launch_paths_agree(pkg):
         del dev, lm
     assert got[1][0].tolist() == got[3][0].tolist()
     assert np.array_equal(got[1][1], got[3][1])
+
+
+def test_streaming_kernel_soak_against_per_phase_path(pkg):
+    """The streaming kernel's exchange of activations between workgroups rests on timing-independent
+    reasoning (every buffer is rewritten two phases after its last read); this repeats it: 30 generations of
+    128 tokens at the benchmark's widths (two layers), different prompts, each compared bit for bit (tokens
+    and final logits) with the per-phase path, stopping at the first difference or error."""
+    from llama2_jl_amd import synth
+    from llama2_jl_amd.inference import DeviceModel
+    plan, kw = FLOW_CASES["q4ks_headline_widths"]
+    lm = _model(pkg, plan, **kw)
+    fast = DeviceModel(lm.config, lm.weights, path=3)
+    slow = DeviceModel(lm.config, lm.weights, path=1)
+    assert fast.path == 3 and slow.path == 1
+    for rep in range(30):
+        prompt = synth.seeded_prompt(1000 + rep, 1 + rep % 40, kw["vocab_size"])
+        fast.reset()
+        slow.reset()
+        a_ids, a_logits = fast.generate_greedy(prompt, 128, want_logits=True)
+        b_ids, b_logits = slow.generate_greedy(prompt, 128, want_logits=True)
+        assert np.asarray(a_ids).tolist() == np.asarray(b_ids).tolist(), rep
+        assert np.array_equal(a_logits.view(np.uint32), b_logits.view(np.uint32)), rep
+    fast.close()
+    slow.close()

@@ -139,3 +139,31 @@ def test_phi3_full_size_against_oracle(pkg, orc):
     assert _rel(logits, ref_logits) <= 1e-3
     dev.close()
     om.close()
+
+
+def test_q4ks_file_mix_falls_to_path_1_with_a_reason(pkg, orc):
+    """The tensor mix a Q4_K_S file is said to carry (q5_K attn_v and ffn_down in the first layers) at the 8B widths,
+    two layers of which the first holds the q5_K tensors: the streaming kernel takes all-q4_K layers only, so the
+    automatic choice falls to one kernel per phase and says why; q and k share a launch, v runs in one of its own.
+    128 greedy tokens against the oracle."""
+    from llama2_jl_amd import synth
+    kw = dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=32000, seq_len=192,
+              rope_freq_base=500000.0, rope_is_neox=False)
+    cfg = pkg.ModelConfig(**kw)
+    lm = synth.synthetic_model(cfg, synth.plan_q4_k_s_file(2, n_first=1), seed=36)
+    assert lm.weights.layers[0].wv.type == 13 and lm.weights.layers[0].w2.type == 13 and lm.weights.layers[1].wv.type == 12
+    prompt = synth.seeded_prompt(99, 32, kw["vocab_size"])
+    dev = lm.device()
+    assert dev.path == 1 and "q4_K" in dev.path_reason
+    om = orc.model_from_language_model(lm, nthreads=16)
+    ids, logits = dev.generate_greedy(prompt, 128, want_logits=True)
+    ref_ids, ref_logits = om.generate_greedy(prompt, 128, orc.GPU_SPEC)
+    assert ids.tolist() == ref_ids.tolist()
+    assert _rel(logits, ref_logits) <= 1e-3
+    dev.close()
+    om.close()
+    # an all-q4_K model of the same widths takes the streaming kernel and gives no reason
+    lm2 = _model(pkg, "PLAN_Q4_K_S", 37, **dict(kw, n_layers=1))
+    dev2 = lm2.device()
+    assert dev2.path == 3 and dev2.path_reason == ""
+    dev2.close()
