@@ -931,8 +931,8 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     DA(m->part, (int64_t)ntiles * c.dim, true);
     m->cache_layer_elems = (int64_t)c.seq_len * m->kv_dim;
     if (m->kv16) {
-        if (m->hs > 128 || m->hs % 16 != 0)
-            return set_err(ctx, L2H_EINVAL, "an fp16 KV cache needs a head size that is a multiple of 16, at most 128");
+        if (m->hs > 128 || m->hs % 32 != 0)
+            return set_err(ctx, L2H_EINVAL, "an fp16 KV cache needs a head size that is a multiple of 32, at most 128");
         if (m->path_request == 2 || m->path_request == 3)
             return set_err(ctx, L2H_EINVAL, "an fp16 KV cache runs on launch path 1 only");
         m->path_request = 1;

@@ -9,6 +9,11 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h) {
     return (float)__builtin_bit_cast(_Float16, h);
 }
 
+// index of element i of head kvh at timestep t in the fp16 K cache
+__device__ __forceinline__ int64_t kc16_index(int kvh, int i, int t, int hs, int seq_len) {
+    return (((int64_t)kvh * (hs >> 3) + (i >> 3)) * seq_len + t) * 8 + (i & 7);
+}
+
 __device__ __forceinline__ double wave_sum_f64(double v) {
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, WAVE);

@@ -123,28 +123,50 @@ __global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, con
     const int lane = threadIdx.x & 63, part = threadIdx.x >> 6;
     const int h0 = blockIdx.y * GH, kvh = h0 / (n_heads / n_kv_heads);
     for (int i = threadIdx.x; i < GH * hs; i += 256) s_q[(i / hs) * 128 + i % hs] = qd[(int64_t)h0 * hs + i];
-    const int per = hs >> 4;  // 16-byte groups per quarter (hs <= 128: at most 8)
     const int t = min(t0 + lane, pos);
-    const int64_t kg = ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;  // group of four elements
-    float4 kv[8];
-#pragma unroll
-    for (int u = 0; u < 8; u++)
-        if (u < per) kv[u] = ldg_nt_kv4<H16>(kc, kg + (int64_t)u * seq_len);
-    __syncthreads();
     double acc[GH];
 #pragma unroll
     for (int g = 0; g < GH; g++) acc[g] = 0.0;
+    if constexpr (H16) {
+        // fp16 cache: 16-byte groups of eight elements, hs / 32 of them per quarter (hs a multiple of 32, at most 128)
+        const int per8 = hs >> 5;
+        const int64_t kg = ((int64_t)kvh * (hs >> 3) + part * per8) * seq_len + t;
+        Half8 kv[4];
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-        if (u < per) {
-            const double k0 = (double)kv[u].x, k1 = (double)kv[u].y, k2 = (double)kv[u].z, k3 = (double)kv[u].w;
+        for (int u = 0; u < 4; u++)
+            if (u < per8) kv[u] = ldg_nt_h8(kc, kg + (int64_t)u * seq_len);
+        __syncthreads();
 #pragma unroll
-            for (int g = 0; g < GH; g++) {
-                const double *qq = s_q + g * 128 + 4 * (part * per + u);
-                acc[g] = fma(qq[0], k0, acc[g]);
-                acc[g] = fma(qq[1], k1, acc[g]);
-                acc[g] = fma(qq[2], k2, acc[g]);
-                acc[g] = fma(qq[3], k3, acc[g]);
+        for (int u = 0; u < 4; u++) {
+            if (u < per8) {
+#pragma unroll
+                for (int g = 0; g < GH; g++) {
+                    const double *qq = s_q + g * 128 + 8 * (part * per8 + u);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[g] = fma(qq[e], (double)kv[u].v[e], acc[g]);
+                }
+            }
+        }
+    } else {
+        const int per = hs >> 4;  // 16-byte groups per quarter (hs <= 128: at most 8)
+        const int64_t kg = ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;  // group of four elements
+        float4 kv[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (u < per) kv[u] = ldg_nt_f4((const float4 *)kc + kg + (int64_t)u * seq_len);
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            if (u < per) {
+                const double k0 = (double)kv[u].x, k1 = (double)kv[u].y, k2 = (double)kv[u].z, k3 = (double)kv[u].w;
+#pragma unroll
+                for (int g = 0; g < GH; g++) {
+                    const double *qq = s_q + g * 128 + 4 * (part * per + u);
+                    acc[g] = fma(qq[0], k0, acc[g]);
+                    acc[g] = fma(qq[1], k1, acc[g]);
+                    acc[g] = fma(qq[2], k2, acc[g]);
+                    acc[g] = fma(qq[3], k3, acc[g]);
+                }
             }
         }
     }
@@ -212,6 +234,72 @@ __global__ __launch_bounds__(256) void attn_av4_kernel(const float *att, const d
         for (int c = 0; c <= pos / 1024; c++) t += psum[(int64_t)(h0 + g) * npsum + c];
         sf[g] = (float)t;
     }
+    if constexpr (H16) {
+        // fp16 cache: thread = (16-byte group i8 of eight elements, timestep group tg of 16); a tile of 64 timesteps is
+        // four loads per thread, all in flight; the four timestep groups of a wavefront are folded with lane
+        // exchanges, the four wavefronts through LDS
+        const int n8 = hs >> 3;  // at most 16
+        const int i8 = threadIdx.x & 15, tg = threadIdx.x >> 4;
+        const bool active = i8 < n8;
+        double acc[GH][8];
+#pragma unroll
+        for (int g = 0; g < GH; g++)
+#pragma unroll
+            for (int c = 0; c < 8; c++) acc[g][c] = 0.0;
+        for (int t0 = c0; t0 < c0 + chunk && t0 <= pos; t0 += 64) {
+            const int nt = min(64, pos + 1 - t0);
+            __syncthreads();
+            for (int i = threadIdx.x; i < GH * 64; i += 256) {
+                const int g = i >> 6, l = i & 63;
+                float sg = sf[0];
+#pragma unroll
+                for (int k = 1; k < GH; k++) sg = g == k ? sf[k] : sg;
+                s_p[g][l] = l < nt ? (double)(att[(int64_t)(h0 + g) * seq_len + t0 + l] / sg) : 0.0;
+            }
+            Half8 v[4];
+            const int64_t vg = ((int64_t)kvh * seq_len + t0) * n8 + i8;
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int l = tg + 16 * u;
+#pragma unroll
+                for (int c = 0; c < 8; c++) v[u].v[c] = 0.f;
+                if (active && l < nt) v[u] = ldg_nt_h8(vc, vg + (int64_t)l * n8);
+            }
+            __syncthreads();
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int l = tg + 16 * u;
+#pragma unroll
+                for (int g = 0; g < GH; g++) {
+                    const double p = s_p[g][l];
+#pragma unroll
+                    for (int c = 0; c < 8; c++) acc[g][c] = fma(p, (double)v[u].v[c], acc[g][c]);
+                }
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < GH; g++)
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                acc[g][c] += __shfl_xor(acc[g][c], 16, WAVE);
+                acc[g][c] += __shfl_xor(acc[g][c], 32, WAVE);
+            }
+        __syncthreads();
+        if (active && (threadIdx.x & 63) < 16) {
+#pragma unroll
+            for (int g = 0; g < GH; g++)
+#pragma unroll
+                for (int c = 0; c < 8; c++) s_red[threadIdx.x >> 6][g][8 * i8 + c] = acc[g][c];
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < GH * hs; i += 256) {
+            const int g = i / hs, e = i % hs;
+            double a = 0.0;
+            for (int k = 0; k < 4; k++) a += s_red[k][g][e];
+            part[((int64_t)split * n_heads + h0 + g) * hs + e] = a;
+        }
+        return;
+    }
     const int n4 = hs >> 2, ngrp = min(8, 256 / n4);  // hs <= 128
     const int i4 = threadIdx.x % n4, tg = threadIdx.x / n4;
     const bool active = tg < ngrp;
@@ -235,7 +323,7 @@ __global__ __launch_bounds__(256) void attn_av4_kernel(const float *att, const d
             for (int u = 0; u < 8; u++) {
                 const int l = tg + ngrp * u;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (l < nt) v[u] = ldg_nt_kv4<H16>(vc, vg + (int64_t)l * n4);
+                if (l < nt) v[u] = ldg_nt_f4((const float4 *)vc + vg + (int64_t)l * n4);
             }
         }
         __syncthreads();

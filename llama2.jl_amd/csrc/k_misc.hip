@@ -182,6 +182,7 @@ __global__ __launch_bounds__(256) void kv_layout_kernel(float *kc, float *vc, fl
     const int64_t vi = ((int64_t)h * seq_len + t) * hs + i;
     if (kv16) {  // fp16 cache: rounded to nearest even on the way in, widened exactly on the way out
         __half *kh = (__half *)kc, *vh = (__half *)vc;
+        const int64_t ki = kc16_index(h, i, t, hs, seq_len);  // (the fp16 K cache groups eight elements)
         if (to_cache) {
             kh[ki] = __float2half_rn(k_lin[gid]);
             vh[vi] = __float2half_rn(v_lin[gid]);

@@ -17,15 +17,26 @@ __device__ __forceinline__ float4 ldg_nt_f4(const float4 *p) {
     const f32x4v t = __builtin_nontemporal_load((const f32x4v *)p);
     return make_float4(t.x, t.y, t.z, t.w);
 }
-// The KV cache holds fp32 (the reference's, src/inference.jl:62-65) or, as an option, fp16 elements in the
-// same index layout.  Group g of four consecutive elements, widened to fp32 (exact):
-template <bool H16>
-__device__ __forceinline__ float4 ldg_nt_kv4(const void *base, int64_t g) {
-    if (!H16) return ldg_nt_f4((const float4 *)base + g);
-    typedef unsigned int u32x2v __attribute__((ext_vector_type(2)));
-    const u32x2v t = __builtin_nontemporal_load((const u32x2v *)base + g);
-    return make_float4(half_bits_to_float((uint16_t)(t.x & 0xFFFF)), half_bits_to_float((uint16_t)(t.x >> 16)),
-                       half_bits_to_float((uint16_t)(t.y & 0xFFFF)), half_bits_to_float((uint16_t)(t.y >> 16)));
+// The KV cache holds fp32 elements (the reference's, src/inference.jl:62-65) or, as an option, fp16 ones.  In both a
+// lane reads 16 bytes per load: the fp32 K cache is [n_kv][hs/4][seq_len][4], the fp16 one [n_kv][hs/8][seq_len][8]; V is
+// [n_kv][seq_len][hs] in both.
+struct Half8 {
+    float v[8];
+};
+// 8 consecutive fp16 elements (group g of 16 bytes), widened to fp32 (exact)
+__device__ __forceinline__ Half8 ldg_nt_h8(const void *base, int64_t g) {
+    typedef unsigned int u32x4v_ __attribute__((ext_vector_type(4)));
+    const u32x4v_ t = __builtin_nontemporal_load((const u32x4v_ *)base + g);
+    Half8 r;
+    r.v[0] = half_bits_to_float((uint16_t)(t.x & 0xFFFF));
+    r.v[1] = half_bits_to_float((uint16_t)(t.x >> 16));
+    r.v[2] = half_bits_to_float((uint16_t)(t.y & 0xFFFF));
+    r.v[3] = half_bits_to_float((uint16_t)(t.y >> 16));
+    r.v[4] = half_bits_to_float((uint16_t)(t.z & 0xFFFF));
+    r.v[5] = half_bits_to_float((uint16_t)(t.z >> 16));
+    r.v[6] = half_bits_to_float((uint16_t)(t.w & 0xFFFF));
+    r.v[7] = half_bits_to_float((uint16_t)(t.w >> 16));
+    return r;
 }
 // element i of a cache <- v (fp16: rounded to nearest even)
 __device__ __forceinline__ void st_kv(void *base, int64_t i, float v, bool h16) {
@@ -607,11 +618,10 @@ __device__ __forceinline__ void finish_row(const PhaseArgs &a, int layer, int64_
             st_f32<COH>(a.y[0] + rr.row, out);  // q is always the first segment of its launch
             st_f64<COH>(a.qd + rr.row, (double)out);
         } else {
-            const int64_t ki = (((int64_t)h * (a.hs >> 2) + (e >> 2)) * a.seq_len + pos) * 4 + (e & 3);
             if (a.kv16)
-                st_kv(at_layer(a.kc, a.cache_stride, layer), ki, out, true);
+                st_kv(at_layer(a.kc, a.cache_stride, layer), kc16_index(h, e, pos, a.hs, a.seq_len), out, true);
             else
-                st_f32<COH>(at_layer(a.kc, a.cache_stride, layer) + ki, out);
+                st_f32<COH>(at_layer(a.kc, a.cache_stride, layer) + (((int64_t)h * (a.hs >> 2) + (e >> 2)) * a.seq_len + pos) * 4 + (e & 3), out);
         }
     }
 }
