@@ -1,12 +1,17 @@
 """Builds libl2hip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
-Usage:  python llama2.jl_amd/build.py [--timeline]
+Usage:  python llama2.jl_amd/build.py [--timeline | --microbench]
 The objects are compiled in parallel (one hipcc per source file) and linked into
 llama2.jl_amd/libl2hip.so.  hipcc cross-compiles: no GPU is needed to build.
 
 --timeline builds llama2.jl_amd/libl2hip_tl.so instead: the same library with -DL2H_TIMELINE, in which the
 streaming decode kernel stamps the wall clock at every phase boundary (llama2.jl_amd/timeline.py prints
 the table).  The product library is not touched.
+
+--microbench builds three stand-alone programs into llama2.jl_amd/build_mb/ (csrc/microbench/): `stream` (how fast
+256 x 16 wavefronts read bytes in the access patterns of the streaming decode kernel), `loop` (that kernel's q4_K
+piece loop alone, with and without its fetches) and `exchange` (one "every workgroup reads the whole vector"
+hand-over through device memory).  Each prints a table; run them on the GPU without arguments.
 """
 import concurrent.futures
 import os
@@ -74,6 +79,23 @@ def build(force=True, verbose=True, timeline=False):
     return lib
 
 
+def build_microbench(verbose=True):
+    out = os.path.join(HERE, "build_mb")
+    os.makedirs(out, exist_ok=True)
+    for name in ("stream", "loop", "exchange"):
+        exe = os.path.join(out, name)
+        cmd = [_hipcc(), os.path.join(CSRC, "microbench", name + ".hip"), "-o", exe, "-O3", "-std=c++17", "-ffp-contract=off",
+               "-I", os.path.join(ROOT, "include"), "-I", CSRC] + DEVICE
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("hipcc failed on %s:\n%s" % (name, r.stdout + r.stderr))
+        if verbose:
+            print("built", exe)
+
+
 if __name__ == "__main__":
-    build(force=True, timeline="--timeline" in sys.argv[1:])
+    if "--microbench" in sys.argv[1:]:
+        build_microbench()
+    else:
+        build(force=True, timeline="--timeline" in sys.argv[1:])
     sys.exit(0)
