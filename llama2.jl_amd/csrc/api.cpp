@@ -762,16 +762,45 @@ static int flow_setup(l2h_model *m) {
         m->flow_why = "norm weight slabs differ";
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ") : L2H_OK;
     }
-    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount)) {
+    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount, a.mixed != 0)) {
         m->flow_why = "its workgroups do not fit the device at once";
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: its workgroups do not fit the device at once")
                         : L2H_OK;
     }
     std::vector<int64_t> off;
-    const int64_t total = k_flow_offsets(a, cls_type, grid, off);
+    int64_t total = 0;
+    FlowTypedTables tt;
+    FlowTypedDev typed;
+    std::vector<void *> tmp;  // tables that only the repack kernels read
+    int rc;
+    if (a.mixed) {
+        k_flow_typed_tables(a, types.data(), cls_type, grid, tt);
+        off = tt.wave_off;
+        total = tt.total;
+        auto up = [&](const void *src, size_t bytes, const void **dst) -> int {
+            void *v = nullptr;
+            HIPCHK(ctx, hipMalloc(&v, std::max<size_t>(bytes, 16)));
+            tmp.push_back(v);
+            HIPCHK(ctx, hipMemcpy(v, src, bytes, hipMemcpyHostToDevice));
+            *dst = v;
+            return L2H_OK;
+        };
+        if ((rc = up(tt.piece_base.data(), tt.piece_base.size() * 8, (const void **)&typed.piece_base)) ||
+            (rc = up(tt.cls_off.data(), tt.cls_off.size() * 8, (const void **)&typed.cls_off)) ||
+            (rc = up(tt.piece_off.data(), tt.piece_off.size() * 8, (const void **)&typed.piece_off)) ||
+            (rc = up(tt.piece_tag.data(), tt.piece_tag.size() * 2, (const void **)&typed.piece_tag))) {
+            for (void *v : tmp) (void)hipFree(v);
+            return rc;
+        }
+        unsigned int *wt = nullptr;
+        if ((rc = dalloc(m, &wt, (int64_t)tt.wave_types.size(), false))) return rc;
+        HIPCHK(ctx, hipMemcpy(wt, tt.wave_types.data(), tt.wave_types.size() * 4, hipMemcpyHostToDevice));
+        a.wave_types = wt;
+    } else {
+        total = k_flow_offsets(a, cls_type, grid, off);
+    }
     unsigned char *stream = nullptr;
     int64_t *off_dev = nullptr;
-    int rc;
     if ((rc = dalloc(m, &stream, total, false))) return rc;
     if ((rc = dalloc(m, &off_dev, (int64_t)off.size(), false))) return rc;
     HIPCHK(ctx, hipMemcpy(off_dev, off.data(), off.size() * 8, hipMemcpyHostToDevice));
@@ -780,13 +809,14 @@ static int flow_setup(l2h_model *m) {
         const DevTensor wo[1] = {m->L(l, L2H_WO)};
         const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
         const DevTensor w2[1] = {m->L(l, L2H_W2)};
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 0, l, qkv, 3, grid, cls_type));
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 1, l, wo, 1, grid, cls_type));
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 2, l, w13, 2, grid, cls_type));
-        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 3, l, w2, 1, grid, cls_type));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 0, l, qkv, 3, grid, cls_type, typed));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 1, l, wo, 1, grid, cls_type, typed));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 2, l, w13, 2, grid, cls_type, typed));
+        HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 3, l, w2, 1, grid, cls_type, typed));
     }
-    HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid, cls_type));
+    HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid, cls_type, typed));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    for (void *v : tmp) HIPCHK(ctx, hipFree(v));
     a.stream = stream;
     a.wave_off = off_dev;
     // the exchanged words live in uncached memory, zeroed like any other allocation
@@ -849,7 +879,7 @@ static hipError_t flow_launch_token(l2h_model *m) {
         if (eb != hipSuccess) return eb;
         g_flow_bound = m;
     }
-    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, m->flow_cls_type, m->flow_grid);
+    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, m->flow_cls_type, m->flow_grid, m->flow_args.mixed != 0);
     if (e == hipSuccess) m->flow_gen += 5u * (unsigned)m->c.n_layers + 2u;
     return e;
 }

@@ -703,6 +703,221 @@ __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigne
     q.end(r, cnt, left0 - q.left);
 }
 
+// ------------------------------------------------------------------------------------------
+// typed pieces: models whose layer matrices are not all q4_K (reference src/kquants.jl:186-408)
+// ------------------------------------------------------------------------------------------
+// A piece is still eight super-blocks of one row, in one of three formats, each with a 16-byte tag at byte 128:
+//   q4_K  1168 B: headers 128 (as above) | tag 16 | quants 1024
+//   q5_K  1424 B: headers 128 | tag 16 | high bits 8 x 32 | quants 1024
+//   q6_K  1696 B: scales 8 x 16 (bytes permuted: dword 2n+h of a super-block = the scales of its groups 0..3 at
+//                 128n + 32g + 16h) | tag 16 | d 8 x 2 | high bits 8 x 64 | low nibbles 1024
+// The ring has FLOWM_D slots of the largest size.  Every piece is fetched with two instructions (the first
+// `head lanes` x 16 bytes, then 1024 bytes), so the count of fetches under way still tells which pieces have landed.
+// The fetch side must know the format of a piece before it has seen it: byte 1 of a piece's tag holds the type of
+// the piece FLOWM_D places further on in the wavefront's stream, which is the one that will be fetched into
+// the slot this piece leaves (byte 0: the piece's own type); the types of a stream's first FLOWM_D pieces come
+// from a table (FlowArgs::wave_types, two bits each).
+#define FLOWM_SLOT 1696
+#define FLOWM_D 4
+__host__ __device__ inline int flowm_piece_bytes(int t) { return t == 0 ? 1168 : (t == 1 ? 1424 : 1696); }
+__host__ __device__ inline int flowm_head_lanes(int t) { return t == 0 ? 9 : (t == 1 ? 25 : 42); }
+
+struct MRing {
+    const unsigned char *gptr;  // next byte of the stream to fetch
+    unsigned lds;               // LDS byte address of slot 0
+    int slot;                   // slot of the piece to use next
+    int held, ready;            // pieces fetched and not yet used; of those, known to have landed
+    int left;                   // pieces of the stream not fetched yet
+    unsigned tq;                // types of the held pieces, two bits each, the next to use lowest
+};
+
+__device__ __forceinline__ void flowm_fetch(const unsigned char *g, unsigned char *slot, int t, int lane) {
+    const int nb = uni(flowm_head_lanes(t));
+    const unsigned char *gl = g + lane * 16;
+    if (lane < nb) __builtin_amdgcn_global_load_lds((const AS1 void *)gl, (AS3 void *)slot, 16, 0, 2);
+    __builtin_amdgcn_global_load_lds((const AS1 void *)(gl + nb * 16), (AS3 void *)(slot + nb * 16), 16, 0, 2);
+}
+
+// the first pieces of a wavefront's stream
+__device__ __forceinline__ void flowm_start(MRing &r, unsigned char *ring_base, unsigned types, int lane) {
+    r.slot = 0;
+    r.held = r.ready = 0;
+    r.tq = 0;
+#pragma unroll
+    for (int j = 0; j < FLOWM_D; j++) {
+        if (uni(r.left) > 0) {
+            const int t = uni((int)((types >> (2 * j)) & 3u));
+            flowm_fetch(r.gptr, ring_base + j * FLOWM_SLOT, t, lane);
+            r.gptr += flowm_piece_bytes(t);
+            r.tq |= (unsigned)t << (2 * j);
+            r.held++;
+            r.left--;
+        }
+    }
+}
+
+// the dword of a q6_K super-block's 16 permuted scale bytes that belongs to a lane: dword 2n + h (c8 = 4n + 2w + h)
+__device__ __forceinline__ uint32_t flow_q6_scales(const uint4 sc, int c8) {
+    const int dn = 2 * (c8 >> 2) + (c8 & 1);
+    return dn == 0 ? sc.x : (dn == 1 ? sc.y : (dn == 2 ? sc.z : sc.w));
+}
+
+// q5_K: the q4_K term with bit 2j / 2j+1 of the lane's 16 high-bit bytes on top of the nibbles
+__device__ __forceinline__ double flow_q5_term(const uint4 w, const uint4 qh, uint32_t d_dmin, int sc_a, int sc_b, int m_a,
+                                               int m_b, int sa, const uint4 xlo, const uint4 xhi, int bs_a, int bs_b,
+                                               float yd) {
+    const int sb = sa + 1;
+    int dot_a = 0, dot_b = 0;
+#define Q5LO(W, H) (((W)&0x0F0F0F0Fu) | ((((H) >> sa) & 0x01010101u) << 4))
+#define Q5HI(W, H) ((((W) >> 4) & 0x0F0F0F0Fu) | ((((H) >> sb) & 0x01010101u) << 4))
+    dot_a = sdot4(Q5LO(w.x, qh.x), xlo.x, dot_a);
+    dot_a = sdot4(Q5LO(w.y, qh.y), xlo.y, dot_a);
+    dot_a = sdot4(Q5LO(w.z, qh.z), xlo.z, dot_a);
+    dot_a = sdot4(Q5LO(w.w, qh.w), xlo.w, dot_a);
+    dot_b = sdot4(Q5HI(w.x, qh.x), xhi.x, dot_b);
+    dot_b = sdot4(Q5HI(w.y, qh.y), xhi.y, dot_b);
+    dot_b = sdot4(Q5HI(w.z, qh.z), xhi.z, dot_b);
+    dot_b = sdot4(Q5HI(w.w, qh.w), xhi.w, dot_b);
+#undef Q5LO
+#undef Q5HI
+    const int i_sc = mad24(sc_a, dot_a, __mul24(sc_b, dot_b));
+    const int i_min = mad24(m_a, bs_a, __mul24(m_b, bs_b));
+    const float dy = half_bits_to_float((uint16_t)(d_dmin & 0xFFFF)) * yd;
+    const float my = half_bits_to_float((uint16_t)(d_dmin >> 16)) * yd;
+    double t = (double)dy * (double)i_sc;
+    t = fma(-(double)my, (double)i_min, t);
+    return t;
+}
+
+// q6_K: the lane's 16 bytes of low nibbles are ql[64n + 32w + 16h ..]: the low nibbles belong to group w (elements
+// 128n + 32w + 16h ..), the high nibbles to group 2 + w (64 elements further on); bits 2g, 2g+1 of the lane's 16
+// high-bit bytes qh[32n + 16h ..] complete group g (src/kquants.jl:333-336); q - 32 is folded in through the q8_K
+// group sums.  scw = the four scales of groups 0..3, d16 the super-block's d.
+__device__ __forceinline__ double flow_q6_term(const uint4 ql, const uint4 qh, uint32_t scw, uint32_t d16, int w32,
+                                               const uint4 xlo, const uint4 xhi, int bs_lo, int bs_hi, float yd) {
+    const int s_lo = 2 * w32, s_hi = 4 + 2 * w32;
+    int d_lo = 0, d_hi = 0;
+#define Q6LO(L, H) (((L)&0x0F0F0F0Fu) | ((((H) >> s_lo) & 0x03030303u) << 4))
+#define Q6HI(L, H) ((((L) >> 4) & 0x0F0F0F0Fu) | ((((H) >> s_hi) & 0x03030303u) << 4))
+    d_lo = sdot4(Q6LO(ql.x, qh.x), xlo.x, d_lo);
+    d_lo = sdot4(Q6LO(ql.y, qh.y), xlo.y, d_lo);
+    d_lo = sdot4(Q6LO(ql.z, qh.z), xlo.z, d_lo);
+    d_lo = sdot4(Q6LO(ql.w, qh.w), xlo.w, d_lo);
+    d_hi = sdot4(Q6HI(ql.x, qh.x), xhi.x, d_hi);
+    d_hi = sdot4(Q6HI(ql.y, qh.y), xhi.y, d_hi);
+    d_hi = sdot4(Q6HI(ql.z, qh.z), xhi.z, d_hi);
+    d_hi = sdot4(Q6HI(ql.w, qh.w), xhi.w, d_hi);
+#undef Q6LO
+#undef Q6HI
+    const int sc_lo = (int)(int8_t)((scw >> (8 * w32)) & 0xFF), sc_hi = (int)(int8_t)((scw >> (8 * (2 + w32))) & 0xFF);
+    // |d - 32 bsum| < 2^18 and |scale| < 2^7: 24-bit (full-rate) multiplies are exact
+    const int i_sc = mad24(sc_lo, d_lo - 32 * bs_lo, __mul24(sc_hi, d_hi - 32 * bs_hi));
+    const float dy = half_bits_to_float((uint16_t)d16) * yd;
+    return (double)dy * (double)i_sc;
+}
+
+// the streaming loop over typed pieces; partial sums as in flow_loop_q4<., true> (four doubles per piece)
+__device__ __forceinline__ void flow_loop_mixed(const FlowGeom &g, MRing &r, unsigned char *ring_base, int wg) {
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int ppr = uni(g.ppr);
+    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    int part = uni(start % ppr);
+    const int blk = lane >> 3, c8 = lane & 7;
+    // q4_K / q5_K: sub-block pair c8 / 2, half c8 % 2.  q6_K: n = c8 / 4, w = (c8 / 2) % 2, h = c8 % 2.
+    const int pair = c8 >> 1, w32 = (c8 >> 1) & 1;
+    const unsigned act = (unsigned)(size_t)s_act;
+    const unsigned x45 = act + blk * 256 + 64 * (c8 >> 1) + 16 * (c8 & 1);                           // then + 32
+    const unsigned x6 = act + blk * 256 + 128 * (c8 >> 2) + 32 * ((c8 >> 1) & 1) + 16 * (c8 & 1);    // then + 64
+    const unsigned bs45 = act + 14336 + 2 * (blk * 16 + 4 * (c8 >> 1) + (c8 & 1));                   // then + 4
+    const unsigned bs6 = act + 14336 + 2 * (blk * 16 + 8 * (c8 >> 2) + 2 * ((c8 >> 1) & 1) + (c8 & 1));  // then + 8
+    const unsigned xd0 = act + 14336 + 1792 + 4 * blk;
+    const unsigned q5h = 144 + blk * 32 + 16 * (c8 & 1), q6h = 160 + blk * 64 + 32 * (c8 >> 2) + 16 * (c8 & 1);
+    int po = part * 32;
+    double *out = s_part + 4 * start + (lane >> 4);
+    double acc = 0.0;
+    int k = cnt;
+    int slot = uni(r.slot), held = uni(r.held), ready = uni(r.ready), left = uni(r.left);
+    unsigned tq = uni(r.tq);
+    const unsigned char *gp = r.gptr;
+#pragma nounroll
+    for (int i = 0; i < cnt; i++) {
+        if (ready == 0) {
+            if (held == FLOWM_D) {  // the fetches return in order: all but the FLOWM_D - 1 youngest pieces are back
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * (FLOWM_D - 1)) : "memory");
+                ready = 1;
+            } else {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                ready = held;
+            }
+        }
+        const int t = (int)(tq & 3u);
+        const unsigned sl = r.lds + (unsigned)(slot * FLOWM_SLOT);
+        const bool six = t == 2;
+        const unsigned a_w = sl + (t == 0 ? 144u : (t == 1 ? 400u : 672u)) + lane * 16;
+        const unsigned a_h = sl + blk * 16;
+        const unsigned a_q = sl + (six ? q6h : q5h);
+        const unsigned a_xlo = (six ? x6 : x45) + po * 64, a_xhi = a_xlo + (six ? 64u : 32u);
+        const unsigned a_bsa = (six ? bs6 : bs45) + po * 8, a_bsb = a_bsa + (six ? 8u : 4u);
+        const unsigned a_yd = xd0 + po, a_tag = sl + 128, a_d = sl + 144 + 2 * blk;
+        uint4 w, hdr, qh, xlo, xhi;
+        int bs_a, bs_b;
+        float yd;
+        uint32_t tag, d16;
+        // (one statement that the compiler does not look into, as in flow_loop_q4)
+        asm volatile(
+            "ds_read_b128 %0, %10\n\tds_read_b128 %1, %11\n\tds_read_b128 %2, %12\n\tds_read_b128 %3, %13\n\t"
+            "ds_read_b128 %4, %14\n\tds_read_i16 %5, %15\n\tds_read_i16 %6, %16\n\tds_read_b32 %7, %17\n\t"
+            "ds_read_b32 %8, %18\n\tds_read_u16 %9, %19\n\ts_waitcnt lgkmcnt(0)"
+            : "=&v"(w), "=&v"(hdr), "=&v"(qh), "=&v"(xlo), "=&v"(xhi), "=&v"(bs_a), "=&v"(bs_b), "=&v"(yd), "=&v"(tag),
+              "=&v"(d16)
+            : "v"(a_w), "v"(a_h), "v"(a_q), "v"(a_xlo), "v"(a_xhi), "v"(a_bsa), "v"(a_bsb), "v"(a_yd), "v"(a_tag), "v"(a_d)
+            : "memory");
+        tq >>= 2;
+        held--;
+        ready--;
+        if (left > 0) {  // the slot is free again: the piece FLOWM_D places on, whose type this piece's tag names
+            const int nt = uni((int)((tag >> 8) & 3u));
+            flowm_fetch(gp, ring_base + slot * FLOWM_SLOT, nt, lane);
+            gp += flowm_piece_bytes(nt);
+            tq |= (unsigned)nt << (2 * held);
+            held++;
+            left--;
+        }
+        slot = slot + 1 == FLOWM_D ? 0 : slot + 1;
+        if (six) {
+            acc += flow_q6_term(w, qh, flow_q6_scales(hdr, c8), d16, w32, xlo, xhi, bs_a, bs_b, yd);
+        } else {
+            int sc_a, sc_b, m_a, m_b;
+            flow_decode_field(flow_field_of(hdr, pair), sc_a, sc_b, m_a, m_b);
+            if (t == 1)
+                acc += flow_q5_term(w, qh, hdr.x, sc_a, sc_b, m_a, m_b, 2 * pair, xlo, xhi, bs_a, bs_b, yd);
+            else
+                acc += flow_q4_term(w, hdr.x, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
+        }
+        // (as FLOW_PIECE_DONE of flow_loop_q4)
+        part++;
+        po += 32;
+        double v_ = 0.0;
+        if (k == 1 || part == ppr) {
+            v_ = row16_sum_f64_dpp(acc);
+            acc = 0.0;
+            po = 0;
+            part = 0;
+        }
+        *out = v_;
+        out += 4;
+        k--;
+    }
+    r.gptr = gp;
+    r.slot = slot;
+    r.held = held;
+    r.ready = ready;
+    r.left = left;
+    r.tq = tq;
+}
+
 // fp32 value of every local row: the pieces' partial sums added in order
 template <bool QUARTERS>
 __device__ __forceinline__ void flow_row_values(int n_local, int ppr) {
@@ -1315,7 +1530,9 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
 // ------------------------------------------------------------------------------------------
 // the kernel; gen0 = epoch of this launch's input (advances by 5 * n_layers + 2 per launch)
 // ------------------------------------------------------------------------------------------
-template <int T_CLS>
+// MIXED: the layers' pieces are typed (flow_loop_mixed) and none travel through registers; the classifier's
+// pieces follow them in the stream in their usual form, and the ring starts afresh for them.
+template <int T_CLS, bool MIXED>
 __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     const FlowArgs &a = c_flow;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1327,16 +1544,33 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
     r.lds = (unsigned)(size_t)ring_base;
     r.issued = r.consumed = r.drain_mark = 0;
     r.off = 0;
-    // the layers' pieces and, where the classifier is q4_K too, its pieces behind them: one stream
-    const int ring_layer = flow_ring_pieces(a.qkv, wg, wave) + flow_ring_pieces(a.wo, wg, wave) +
-                           flow_ring_pieces(a.w13, wg, wave) + flow_ring_pieces(a.w2, wg, wave);
-    r.left = a.n_layers * ring_layer + (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces(a.cls, wg, wave) : 0);
-    ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
-    // the register pieces follow the ring's part of the stream, in the order in which they are used
-    const unsigned char *reg_ptr = uni(r.gptr + (int64_t)a.n_layers * ring_layer * FLOW_SLOT +
-                                       (int64_t)flow_wave_pieces(a.cls, wg, wave) * (T_CLS == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT));
+    MRing mr;
+    unsigned char *mring_base = s_ring + wave * (FLOWM_D * FLOWM_SLOT);
+    const unsigned char *reg_ptr = nullptr;
     RegPieces rp;
-    flow_top_up_q4(r, ring_base, lane);
+    if constexpr (MIXED) {
+        mr.gptr = r.gptr;
+        mr.lds = (unsigned)(size_t)mring_base;
+        mr.left = a.n_layers * (flow_wave_pieces(a.qkv, wg, wave) + flow_wave_pieces(a.wo, wg, wave) +
+                                flow_wave_pieces(a.w13, wg, wave) + flow_wave_pieces(a.w2, wg, wave));
+        {
+            const unsigned long long p = (unsigned long long)mr.gptr;
+            mr.gptr = (const unsigned char *)(((unsigned long long)uni((unsigned)(p >> 32)) << 32) | uni((unsigned)p));
+            mr.lds = uni(mr.lds);
+            mr.left = uni(mr.left);
+        }
+        flowm_start(mr, mring_base, uni(a.wave_types[wg * FLOW_NW + wave]), lane);
+    } else {
+        // the layers' pieces and, where the classifier is q4_K too, its pieces behind them: one stream
+        const int ring_layer = flow_ring_pieces(a.qkv, wg, wave) + flow_ring_pieces(a.wo, wg, wave) +
+                               flow_ring_pieces(a.w13, wg, wave) + flow_ring_pieces(a.w2, wg, wave);
+        r.left = a.n_layers * ring_layer + (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces(a.cls, wg, wave) : 0);
+        ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
+        // the register pieces follow the ring's part of the stream, in the order in which they are used
+        reg_ptr = uni(r.gptr + (int64_t)a.n_layers * ring_layer * FLOW_SLOT +
+                      (int64_t)flow_wave_pieces(a.cls, wg, wave) * (T_CLS == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT));
+        flow_top_up_q4(r, ring_base, lane);
+    }
 
 #ifdef L2H_TIMELINE
     int tl_n = 0;
@@ -1359,6 +1593,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         flow_drain(r); \
         return;        \
     } while (0)
+    // (flow_drain waits for everything this wavefront has requested, whichever ring it went to)
 
     // ---- this step's token, position and RoPE angles (reference src/inference.jl:122-127) ----
     const int pos = a.ctl->pos;
@@ -1398,8 +1633,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             asm volatile("" : "+v"(tid));
             const int lane = tid & 63;
             const FlowGeom g = flow_geom(a, kind);
-            const int n_reg = uni(flow_reg_pieces(g, wg, wave));
-            if (kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
+            const int n_reg = MIXED ? 0 : uni(flow_reg_pieces(g, wg, wave));
+            if (!MIXED && kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
                 ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, a.dim, nw, tok)
@@ -1413,7 +1648,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                                                     : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
                     if (!uni((int)fine)) LEAVE();
                 }
-                flow_reg_fetch(rp, reg_ptr, n_reg, lane);  // (after the attention: its loads would wait behind these)
+                if (!MIXED) flow_reg_fetch(rp, reg_ptr, n_reg, lane);  // (after the attention: its loads would wait behind these)
                 FTL();
                 ok = flow_stage<PRO_QUANT, SRC_BARE>(a.xo + (int64_t)(e_att & 1u) * a.dim, a.dim, nullptr, tok);
             } else if (kind == 2) {
@@ -1430,10 +1665,16 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             // what the ring holds has landed by now: after this wait the first FLOW_D pieces need none,
             // and the cache lines requested next do not stand between the loop and its pieces
             flow_drain(r);
-            flow_reg_arrived(rp);
+            if constexpr (MIXED)
+                mr.ready = uni(mr.held);
+            else
+                flow_reg_arrived(rp);
             FTL();
             if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
-            flow_loop_q4<true, true>(g, r, ring_base, wg, rp, n_reg);
+            if constexpr (MIXED)
+                flow_loop_mixed(g, mr, mring_base, wg);
+            else
+                flow_loop_q4<true, true>(g, r, ring_base, wg, rp, n_reg);
             FTL();
             FTLS();
             if (kind == 0)
@@ -1450,13 +1691,18 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 
     // ---- final rmsnorm (:309) + classifier (:312); q6_K pieces are larger: the ring starts afresh ----
     const unsigned e_fin = E0 + 5u * (unsigned)a.n_layers, e_cls = e_fin + 1;
-    if (T_CLS == L2H_TYPE_Q6_K) {
+    if (MIXED || T_CLS == L2H_TYPE_Q6_K) {
+        // (the last epilogue's barrier lies behind every wavefront's last piece: the ring areas can be cut anew)
         flow_drain(r);
+        if constexpr (MIXED) r.gptr = mr.gptr;
         r.issued = r.consumed = r.drain_mark = 0;
         r.off = 0;
         r.left = flow_wave_pieces(a.cls, wg, wave);
         ring_uniform(r);
-        flow_top_up_q6(r, ring_base, lane);
+        if (T_CLS == L2H_TYPE_Q6_K)
+            flow_top_up_q6(r, ring_base, lane);
+        else
+            flow_top_up_q4(r, ring_base, lane);
     }
     if (!uni(flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, a.rms_final, tok))) LEAVE();
     flow_drain(r);
@@ -1500,6 +1746,8 @@ struct FlowRepackArgs {
     int layer, n_layers, cls_piece_bytes;
     DevTensor w[3];
     int dim, kv_dim, hs, neox;
+    int mixed;  // typed pieces: placed by the tables
+    FlowTypedDev typed;
 };
 
 // one 64-thread workgroup copies one piece from the per-tensor field streams into its place
@@ -1519,9 +1767,36 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
     const DevTensor &t = seg == 0 ? p.w[0] : (seg == 1 ? p.w[1] : p.w[2]);
     const int64_t layer_b = flow_layer_bytes(p.g4, wg, wave, 4);
     const int lane = threadIdx.x;
+    if (p.mixed && p.kind < 4) {
+        // typed piece: entry of the tables = the wavefront's pieces of earlier layers and phases + idx
+        int before = 0, per_layer = 0;
+        for (int k = 0; k < 4; k++) {
+            const int c = flow_wave_pieces(p.g4[k], wg, wave);
+            per_layer += c;
+            if (k < p.kind) before += c;
+        }
+        const int64_t e = p.typed.piece_base[wg * FLOW_NW + wave] + (int64_t)p.layer * per_layer + before + idx;
+        uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + p.typed.piece_off[e]);
+        const int64_t blk0 = row * t.nb + part * 8;
+        if (lane == 0) dst[8] = make_uint4((uint32_t)p.typed.piece_tag[e], 0u, 0u, 0u);
+        if (t.type == L2H_TYPE_Q4_K) {
+            if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
+            dst[9 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+        } else if (t.type == L2H_TYPE_Q5_K) {
+            if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
+            if (lane < 16) dst[9 + lane] = ((const uint4 *)(t.qh + blk0 * 32))[lane];
+            dst[25 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+        } else {  // q6_K
+            if (lane < 8) dst[lane] = ((const uint4 *)(t.sc6 + blk0 * 4))[lane];
+            if (lane == 1) dst[9] = ((const uint4 *)(t.d6 + blk0))[0];
+            if (lane < 32) dst[10 + lane] = ((const uint4 *)(t.qh + blk0 * 64))[lane];
+            dst[42 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+        }
+        return;
+    }
+    const int64_t cls_at = p.mixed ? p.typed.cls_off[wg * FLOW_NW + wave] : (int64_t)p.n_layers * layer_b;
     if (t.type == L2H_TYPE_Q4_K) {
-        int64_t off = p.kind == 4 ? (int64_t)p.n_layers * layer_b
-                                  : (int64_t)p.layer * layer_b + flow_layer_bytes(p.g4, wg, wave, p.kind);
+        int64_t off = p.kind == 4 ? cls_at : (int64_t)p.layer * layer_b + flow_layer_bytes(p.g4, wg, wave, p.kind);
         int at = idx;
         if (p.kind < 4) {
             const int n_ring = flow_ring_pieces(g, wg, wave);
@@ -1536,7 +1811,7 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
         if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
         dst[8 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
     } else {  // q6_K classifier
-        const int64_t off = (int64_t)p.n_layers * layer_b;
+        const int64_t off = cls_at;
         uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + off + (int64_t)idx * FLOW_Q6_PIECE);
         const int64_t blk0 = row * t.nb + part * 16;
         const uint4 *ql = (const uint4 *)(t.qs + blk0 * 128), *qh = (const uint4 *)(t.qh + blk0 * 64);
@@ -1570,8 +1845,14 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
         if (why) *why = m;
         return false;
     };
-    for (int i = 0; i < n_layer_types; i++)
-        if (layer_types[i] != L2H_TYPE_Q4_K) return no("layer matrices must be q4_K");
+    a.mixed = 0;
+    for (int i = 0; i < n_layer_types; i++) {
+        const int t = layer_types[i];
+        if (t != L2H_TYPE_Q4_K && t != L2H_TYPE_Q5_K && t != L2H_TYPE_Q6_K) return no("layer matrices must be q4_K, q5_K or q6_K");
+        if (t != L2H_TYPE_Q4_K) a.mixed = 1;
+    }
+    for (int l = 0; l * 7 + 6 < n_layer_types; l++)  // (w1 and w3 rows alternate within a workgroup's pieces)
+        if (layer_types[l * 7 + 4] != layer_types[l * 7 + 6]) return no("w1 and w3 of a layer must have one type");
     if (cls_type != L2H_TYPE_Q4_K && cls_type != L2H_TYPE_Q6_K) return no("classifier must be q4_K or q6_K");
     if (a.dim % 2048 != 0 || a.hidden % 2048 != 0) return no("dim and hidden_dim must be multiples of 2048");
     if (cls_type == L2H_TYPE_Q6_K && a.dim % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
@@ -1612,8 +1893,55 @@ int64_t k_flow_offsets(const FlowArgs &a, int cls_type, int grid, std::vector<in
     return total + 4096;  // the last fetches of a stream may be issued past a workgroup's final piece: none are, but pad anyway
 }
 
+void k_flow_typed_tables(const FlowArgs &a, const int *layer_types, int cls_type, int grid, FlowTypedTables &t) {
+    const FlowGeom g4[4] = {a.qkv, a.wo, a.w13, a.w2};
+    const size_t nw = (size_t)grid * FLOW_NW;
+    t.wave_off.assign(nw, 0);
+    t.piece_base.assign(nw, 0);
+    t.cls_off.assign(nw, 0);
+    t.wave_types.assign(nw, 0u);
+    t.piece_off.clear();
+    t.piece_tag.clear();
+    const int cls_piece = cls_type == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT;
+    int64_t total = 0;
+    std::vector<int> types;
+    for (int wg = 0; wg < grid; wg++)
+        for (int w = 0; w < FLOW_NW; w++) {
+            const size_t wi = (size_t)wg * FLOW_NW + w;
+            t.wave_off[wi] = total;
+            t.piece_base[wi] = (int64_t)t.piece_off.size();
+            types.clear();
+            int64_t off = 0;
+            for (int l = 0; l < a.n_layers; l++)
+                for (int kind = 0; kind < 4; kind++) {
+                    const FlowGeom &g = g4[kind];
+                    const int cnt = flow_wave_pieces(g, wg, w), start = flow_wave_start(g, wg, w);
+                    for (int i = 0; i < cnt; i++) {
+                        const int L = wg * g.rpw + (start + i) / g.ppr;
+                        int seg, row;
+                        flow_row_src(kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
+                        const int slot = kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 : 5));
+                        const int ty = layer_types[l * 7 + slot] - L2H_TYPE_Q4_K;
+                        t.piece_off.push_back(off);
+                        types.push_back(ty);
+                        off += flowm_piece_bytes(ty);
+                    }
+                }
+            const size_t n = types.size();
+            for (size_t i = 0; i < n; i++)
+                t.piece_tag.push_back((uint16_t)(types[i] | ((i + FLOWM_D < n ? types[i + FLOWM_D] : 3) << 8)));
+            unsigned first = 0;
+            for (size_t j = 0; j < (size_t)FLOWM_D && j < n; j++) first |= (unsigned)types[j] << (2 * j);
+            t.wave_types[wi] = first;
+            t.cls_off[wi] = off;
+            off += (int64_t)flow_wave_pieces(a.cls, wg, w) * cls_piece;
+            total += (off + 255) & ~(int64_t)255;
+        }
+    t.total = total + 4096;
+}
+
 hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream, const int64_t *wave_off_dev, int kind,
-                         int layer, const DevTensor *w, int nw, int grid, int cls_type) {
+                         int layer, const DevTensor *w, int nw, int grid, int cls_type, const FlowTypedDev &typed) {
     FlowRepackArgs p{};
     p.stream = stream;
     p.wave_off = wave_off_dev;
@@ -1631,6 +1959,8 @@ hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream
     p.kv_dim = a.kv_dim;
     p.hs = a.hs;
     p.neox = a.neox;
+    p.mixed = a.mixed;
+    p.typed = typed;
     const FlowGeom &g = kind == 4 ? a.cls : p.g4[kind];
     hipLaunchKernelGGL(flow_repack_kernel, dim3((unsigned)(grid * g.rpw * g.ppr)), dim3(64), 0, s, p);
     return hipGetLastError();
@@ -1647,9 +1977,16 @@ hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a) {
 // else.  The kernel has no grid-wide barrier and every wait in it is bounded, so residency is what makes it
 // fast, not what makes it correct: workgroups that had to wait for a CU would let the others run into their
 // wait limit, and the launch would end with the error that l2h_model_set_wait_limit describes.
-bool k_flow_fits(int cls_type, int grid, int n_cu) {
-    const void *fn = cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K>
-                                               : (const void *)flow_token_kernel<L2H_TYPE_Q4_K>;
+static const void *flow_kernel_fn(int cls_type, bool mixed) {
+    if (mixed)
+        return cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K, true>
+                                         : (const void *)flow_token_kernel<L2H_TYPE_Q4_K, true>;
+    return cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K, false>
+                                     : (const void *)flow_token_kernel<L2H_TYPE_Q4_K, false>;
+}
+
+bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed) {
+    const void *fn = flow_kernel_fn(cls_type, mixed);
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 1024, 0) != hipSuccess) return false;
     return per_cu >= 1 && (int64_t)per_cu * n_cu >= grid;
@@ -1657,9 +1994,8 @@ bool k_flow_fits(int cls_type, int grid, int n_cu) {
 
 // A plain launch: a cooperative one costs about 20 µs more per token on this stack, and all it would add is the
 // residency check that k_flow_fits makes once.
-hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid) {
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid, bool mixed) {
     void *args[] = {&gen0};
-    const void *fn = cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K>
-                                               : (const void *)flow_token_kernel<L2H_TYPE_Q4_K>;
+    const void *fn = flow_kernel_fn(cls_type, mixed);
     return hipLaunchKernel(fn, dim3(grid), dim3(1024), args, 0, s);
 }

@@ -161,18 +161,36 @@ struct FlowArgs {
     int dim, hidden, hs, n_heads, n_kv_heads, kv_dim, seq_len, n_layers, vocab, neox;
     float theta_scale;
     FlowGeom qkv, wo, w13, w2, cls;
+    // layer matrices that are not all q4_K: typed pieces (k_flow.hip), the types of every wavefront's first pieces
+    int mixed;
+    const unsigned int *wave_types;  // [grid * 16]
 #ifdef L2H_TIMELINE
     long long *timeline;  // profiling build only: [workgroup][64] wall-clock stamps of the first phases
 #endif
 };
+// layer_types: per layer the ggml types of wq, wk, wv, wo, w1, w2, w3 (seven numbers a layer)
 bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls_type, int grid, std::string *why);
 int64_t k_flow_offsets(const FlowArgs &a, int cls_type, int grid, std::vector<int64_t> &off);
+// Where every typed piece goes (a.mixed): per wavefront the stream's offset, the index of its first piece in the
+// per-piece tables, where its classifier pieces start, the types of its first pieces; per piece the byte offset in
+// the wavefront's stream and the tag (own type | type of the piece FLOWM_D places on << 8, 3 = none).
+struct FlowTypedTables {
+    std::vector<int64_t> wave_off, piece_base, cls_off, piece_off;
+    std::vector<uint16_t> piece_tag;
+    std::vector<unsigned int> wave_types;
+    int64_t total = 0;
+};
+void k_flow_typed_tables(const FlowArgs &a, const int *layer_types, int cls_type, int grid, FlowTypedTables &t);
+struct FlowTypedDev {  // the same on the device, for the repack kernel (null for a model of q4_K layers)
+    const int64_t *piece_base = nullptr, *cls_off = nullptr, *piece_off = nullptr;
+    const uint16_t *piece_tag = nullptr;
+};
 // kind 0 q|k|v, 1 wo, 2 w1|w3, 3 w2 (of `layer`), 4 classifier; w: the phase's tensors
 hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream, const int64_t *wave_off_dev, int kind,
-                         int layer, const DevTensor *w, int nw, int grid, int cls_type);
+                         int layer, const DevTensor *w, int nw, int grid, int cls_type, const FlowTypedDev &typed);
 hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a);
-hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid);
-bool k_flow_fits(int cls_type, int grid, int n_cu);
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid, bool mixed);
+bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed);
 
 // ---- launchers (kernel files) ----------------------------------------------------------------
 // Each returns hipGetLastError() of its launch.

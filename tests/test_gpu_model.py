@@ -17,10 +17,11 @@ def _rel(a, b):
 
 
 def _model(pkg, plan_name, **kw):
+    """plan_name: the name of one of synth's tensor-type plans, or a plan itself (role -> type or list of types per layer)"""
     from llama2_jl_amd import synth
     cfg = pkg.ModelConfig(**kw)
-    return synth.synthetic_model(cfg, getattr(synth, plan_name), seed=kw.get("dim", 0) + 11,
-                                 share_classifier=(plan_name == "PLAN_F32"))
+    plan = getattr(synth, plan_name) if isinstance(plan_name, str) else plan_name
+    return synth.synthetic_model(cfg, plan, seed=kw.get("dim", 0) + 11, share_classifier=(plan_name == "PLAN_F32"))
 
 
 CASES = {
@@ -149,6 +150,16 @@ FLOW_CASES = {
     "q4ks_headline_widths": ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8,
                                                  vocab_size=32000, seq_len=192, rope_freq_base=500000.0,
                                                  rope_is_neox=False)),
+    # layer matrices of other types than q4_K travel as typed pieces (reference src/kquants.jl:186-408):
+    # q5_K attention and up/gate, q6_K down and output
+    "q5km_typed": ("PLAN_Q5_K_M", dict(dim=4096, hidden_dim=2048, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=600,
+                                       seq_len=96, rope_freq_base=500000.0, rope_is_neox=False)),
+    # every type in every role, different from layer to layer (the type of a piece's successor is carried in the stream
+    # across phase and layer boundaries), q4_K output
+    "all_types_typed": (dict(emb=12, output=12, wq=[14, 12, 13], wk=[13, 14, 12], wv=[12, 13, 14], wo=[14, 13, 12],
+                             w1=[13, 12, 14], w3=[13, 12, 14], w2=[13, 14, 12]),
+                        dict(dim=2048, hidden_dim=4096, n_layers=3, n_heads=16, n_kv_heads=4, vocab_size=1000, seq_len=96,
+                             rope_freq_base=10000.0, rope_is_neox=True)),
 }
 
 

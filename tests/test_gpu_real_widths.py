@@ -141,11 +141,12 @@ def test_phi3_full_size_against_oracle(pkg, orc):
     om.close()
 
 
-def test_q4ks_file_mix_falls_to_path_1_with_a_reason(pkg, orc):
+def test_q4ks_file_mix_runs_on_the_streaming_kernel(pkg, orc):
     """The tensor mix a Q4_K_S file is said to carry (q5_K attn_v and ffn_down in the first layers) at the 8B widths,
-    two layers of which the first holds the q5_K tensors: the streaming kernel takes all-q4_K layers only, so the
-    automatic choice falls to one kernel per phase and says why; q and k share a launch, v runs in one of its own.
-    128 greedy tokens against the oracle."""
+    two layers of which the first holds the q5_K tensors: the streaming kernel takes it with typed pieces (q4_K and
+    q5_K rows next to each other in the q|k|v phase).  128 greedy tokens against the oracle, and the per-phase path
+    bit for bit.  A model the kernel cannot take (dim 3072: rows are not whole pieces) falls to one kernel per phase
+    and says why."""
     from llama2_jl_amd import synth
     kw = dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=32000, seq_len=192,
               rope_freq_base=500000.0, rope_is_neox=False)
@@ -154,7 +155,7 @@ def test_q4ks_file_mix_falls_to_path_1_with_a_reason(pkg, orc):
     assert lm.weights.layers[0].wv.type == 13 and lm.weights.layers[0].w2.type == 13 and lm.weights.layers[1].wv.type == 12
     prompt = synth.seeded_prompt(99, 32, kw["vocab_size"])
     dev = lm.device()
-    assert dev.path == 1 and "q4_K" in dev.path_reason
+    assert dev.path == 3 and dev.path_reason == ""
     om = orc.model_from_language_model(lm, nthreads=16)
     ids, logits = dev.generate_greedy(prompt, 128, want_logits=True)
     ref_ids, ref_logits = om.generate_greedy(prompt, 128, orc.GPU_SPEC)
@@ -162,8 +163,13 @@ def test_q4ks_file_mix_falls_to_path_1_with_a_reason(pkg, orc):
     assert _rel(logits, ref_logits) <= 1e-3
     dev.close()
     om.close()
-    # an all-q4_K model of the same widths takes the streaming kernel and gives no reason
-    lm2 = _model(pkg, "PLAN_Q4_K_S", 37, **dict(kw, n_layers=1))
-    dev2 = lm2.device()
-    assert dev2.path == 3 and dev2.path_reason == ""
-    dev2.close()
+    dev1 = lm.device(path=1)
+    ids1, logits1 = dev1.generate_greedy(prompt, 128, want_logits=True)
+    dev1.close()
+    assert ids1.tolist() == ids.tolist()
+    assert np.array_equal(logits1.view(np.uint32), logits.view(np.uint32))
+    lm3 = _model(pkg, "PLAN_Q4_K", 37, **dict(kw, dim=3072, hidden_dim=8192, n_heads=32, n_kv_heads=32, n_layers=1,
+                                              vocab_size=1000))
+    dev3 = lm3.device()
+    assert dev3.path == 1 and "2048" in dev3.path_reason
+    dev3.close()
