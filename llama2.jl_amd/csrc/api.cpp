@@ -767,6 +767,15 @@ static int flow_setup(l2h_model *m) {
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: its workgroups do not fit the device at once")
                         : L2H_OK;
     }
+    if (a.f32) {  // fp32 model: no streams, the kernel reads the tensors where they lie
+        const int roles[7] = {L2H_WQ, L2H_WK, L2H_WV, L2H_WO, L2H_W1, L2H_W3, L2H_W2};
+        for (int i = 0; i < 7; i++) {
+            a.f_w[i] = m->L(0, roles[i]).f32;
+            a.f_stride[i] = m->L(0, roles[i]).layer_stride / 4;
+        }
+        a.f_w[7] = m->glob[L2H_OUTPUT].f32;
+        a.f_stride[7] = 0;
+    }
     std::vector<int64_t> off;
     int64_t total = 0;
     FlowTypedTables tt;
@@ -796,15 +805,17 @@ static int flow_setup(l2h_model *m) {
         if ((rc = dalloc(m, &wt, (int64_t)tt.wave_types.size(), false))) return rc;
         HIPCHK(ctx, hipMemcpy(wt, tt.wave_types.data(), tt.wave_types.size() * 4, hipMemcpyHostToDevice));
         a.wave_types = wt;
-    } else {
+    } else if (!a.f32) {
         total = k_flow_offsets(a, cls_type, grid, off);
     }
     unsigned char *stream = nullptr;
     int64_t *off_dev = nullptr;
-    if ((rc = dalloc(m, &stream, total, false))) return rc;
-    if ((rc = dalloc(m, &off_dev, (int64_t)off.size(), false))) return rc;
-    HIPCHK(ctx, hipMemcpy(off_dev, off.data(), off.size() * 8, hipMemcpyHostToDevice));
-    for (int l = 0; l < c.n_layers; l++) {
+    if (!a.f32) {
+        if ((rc = dalloc(m, &stream, total, false))) return rc;
+        if ((rc = dalloc(m, &off_dev, (int64_t)off.size(), false))) return rc;
+        HIPCHK(ctx, hipMemcpy(off_dev, off.data(), off.size() * 8, hipMemcpyHostToDevice));
+    }
+    for (int l = 0; l < c.n_layers && !a.f32; l++) {
         const DevTensor qkv[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
         const DevTensor wo[1] = {m->L(l, L2H_WO)};
         const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
@@ -814,7 +825,7 @@ static int flow_setup(l2h_model *m) {
         HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 2, l, w13, 2, grid, cls_type, typed));
         HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 3, l, w2, 1, grid, cls_type, typed));
     }
-    HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid, cls_type, typed));
+    if (!a.f32) HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid, cls_type, typed));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
     for (void *v : tmp) HIPCHK(ctx, hipFree(v));
     a.stream = stream;

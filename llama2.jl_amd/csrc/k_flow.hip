@@ -1717,6 +1717,196 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 }
 
 // ------------------------------------------------------------------------------------------
+// models of fp32 matrices (llama2.c checkpoints, reference src/load_karpathy.jl:32-59; matmul!, src/matmul.jl:3-11):
+// the same kernel without streams.  A model of this kind is small (the largest llama2.c checkpoint is 0.4 GB) and
+// its rows are read where the tensors lie; what the one launch saves is the 40-odd launches per token.
+// Activations stay fp32 in LDS (no q8_K), products are exact in fp64 and summed in fp64, as in matvec_f32_kernel.
+// ------------------------------------------------------------------------------------------
+// the input vector of a phase -> fp32 in this workgroup's LDS; K <= 4096 and a multiple of 4
+template <int PRO, int SRC>
+__device__ __noinline__ bool flow_stage_xf(const void *src, int K, const float *normw, int tok) {
+    src = uni(src), K = uni(K), normw = uni(normw), tok = uni(tok);
+    const FlowArgs &a = c_flow;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int idx = 256 * wave + 4 * lane;
+    const bool mine = idx < K;  // (K is a multiple of 4: a lane's four words are all inside or all outside)
+    constexpr bool rms = PRO == PRO_RMSNORM;
+    float xv[4] = {0.f, 0.f, 0.f, 0.f}, wv[4] = {0.f, 0.f, 0.f, 0.f};
+    bool ok = true;
+    if (rms && mine) {
+        const float4 t = *(const float4 *)(normw + idx);
+        wv[0] = t.x, wv[1] = t.y, wv[2] = t.z, wv[3] = t.w;
+    }
+    if (SRC == SRC_EMB) {
+        if (mine)
+#pragma unroll
+            for (int k = 0; k < 4; k++) xv[k] = dequant_elem(a.emb, tok, idx + k);
+    } else {
+        unsigned spins = 0;
+        u32x4v w0 = {FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY};
+        const unsigned *pb = (const unsigned *)src + idx;
+        if (!mine) w0 = (u32x4v){0u, 0u, 0u, 0u};
+        for (;;) {
+            const bool full = w0.x != FLOW_EMPTY && w0.y != FLOW_EMPTY && w0.z != FLOW_EMPTY && w0.w != FLOW_EMPTY;
+            if (!full) POLL_BARE1(w0, pb);
+            const bool all = w0.x != FLOW_EMPTY && w0.y != FLOW_EMPTY && w0.z != FLOW_EMPTY && w0.w != FLOW_EMPTY;
+            if (__ballot(!all) == 0ull) break;
+            if (++spins > a.spin_limit ||
+                ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                ok = false;
+                break;
+            }
+        }
+        xv[0] = __uint_as_float(w0.x), xv[1] = __uint_as_float(w0.y), xv[2] = __uint_as_float(w0.z), xv[3] = __uint_as_float(w0.w);
+    }
+    if (!ok) s_flag = 1;
+    if (rms) {  // rmsnorm! (reference src/inference.jl:102-110)
+        double acc = 0.0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) acc = fma((double)xv[k], (double)xv[k], acc);
+        acc = wave_sum_f64_dpp(acc);
+        if (lane == 0) s_red[wave] = acc;
+    }
+    __syncthreads();
+    if (s_flag) {
+        if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return false;
+    }
+    if (rms) {
+        double t = 0.0;
+        for (int w = 0; w < FLOW_NW; w++) t += s_red[w];
+        float ss = (float)t;
+        ss /= (float)K;
+        ss += 1e-5f;
+        ss = 1.0f / sqrtf(ss);
+#pragma unroll
+        for (int k = 0; k < 4; k++) xv[k] = wv[k] * (ss * xv[k]);
+    }
+    if (mine) ((float4 *)s_act)[64 * wave + lane] = make_float4(xv[0], xv[1], xv[2], xv[3]);
+    __syncthreads();
+    return true;
+}
+
+// the rows of one phase for one workgroup: a wavefront takes a contiguous run of the workgroup's rows, two at a
+// time; partial sums in the layout the epilogues expect (a row is one "piece": four doubles, the sums of 16 lanes
+// each; CLS: one double per row)
+template <bool CLS>
+__device__ __forceinline__ void flow_loop_f32(const FlowGeom &g, int kind, int layer, int wg, int K) {
+    const FlowArgs &a = c_flow;
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    const float4 *x4 = (const float4 *)s_act;
+    const int n4 = K >> 2;
+    for (int i = 0; i < cnt; i += 2) {
+        const float4 *w4[2];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+            const int L = wg * g.rpw + start + min(i + r, cnt - 1);
+            int seg, row;
+            flow_row_src(CLS ? 1 : kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
+            const int wi = CLS ? 7 : (kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 + seg : 6)));
+            w4[r] = (const float4 *)(a.f_w[wi] + (CLS ? (int64_t)0 : (int64_t)layer * a.f_stride[wi]) + (int64_t)row * K);
+        }
+        double acc0 = 0.0, acc1 = 0.0;
+        for (int j = lane; j < n4; j += 64) {
+            const float4 wa = ldg_nt_f4(w4[0] + j), wb = ldg_nt_f4(w4[1] + j), xv = x4[j];
+            acc0 = fma((double)wa.x, (double)xv.x, acc0);
+            acc0 = fma((double)wa.y, (double)xv.y, acc0);
+            acc0 = fma((double)wa.z, (double)xv.z, acc0);
+            acc0 = fma((double)wa.w, (double)xv.w, acc0);
+            acc1 = fma((double)wb.x, (double)xv.x, acc1);
+            acc1 = fma((double)wb.y, (double)xv.y, acc1);
+            acc1 = fma((double)wb.z, (double)xv.z, acc1);
+            acc1 = fma((double)wb.w, (double)xv.w, acc1);
+        }
+        if (CLS) {
+            const double v0 = wave_sum_f64_dpp(acc0), v1 = wave_sum_f64_dpp(acc1);
+            if (lane == 0) {
+                s_part[start + i] = v0;
+                if (i + 1 < cnt) s_part[start + i + 1] = v1;
+            }
+        } else {
+            const double v0 = row16_sum_f64_dpp(acc0), v1 = row16_sum_f64_dpp(acc1);
+            s_part[4 * (start + i) + (lane >> 4)] = v0;
+            if (i + 1 < cnt) s_part[4 * (start + i + 1) + (lane >> 4)] = v1;
+        }
+    }
+}
+
+__global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
+    const FlowArgs &a = c_flow;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wg = blockIdx.x, nwg = gridDim.x;
+    (void)wave;
+    // ---- this step's token, position and RoPE angles (reference src/inference.jl:122-127) ----
+    const int pos = a.ctl->pos;
+    const int tok = a.ctl->step < a.ctl->n_prompt ? a.prompt[a.ctl->step] : a.ctl->last_argmax;
+    if (tid == 0) s_flag = 0;
+    if (tid < (a.hs >> 1)) {
+        float theta = 1.0f * (float)pos;
+        for (int k = 0; k < tid; k++) theta *= a.theta_scale;
+        s_rope[2 * tid] = (float)cos((double)theta);
+        s_rope[2 * tid + 1] = (float)sin((double)theta);
+    }
+    const unsigned E0 = gen0;
+    const int att_stride = nwg / a.n_heads;
+    const int att_h = uni(wg / att_stride);
+    const bool is_att = uni((int)(att_h < a.n_heads && wg % att_stride == att_h % att_stride)) != 0;
+    {
+        const int lo = wg * a.wo.rpw, n = flow_n_local(a.wo, wg);
+        if (tid < n) bare_store(a.x_a + lo + tid, bare_of(dequant_elem(a.emb, tok, lo + tid)));
+    }
+    for (int l = 0; l < a.n_layers; l++) {
+        const unsigned e_x = E0 + 5u * (unsigned)l;
+        const unsigned e_q = e_x + 1, e_att = e_x + 2, e_w13 = e_x + 4;
+#pragma nounroll
+        for (int kind = 0; kind < 4; kind++) {
+            bool ok;
+            const FlowGeom g = flow_geom(a, kind);
+            if (kind == 0) {
+                const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
+                ok = l == 0 ? flow_stage_xf<PRO_RMSNORM, SRC_EMB>(nullptr, a.dim, nw, tok)
+                            : flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, nw, tok);
+            } else if (kind == 1) {
+                if (is_att || pos >= FLOW_ATT_SHORT) {
+                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_split(l, pos, e_q, e_att)
+                                      : a.hs == 128 ? flow_attention_short<128>(l, att_h, pos, e_q, e_att)
+                                      : a.hs == 64  ? flow_attention_short<64>(l, att_h, pos, e_q, e_att)
+                                                    : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
+                    if (!uni((int)fine)) return;
+                }
+                ok = flow_stage_xf<PRO_QUANT, SRC_BARE>(a.xo + (int64_t)(e_att & 1u) * a.dim, a.dim, nullptr, tok);
+            } else if (kind == 2) {
+                ok = flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_b, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
+            } else {
+                ok = flow_stage_xf<PRO_QUANT, SRC_BARE>(a.hbw + (int64_t)(e_w13 & 1u) * a.hidden, a.hidden, nullptr, tok);
+            }
+            if (!uni(ok)) return;
+            unsigned oldw = 0;
+            if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = bare_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
+            if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
+            flow_loop_f32<false>(g, kind, l, wg, kind == 3 ? a.hidden : a.dim);
+            if (kind == 0)
+                flow_finish_qkv(l, wg, pos, e_q);
+            else if (kind == 1)
+                flow_finish_resid(1, wg, oldw);
+            else if (kind == 2)
+                flow_finish_w13(wg, e_w13);
+            else
+                flow_finish_resid(3, wg, oldw);
+        }
+    }
+    // ---- final rmsnorm (:309) + classifier (:312) ----
+    const unsigned e_fin = E0 + 5u * (unsigned)a.n_layers, e_cls = e_fin + 1;
+    if (!uni(flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, a.rms_final, tok))) return;
+    flow_loop_f32<true>(a.cls, 4, 0, wg, a.dim);
+    flow_finish_cls(wg, e_cls);
+    if (wg == 0) flow_pick_token(nwg, e_cls);
+}
+
+// ------------------------------------------------------------------------------------------
 // building the streams (once per model)
 // ------------------------------------------------------------------------------------------
 // bytes a wavefront's stream holds for one layer, and before phase `kind` within a layer
@@ -1833,7 +2023,7 @@ static FlowGeom make_geom(int64_t n_rows, int64_t K, int type, int grid) {
     int rpw = (int)((n_rows + grid - 1) / grid);
     rpw += rpw & 1;
     g.rpw = rpw;
-    g.ppr = (int)(K / 256) / (type == L2H_TYPE_Q6_K ? 16 : 8);
+    g.ppr = type == L2H_TYPE_F32 ? 1 : (int)(K / 256) / (type == L2H_TYPE_Q6_K ? 16 : 8);
     return g;
 }
 
@@ -1846,6 +2036,33 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
         return false;
     };
     a.mixed = 0;
+    a.f32 = 0;
+    {
+        bool all_f32 = cls_type == L2H_TYPE_F32;
+        for (int i = 0; i < n_layer_types; i++) all_f32 = all_f32 && layer_types[i] == L2H_TYPE_F32;
+        if (all_f32) {  // rows of fp32 weights, read where they lie: a row is one "piece"
+            if (a.dim % 4 != 0 || a.hidden % 4 != 0 || a.dim > 4096 || a.hidden > 4096)
+                return no("fp32 models: dim and hidden_dim must be multiples of 4, at most 4096");
+            if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 128)) return no("head size must be 32, 64 or 128");
+            const int G = grid / a.n_heads;
+            if (G < 1 || a.hs % G != 0 || G > 64) return no("head size must be a multiple of workgroups / heads");
+            const size_t run = (size_t)((((a.seq_len + G - 1) / G) + 63) & ~63);
+            const size_t att = (size_t)a.hs * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 + run * 4 + (size_t)a.hs * 8 + 64 * 8;
+            if (att > FLOW_ACT_BYTES) return no("sequence too long for the attention area");
+            a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim, L2H_TYPE_F32, grid);
+            a.wo = make_geom(a.dim, a.dim, L2H_TYPE_F32, grid);
+            a.w13 = make_geom(2 * (int64_t)a.hidden, a.dim, L2H_TYPE_F32, grid);
+            a.w2 = make_geom(a.dim, a.hidden, L2H_TYPE_F32, grid);
+            a.cls = make_geom(a.vocab, a.dim, L2H_TYPE_F32, grid);
+            const FlowGeom *gs[5] = {&a.qkv, &a.wo, &a.w13, &a.w2, &a.cls};
+            for (const FlowGeom *g : gs)
+                if (g->rpw > FLOW_MAX_ROWS || g->rpw > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
+                    return no("too many rows per workgroup");
+            if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
+            a.f32 = 1;
+            return true;
+        }
+    }
     for (int i = 0; i < n_layer_types; i++) {
         const int t = layer_types[i];
         if (t != L2H_TYPE_Q4_K && t != L2H_TYPE_Q5_K && t != L2H_TYPE_Q6_K) return no("layer matrices must be q4_K, q5_K or q6_K");
@@ -1978,6 +2195,7 @@ hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a) {
 // fast, not what makes it correct: workgroups that had to wait for a CU would let the others run into their
 // wait limit, and the launch would end with the error that l2h_model_set_wait_limit describes.
 static const void *flow_kernel_fn(int cls_type, bool mixed) {
+    if (cls_type == L2H_TYPE_F32) return (const void *)flow_f32_kernel;
     if (mixed)
         return cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K, true>
                                          : (const void *)flow_token_kernel<L2H_TYPE_Q4_K, true>;

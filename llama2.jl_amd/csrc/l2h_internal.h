@@ -164,6 +164,11 @@ struct FlowArgs {
     // layer matrices that are not all q4_K: typed pieces (k_flow.hip), the types of every wavefront's first pieces
     int mixed;
     const unsigned int *wave_types;  // [grid * 16]
+    // a model of fp32 matrices (llama2.c files): no streams, the rows are read where the tensors lie.
+    // f_w: wq, wk, wv, wo, w1, w3, w2 of layer 0 and the classifier; f_stride: floats from a layer's tensor to the next layer's
+    int f32;
+    const float *f_w[8];
+    int64_t f_stride[8];
 #ifdef L2H_TIMELINE
     long long *timeline;  // profiling build only: [workgroup][64] wall-clock stamps of the first phases
 #endif

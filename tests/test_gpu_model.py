@@ -150,6 +150,10 @@ FLOW_CASES = {
     "q4ks_headline_widths": ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8,
                                                  vocab_size=32000, seq_len=192, rope_freq_base=500000.0,
                                                  rope_is_neox=False)),
+    # fp32 matrices (llama2.c checkpoints): no streams, rows read where the tensors lie; hidden_dim not a multiple of 256,
+    # classifier shared with the embedding
+    "f32_rows": ("PLAN_F32", dict(dim=256, hidden_dim=344, n_layers=3, n_heads=8, n_kv_heads=4, vocab_size=500, seq_len=96,
+                                  rope_freq_base=10000.0, rope_is_neox=False)),
     # layer matrices of other types than q4_K travel as typed pieces (reference src/kquants.jl:186-408):
     # q5_K attention and up/gate, q6_K down and output
     "q5km_typed": ("PLAN_Q5_K_M", dict(dim=4096, hidden_dim=2048, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=600,
