@@ -133,8 +133,9 @@ __host__ __device__ inline int flow_ring_pieces(const FlowGeom &g, int wg, int w
 
 // logical row L of a phase -> (tensor of the phase, row in it).  Logical rows put the two rows an
 // epilogue combines next to each other: (w1 row u, w3 row u) and the two halves of a RoPE pair.
+// (any_hs: head sizes that are not powers of two)
 __host__ __device__ inline void flow_row_src(int kind, int L, int dim, int kv_dim, int hs, int neox, int &seg,
-                                             int &row) {
+                                             int &row, bool any_hs = false) {
     if (kind == 2) {  // w1 | w3
         seg = L & 1;
         row = L >> 1;
@@ -148,7 +149,7 @@ __host__ __device__ inline void flow_row_src(int kind, int L, int dim, int kv_di
     seg = L < dim ? 0 : (L < dim + kv_dim ? 1 : 2);
     row = L - (seg == 0 ? 0 : (seg == 1 ? dim : dim + kv_dim));
     if (neox && seg != 2) {  // neox pairs element i with i + hs/2 (reference src/inference.jl:146)
-        const int e = row & (hs - 1);  // hs is a power of two (32, 64 or 128)
+        const int e = any_hs ? row % hs : row & (hs - 1);  // (a power of two unless any_hs)
         row = (row - e) + (e >> 1) + ((e & 1) ? (hs >> 1) : 0);
     }
 }
@@ -952,6 +953,7 @@ __device__ __forceinline__ float flow_row_value4(int lr, int ppr) {
 // a round trip to memory that would stand between the publication of a phase's results and the next
 // phase's requests.)
 // rope! (reference src/inference.jl:112-157) and the cache append (:259-260)
+template <bool ANY_HS = false>
 __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
     l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
@@ -962,17 +964,17 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
     if (tid >= n_local) return;
     const int L = wg * a.qkv.rpw + tid;
     int seg, row;
-    flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
+    flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row, ANY_HS);
     const float val = flow_row_value4(tid, a.qkv.ppr), other = flow_row_value4(tid ^ 1, a.qkv.ppr);
-    const int hs_log = 31 - __builtin_clz(a.hs);  // a power of two
-    const int hh = row >> hs_log, e = row & (a.hs - 1);
+    const int hs_log = 31 - __builtin_clz(a.hs);  // (a power of two unless ANY_HS)
+    const int hh = ANY_HS ? row / a.hs : row >> hs_log, e = ANY_HS ? row - hh * a.hs : row & (a.hs - 1);
     if (seg == 2) {
         (a.vc + (int64_t)l * a.cache_layer_elems)[((int64_t)hh * a.seq_len + pos) * a.hs + e] = val;
         tag_store(a.vcur + row, val, e_q);
         return;
     }
     const int half = a.hs >> 1;
-    const int i = a.neox ? (e & (half - 1)) : (e >> 1);
+    const int i = a.neox ? (ANY_HS ? (e >= half ? e - half : e) : (e & (half - 1))) : (e >> 1);
     const float c = s_rope[2 * i], s = s_rope[2 * i + 1];
     const int rr = tid & 1;
     // complex product (re + i im)(c + i s), each of the four products rounded
@@ -1160,7 +1162,10 @@ template <int HS>
 __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, unsigned e_in, unsigned e_out) {
     layer = uni(layer), h = uni(h), pos = uni(pos), e_in = uni(e_in), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
-    constexpr int hs = HS, n4 = HS >> 2, ngrp = FLOW_NW * 64 / n4, per = HS >> 4, NV = FLOW_ATT_SHORT / ngrp;
+    // (values: the 16-byte groups of a row are mapped onto n4p lanes, the next power of two; lanes beyond n4 idle)
+    constexpr int hs = HS, n4 = HS >> 2, n4p = n4 <= 8 ? 8 : (n4 <= 16 ? 16 : 32), ngrp = FLOW_NW * 64 / n4p, per = HS >> 4,
+                  NV = FLOW_ATT_SHORT / ngrp;
+    static_assert(HS % 16 == 0 && HS <= 128, "head size");
     const int seq_len = a.seq_len, np = pos + 1;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
     const float *kc = a.kc + (int64_t)layer * a.cache_layer_elems;
@@ -1203,7 +1208,8 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
     // scores: lane = (timestep p16 of the wavefront's 16, quarter of the head dimension);
     // values: thread = (16-byte group i4 of the head dimension, timestep group grp), timesteps grp + u * ngrp
     const int p16 = lane & 15, part = lane >> 4, t = 16 * wave + p16;
-    const int i4 = tid & (n4 - 1), grp = tid / n4;
+    const int i4 = tid & (n4p - 1), grp = tid / n4p;
+    const bool v_lane = n4p == n4 || i4 < n4;
     float4 kv[per], v[NV];
     {
         const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
@@ -1242,8 +1248,10 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
         for (int u = 0; u < NV; u++) {
             const int tv = grp + u * ngrp;
             v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (tv < pos) v[u] = vp[(int64_t)tv * n4];
-            else if (tv == pos) v[u] = ((const float4 *)s_vcur)[i4];
+            if (v_lane) {
+                if (tv < pos) v[u] = vp[(int64_t)tv * n4];
+                else if (tv == pos) v[u] = ((const float4 *)s_vcur)[i4];
+            }
         }
         // the quarters are added in order (fp64)
         const double a1 = __shfl(acc, p16 + 16, WAVE), a2 = __shfl(acc, p16 + 32, WAVE), a3 = __shfl(acc, p16 + 48, WAVE);
@@ -1281,7 +1289,7 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
             }
         }
 #pragma unroll
-        for (int off = n4; off < 64; off <<= 1)
+        for (int off = n4p; off < 64; off <<= 1)
 #pragma unroll
             for (int c = 0; c < 4; c++) acc[c] += __shfl_xor(acc[c], off, WAVE);
         if (lane < n4) {
@@ -1463,10 +1471,12 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     const float sf = (float)tot;  // softmax!'s sum (reference src/inference.jl:169-174)
     // values: thread = (16-byte group i4 of the head dimension, timestep group), up to eight loads in flight; the
     // groups of one wavefront are folded with lane exchanges, the rest through LDS
-    const int n4 = hs >> 2;  // a power of two (hs 32, 64, 128)
-    const int ngrp = blockDim.x / n4;
+    // (the 16-byte groups of a row are mapped onto n4p lanes, the next power of two; lanes beyond n4 idle)
+    const int n4 = hs >> 2, n4p = n4 <= 8 ? 8 : (n4 <= 16 ? 16 : 32);
+    const int ngrp = blockDim.x / n4p;
     {
-        const int i4 = tid & (n4 - 1), grp = tid / n4;
+        const int i4 = tid & (n4p - 1), grp = tid / n4p;
+        const bool v_lane = i4 < n4;
         const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
         double acc[4] = {0.0, 0.0, 0.0, 0.0};
         for (int t0 = lo + grp; t0 < hi; t0 += 8 * ngrp) {
@@ -1475,7 +1485,7 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
             for (int u = 0; u < 8; u++) {
                 const int t = t0 + u * ngrp;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (t < hi) v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : vp[(int64_t)t * n4];
+                if (t < hi && v_lane) v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : vp[(int64_t)t * n4];
             }
 #pragma unroll
             for (int u = 0; u < 8; u++) {
@@ -1489,7 +1499,7 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                 }
             }
         }
-        for (int off = n4; off < 64; off <<= 1)
+        for (int off = n4p; off < 64; off <<= 1)
 #pragma unroll
             for (int c = 0; c < 4; c++) acc[c] += __shfl_xor(acc[c], off, WAVE);
         if ((tid & 63) < n4) {
@@ -1643,6 +1653,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                 // (a long cache is shared by all the workgroups of a head, a short one read by one of them)
                 if (is_att || pos >= FLOW_ATT_SHORT) {
                     const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_split(l, pos, e_q, e_att)
+                                      : (MIXED && a.hs == 96) ? flow_attention_short<96>(l, att_h, pos, e_q, e_att)
                                       : a.hs == 128 ? flow_attention_short<128>(l, att_h, pos, e_q, e_att)
                                       : a.hs == 64  ? flow_attention_short<64>(l, att_h, pos, e_q, e_att)
                                                     : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
@@ -1671,14 +1682,24 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                 flow_reg_arrived(rp);
             FTL();
             if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
-            if constexpr (MIXED)
+            if constexpr (MIXED) {
+                // rows of dim inputs padded to whole pieces: the q8_K blocks beyond dim are zero (d = 0, no quants)
+                if (kind != 3 && a.dim_pad > a.dim) {
+                    const int b0 = a.dim >> 8, nbz = (a.dim_pad - a.dim) >> 8;
+                    unsigned char *q8 = (unsigned char *)s_act;
+                    for (int i = tid; i < nbz * 64; i += 1024) ((uint32_t *)(q8 + 256 * b0))[i] = 0u;
+                    if (tid < nbz * 8) ((uint32_t *)(q8 + 14336 + 32 * b0))[tid] = 0u;
+                    if (tid < nbz) ((float *)(q8 + 14336 + 1792))[b0 + tid] = 0.f;
+                    __syncthreads();
+                }
                 flow_loop_mixed(g, mr, mring_base, wg);
-            else
+            } else {
                 flow_loop_q4<true, true>(g, r, ring_base, wg, rp, n_reg);
+            }
             FTL();
             FTLS();
             if (kind == 0)
-                flow_finish_qkv(l, wg, pos, e_q);
+                flow_finish_qkv<MIXED>(l, wg, pos, e_q);
             else if (kind == 1)
                 flow_finish_resid(1, wg, oldw);
             else if (kind == 2)
@@ -1705,6 +1726,14 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             flow_top_up_q4(r, ring_base, lane);
     }
     if (!uni(flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, a.rms_final, tok))) LEAVE();
+    if (MIXED && a.dim_pad > a.dim) {
+        const int b0 = a.dim >> 8, nbz = (a.dim_pad - a.dim) >> 8;
+        unsigned char *q8 = (unsigned char *)s_act;
+        for (int i = tid; i < nbz * 64; i += 1024) ((uint32_t *)(q8 + 256 * b0))[i] = 0u;
+        if (tid < nbz * 8) ((uint32_t *)(q8 + 14336 + 32 * b0))[tid] = 0u;
+        if (tid < nbz) ((float *)(q8 + 14336 + 1792))[b0 + tid] = 0.f;
+        __syncthreads();
+    }
     flow_drain(r);
     if (T_CLS == L2H_TYPE_Q6_K)
         flow_loop_q6(a.cls, r, ring_base, wg);
@@ -1952,7 +1981,7 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
     const int L = wg * g.rpw + j / g.ppr;
     const int part = j % g.ppr;
     int seg, row32;
-    flow_row_src(p.kind == 4 ? 1 : p.kind, L, p.dim, p.kv_dim, p.hs, p.neox, seg, row32);
+    flow_row_src(p.kind == 4 ? 1 : p.kind, L, p.dim, p.kv_dim, p.hs, p.neox, seg, row32, true);
     const int64_t row = row32;
     const DevTensor &t = seg == 0 ? p.w[0] : (seg == 1 ? p.w[1] : p.w[2]);
     const int64_t layer_b = flow_layer_bytes(p.g4, wg, wave, 4);
@@ -1968,19 +1997,28 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
         const int64_t e = p.typed.piece_base[wg * FLOW_NW + wave] + (int64_t)p.layer * per_layer + before + idx;
         uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + p.typed.piece_off[e]);
         const int64_t blk0 = row * t.nb + part * 8;
+        // super-blocks of the piece that the row has (fewer than 8 where the row is padded to whole pieces: the
+        // others are written as zeros, d = 0)
+        const int nbv = (int)min((int64_t)8, max((int64_t)0, t.nb - (int64_t)part * 8));
+        const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
         if (lane == 0) dst[8] = make_uint4((uint32_t)p.typed.piece_tag[e], 0u, 0u, 0u);
         if (t.type == L2H_TYPE_Q4_K) {
-            if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
-            dst[9 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+            if (lane < 8) dst[lane] = lane < nbv ? flow_encode_hdr(t.hdr[blk0 + lane]) : z4;
+            dst[9 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
         } else if (t.type == L2H_TYPE_Q5_K) {
-            if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
-            if (lane < 16) dst[9 + lane] = ((const uint4 *)(t.qh + blk0 * 32))[lane];
-            dst[25 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+            if (lane < 8) dst[lane] = lane < nbv ? flow_encode_hdr(t.hdr[blk0 + lane]) : z4;
+            if (lane < 16) dst[9 + lane] = (lane >> 1) < nbv ? ((const uint4 *)(t.qh + blk0 * 32))[lane] : z4;
+            dst[25 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
         } else {  // q6_K
-            if (lane < 8) dst[lane] = ((const uint4 *)(t.sc6 + blk0 * 4))[lane];
-            if (lane == 1) dst[9] = ((const uint4 *)(t.d6 + blk0))[0];
-            if (lane < 32) dst[10 + lane] = ((const uint4 *)(t.qh + blk0 * 64))[lane];
-            dst[42 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+            if (lane < 8) dst[lane] = lane < nbv ? ((const uint4 *)(t.sc6 + blk0 * 4))[lane] : z4;
+            if (lane == 1) {
+                uint16_t dd[8];
+                for (int b = 0; b < 8; b++) dd[b] = b < nbv ? t.d6[blk0 + b] : (uint16_t)0;
+                dst[9] = make_uint4(dd[0] | (uint32_t)dd[1] << 16, dd[2] | (uint32_t)dd[3] << 16, dd[4] | (uint32_t)dd[5] << 16,
+                                    dd[6] | (uint32_t)dd[7] << 16);
+            }
+            if (lane < 32) dst[10 + lane] = (lane >> 2) < nbv ? ((const uint4 *)(t.qh + blk0 * 64))[lane] : z4;
+            dst[42 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
         }
         return;
     }
@@ -1998,18 +2036,27 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
         }
         uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + off + (int64_t)at * FLOW_SLOT);
         const int64_t blk0 = row * t.nb + part * 8;
-        if (lane < 8) dst[lane] = flow_encode_hdr(t.hdr[blk0 + lane]);
-        dst[8 + lane] = ((const uint4 *)(t.qs + blk0 * 128))[lane];
+        const int nbv = (int)min((int64_t)8, max((int64_t)0, t.nb - (int64_t)part * 8));  // (8 unless the row is padded)
+        const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
+        if (lane < 8) dst[lane] = lane < nbv ? flow_encode_hdr(t.hdr[blk0 + lane]) : z4;
+        dst[8 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
     } else {  // q6_K classifier
         const int64_t off = cls_at;
         uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + off + (int64_t)idx * FLOW_Q6_PIECE);
         const int64_t blk0 = row * t.nb + part * 16;
+        const int nbv = (int)min((int64_t)16, max((int64_t)0, t.nb - (int64_t)part * 16));  // (16 unless the row is padded)
+        const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
         const uint4 *ql = (const uint4 *)(t.qs + blk0 * 128), *qh = (const uint4 *)(t.qh + blk0 * 64);
-        dst[lane] = ql[lane];
-        dst[64 + lane] = ql[64 + lane];
-        dst[128 + lane] = qh[lane];
-        if (lane < 16) dst[192 + lane] = ((const uint4 *)(t.sc6 + blk0 * 4))[lane];
-        if (lane < 2) dst[208 + lane] = ((const uint4 *)(t.d6 + blk0))[lane];
+        dst[lane] = (lane >> 3) < nbv ? ql[lane] : z4;
+        dst[64 + lane] = 8 + (lane >> 3) < nbv ? ql[64 + lane] : z4;
+        dst[128 + lane] = (lane >> 2) < nbv ? qh[lane] : z4;
+        if (lane < 16) dst[192 + lane] = lane < nbv ? ((const uint4 *)(t.sc6 + blk0 * 4))[lane] : z4;
+        if (lane < 2) {
+            uint16_t dd[8];
+            for (int b = 0; b < 8; b++) dd[b] = 8 * lane + b < nbv ? t.d6[blk0 + 8 * lane + b] : (uint16_t)0;
+            dst[208 + lane] = make_uint4(dd[0] | (uint32_t)dd[1] << 16, dd[2] | (uint32_t)dd[3] << 16,
+                                         dd[4] | (uint32_t)dd[5] << 16, dd[6] | (uint32_t)dd[7] << 16);
+        }
     }
 }
 
@@ -2060,6 +2107,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
                     return no("too many rows per workgroup");
             if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
             a.f32 = 1;
+            a.dim_pad = a.dim;
             return true;
         }
     }
@@ -2071,21 +2119,27 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     for (int l = 0; l * 7 + 6 < n_layer_types; l++)  // (w1 and w3 rows alternate within a workgroup's pieces)
         if (layer_types[l * 7 + 4] != layer_types[l * 7 + 6]) return no("w1 and w3 of a layer must have one type");
     if (cls_type != L2H_TYPE_Q4_K && cls_type != L2H_TYPE_Q6_K) return no("classifier must be q4_K or q6_K");
-    if (a.dim % 2048 != 0 || a.hidden % 2048 != 0) return no("dim and hidden_dim must be multiples of 2048");
-    if (cls_type == L2H_TYPE_Q6_K && a.dim % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
-    if (a.hidden > 14336 || a.dim > 4096) return no("dim above 4096 or hidden_dim above 14336");
-    if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 128)) return no("head size must be 32, 64 or 128");
+    // rows of dim inputs may be padded with zero super-blocks to whole pieces if that adds a third at most (dim 3072
+    // -> 4096); such a model, and one with head size 96, runs as typed pieces
+    a.dim_pad = (a.dim + 2047) / 2048 * 2048;
+    if (a.dim % 256 != 0 || (int64_t)a.dim * 4 < (int64_t)a.dim_pad * 3 || a.hidden % 2048 != 0)
+        return no("dim must be a multiple of 2048 (or of 256 and within a quarter below one), hidden_dim a multiple of 2048");
+    if (a.dim_pad != a.dim) a.mixed = 1;
+    if (cls_type == L2H_TYPE_Q6_K && a.dim_pad % 4096 != 0) return no("a q6_K classifier needs dim to be a multiple of 4096");
+    if (a.hidden > 14336 || a.dim_pad > 4096) return no("dim above 4096 or hidden_dim above 14336");
+    if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 96 && a.hs != 128)) return no("head size must be 32, 64, 96 or 128");
+    if (a.hs == 96) a.mixed = 1;
     // the split attention of long caches: q, the partial sums, one member's run of scores, k and v of the position, G numbers
     const int G = grid / a.n_heads;
     if (G < 1 || a.hs % G != 0 || G > 64) return no("head size must be a multiple of workgroups / heads");
     const size_t run = (size_t)((((a.seq_len + G - 1) / G) + 63) & ~63);
     const size_t att = (size_t)a.hs * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 + run * 4 + (size_t)a.hs * 8 + 64 * 8;
     if (att > FLOW_ACT_BYTES) return no("sequence too long for the attention area");
-    a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim, L2H_TYPE_Q4_K, grid);
-    a.wo = make_geom(a.dim, a.dim, L2H_TYPE_Q4_K, grid);
-    a.w13 = make_geom(2 * (int64_t)a.hidden, a.dim, L2H_TYPE_Q4_K, grid);
+    a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim_pad, L2H_TYPE_Q4_K, grid);
+    a.wo = make_geom(a.dim, a.dim_pad, L2H_TYPE_Q4_K, grid);
+    a.w13 = make_geom(2 * (int64_t)a.hidden, a.dim_pad, L2H_TYPE_Q4_K, grid);
     a.w2 = make_geom(a.dim, a.hidden, L2H_TYPE_Q4_K, grid);
-    a.cls = make_geom(a.vocab, a.dim, cls_type, grid);
+    a.cls = make_geom(a.vocab, a.dim_pad, cls_type, grid);
     const FlowGeom *gs[5] = {&a.qkv, &a.wo, &a.w13, &a.w2, &a.cls};
     for (const FlowGeom *g : gs)
         if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
@@ -2136,7 +2190,7 @@ void k_flow_typed_tables(const FlowArgs &a, const int *layer_types, int cls_type
                     for (int i = 0; i < cnt; i++) {
                         const int L = wg * g.rpw + (start + i) / g.ppr;
                         int seg, row;
-                        flow_row_src(kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
+                        flow_row_src(kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row, true);
                         const int slot = kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 : 5));
                         const int ty = layer_types[l * 7 + slot] - L2H_TYPE_Q4_K;
                         t.piece_off.push_back(off);

@@ -150,6 +150,10 @@ FLOW_CASES = {
     "q4ks_headline_widths": ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8,
                                                  vocab_size=32000, seq_len=192, rope_freq_base=500000.0,
                                                  rope_is_neox=False)),
+    # the Phi-3 shape: dim 3072 is 1.5 pieces per row (rows padded with zero super-blocks to 4096 in the streams), head
+    # size 96 is not a power of two, neox RoPE, no GQA
+    "phi3_widths": ("PLAN_Q4_K", dict(dim=3072, hidden_dim=2048, n_layers=2, n_heads=32, n_kv_heads=32, vocab_size=512,
+                                      seq_len=128, rope_freq_base=10000.0, rope_is_neox=True)),
     # fp32 matrices (llama2.c checkpoints): no streams, rows read where the tensors lie; hidden_dim not a multiple of 256,
     # classifier shared with the embedding
     "f32_rows": ("PLAN_F32", dict(dim=256, hidden_dim=344, n_layers=3, n_heads=8, n_kv_heads=4, vocab_size=500, seq_len=96,
@@ -266,7 +270,8 @@ def test_kv_prefill_and_long_context(pkg, orc, rng, path, seq_len):
 
 @pytest.mark.parametrize("case,n_pre,seq_len", [("all_q4", 250, 384), ("all_q4", 300, 384), ("all_q4", 1500, 1600),
                                                 ("all_q4_neox", 1000, 1100), ("q4ks_headline_widths", 2100, 4096),
-                                                ("q4ks_headline_widths", 4070, 4096)])
+                                                ("q4ks_headline_widths", 4070, 4096), ("phi3_widths", 700, 800),
+                                                ("q5km_typed", 900, 1024)])
 def test_streaming_kernel_long_cache(pkg, orc, rng, case, n_pre, seq_len):
     """Path 3 decoding into a pre-filled cache: from 250 the run crosses position 256, where the kernel
     changes from its short-cache attention (one workgroup per head) to the one in which all workgroups of a

@@ -145,8 +145,8 @@ def test_q4ks_file_mix_runs_on_the_streaming_kernel(pkg, orc):
     """The tensor mix a Q4_K_S file is said to carry (q5_K attn_v and ffn_down in the first layers) at the 8B widths,
     two layers of which the first holds the q5_K tensors: the streaming kernel takes it with typed pieces (q4_K and
     q5_K rows next to each other in the q|k|v phase).  128 greedy tokens against the oracle, and the per-phase path
-    bit for bit.  A model the kernel cannot take (dim 3072: rows are not whole pieces) falls to one kernel per phase
-    and says why."""
+    bit for bit.  A model the kernel cannot take (dim 1024: rows are half a piece) falls to one kernel per
+    phase and says why."""
     from llama2_jl_amd import synth
     kw = dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=32000, seq_len=192,
               rope_freq_base=500000.0, rope_is_neox=False)
@@ -168,7 +168,7 @@ def test_q4ks_file_mix_runs_on_the_streaming_kernel(pkg, orc):
     dev1.close()
     assert ids1.tolist() == ids.tolist()
     assert np.array_equal(logits1.view(np.uint32), logits.view(np.uint32))
-    lm3 = _model(pkg, "PLAN_Q4_K", 37, **dict(kw, dim=3072, hidden_dim=8192, n_heads=32, n_kv_heads=32, n_layers=1,
+    lm3 = _model(pkg, "PLAN_Q4_K", 37, **dict(kw, dim=1024, hidden_dim=4096, n_heads=8, n_kv_heads=8, n_layers=1,
                                               vocab_size=1000))
     dev3 = lm3.device()
     assert dev3.path == 1 and "2048" in dev3.path_reason
