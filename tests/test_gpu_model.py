@@ -429,24 +429,27 @@ def test_full_size_model_launch_paths_agree(pkg):
     assert np.array_equal(got[1][1], got[3][1])
 
 
-def test_streaming_kernel_soak_against_per_phase_path(pkg):
+@pytest.mark.parametrize("case,reps,n_new", [("q4ks_headline_widths", 30, 128), ("q5km_typed", 12, 60),
+                                             ("all_types_typed", 12, 60), ("phi3_widths", 12, 80), ("f32_rows", 12, 60)])
+def test_streaming_kernel_soak_against_per_phase_path(pkg, case, reps, n_new):
     """The streaming kernel's exchange of activations between workgroups rests on timing-independent
-    reasoning (every buffer is rewritten two phases after its last read); this repeats it: 30 generations of
-    128 tokens at the benchmark's widths (two layers), different prompts, each compared bit for bit (tokens
-    and final logits) with the per-phase path, stopping at the first difference or error."""
+    reasoning (every buffer is rewritten two phases after its last read); this repeats it: generations of
+    up to 128 tokens (30 of them at the benchmark's widths, two layers; a dozen for each other form of the
+    kernel: typed pieces, padded rows with head size 96, fp32 rows), different prompts, each compared bit for
+    bit (tokens and final logits) with the per-phase path, stopping at the first difference or error."""
     from llama2_jl_amd import synth
     from llama2_jl_amd.inference import DeviceModel
-    plan, kw = FLOW_CASES["q4ks_headline_widths"]
+    plan, kw = FLOW_CASES[case]
     lm = _model(pkg, plan, **kw)
     fast = DeviceModel(lm.config, lm.weights, path=3)
     slow = DeviceModel(lm.config, lm.weights, path=1)
     assert fast.path == 3 and slow.path == 1
-    for rep in range(30):
-        prompt = synth.seeded_prompt(1000 + rep, 1 + rep % 40, kw["vocab_size"])
+    for rep in range(reps):
+        prompt = synth.seeded_prompt(1000 + rep, 1 + rep % (40 if n_new == 128 else 20), kw["vocab_size"])
         fast.reset()
         slow.reset()
-        a_ids, a_logits = fast.generate_greedy(prompt, 128, want_logits=True)
-        b_ids, b_logits = slow.generate_greedy(prompt, 128, want_logits=True)
+        a_ids, a_logits = fast.generate_greedy(prompt, n_new, want_logits=True)
+        b_ids, b_logits = slow.generate_greedy(prompt, n_new, want_logits=True)
         assert np.asarray(a_ids).tolist() == np.asarray(b_ids).tolist(), rep
         assert np.array_equal(a_logits.view(np.uint32), b_logits.view(np.uint32)), rep
     fast.close()
