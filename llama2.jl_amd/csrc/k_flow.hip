@@ -1469,7 +1469,8 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     double tot = 0.0;
     for (int k = 0; k < G; k++) tot += s_x[k];
     const float sf = (float)tot;  // softmax!'s sum (reference src/inference.jl:169-174)
-    // values: thread = (16-byte group i4 of the head dimension, timestep group), up to eight loads in flight; the
+    // values: thread = (16-byte group i4 of the head dimension, timestep group), four loads in flight (with eight the
+    // function needs callee-saved registers, and saving them to scratch costs more than the deeper loads gain); the
     // groups of one wavefront are folded with lane exchanges, the rest through LDS
     // (the 16-byte groups of a row are mapped onto n4p lanes, the next power of two; lanes beyond n4 idle)
     const int n4 = hs >> 2, n4p = n4 <= 8 ? 8 : (n4 <= 16 ? 16 : 32);
@@ -1479,16 +1480,16 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         const bool v_lane = i4 < n4;
         const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
         double acc[4] = {0.0, 0.0, 0.0, 0.0};
-        for (int t0 = lo + grp; t0 < hi; t0 += 8 * ngrp) {
-            float4 v[8];
+        for (int t0 = lo + grp; t0 < hi; t0 += 4 * ngrp) {
+            float4 v[4];
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < 4; u++) {
                 const int t = t0 + u * ngrp;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (t < hi && v_lane) v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : vp[(int64_t)t * n4];
             }
 #pragma unroll
-            for (int u = 0; u < 8; u++) {
+            for (int u = 0; u < 4; u++) {
                 const int t = t0 + u * ngrp;
                 if (t < hi) {
                     const double p = (double)(s_att[t - lo] / sf);
