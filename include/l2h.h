@@ -93,7 +93,8 @@ int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t 
  * reference: the rows appended by transformer! (and those passed to l2h_kv_write) are rounded to binary16
  * (nearest even) and widened again when the attention reads them, so a decode step reads half the cache
  * bytes; everything else computes as before.  Needs a head size that is a multiple of 32, at most 128; runs
- * on launch path 1; l2h_prefill is not available (L2H_ESTATE).  l2h_kv_read returns the rounded values. */
+ * on launch paths 1 and 3 (not 2); l2h_prefill is not available (L2H_ESTATE).  l2h_kv_read returns the
+ * rounded values. */
 enum { L2H_KV_F32 = 0, L2H_KV_F16 = 1 };
 int l2h_model_set_kv_type(l2h_model *m, int kv_type);
 /* How transformer! is launched (before finalize): 0 = automatic (3 where the model fits it, else 1),

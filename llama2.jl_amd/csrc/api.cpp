@@ -411,7 +411,6 @@ extern "C" int l2h_model_set_path(l2h_model *m, int path) {
 
 extern "C" const char *l2h_model_path_reason(l2h_model *m) {
     if (!m || !m->finalized) return "";
-    if (m->kv16) return "an fp16 KV cache runs on launch path 1";
     return m->flow_why.c_str();
 }
 
@@ -748,6 +747,7 @@ static int flow_setup(l2h_model *m) {
     a.vocab = c.vocab_size;
     a.neox = c.rope_is_neox;
     a.theta_scale = m->theta_scale;
+    a.kv16 = m->kv16;
     std::vector<int> types;
     for (int l = 0; l < c.n_layers; l++)
         for (int r : {L2H_WQ, L2H_WK, L2H_WV, L2H_WO, L2H_W1, L2H_W2, L2H_W3}) types.push_back(m->L(l, r).type);
@@ -974,9 +974,7 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     if (m->kv16) {
         if (m->hs > 128 || m->hs % 32 != 0)
             return set_err(ctx, L2H_EINVAL, "an fp16 KV cache needs a head size that is a multiple of 32, at most 128");
-        if (m->path_request == 2 || m->path_request == 3)
-            return set_err(ctx, L2H_EINVAL, "an fp16 KV cache runs on launch path 1 only");
-        m->path_request = 1;
+        if (m->path_request == 2) return set_err(ctx, L2H_EINVAL, "an fp16 KV cache does not run on launch path 2");
     }
     // (an fp16 cache takes half the floats)
     DA(m->kc, m->cache_layer_elems * c.n_layers / (m->kv16 ? 2 : 1) + 1, true);

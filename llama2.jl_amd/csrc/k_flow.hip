@@ -969,6 +969,12 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
     const int hs_log = 31 - __builtin_clz(a.hs);  // (a power of two unless ANY_HS)
     const int hh = ANY_HS ? row / a.hs : row >> hs_log, e = ANY_HS ? row - hh * a.hs : row & (a.hs - 1);
     if (seg == 2) {
+        if (ANY_HS && a.kv16) {  // fp16 cache: the row is rounded on append, and the attention sees the rounded value
+            const __half hv = __float2half_rn(val);
+            ((__half *)a.vc + (int64_t)l * a.cache_layer_elems)[((int64_t)hh * a.seq_len + pos) * a.hs + e] = hv;
+            tag_store(a.vcur + row, __half2float(hv), e_q);
+            return;
+        }
         (a.vc + (int64_t)l * a.cache_layer_elems)[((int64_t)hh * a.seq_len + pos) * a.hs + e] = val;
         tag_store(a.vcur + row, val, e_q);
         return;
@@ -982,6 +988,10 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
     const float out = rr == 0 ? (re * c) - (im * s) : (re * s) + (im * c);
     if (seg == 0) {
         tag_store(a.q + row, out, e_q);
+    } else if (ANY_HS && a.kv16) {
+        const __half hv = __float2half_rn(out);
+        ((__half *)a.kc + (int64_t)l * a.cache_layer_elems)[kc16_index(hh, e, pos, a.hs, a.seq_len)] = hv;
+        tag_store(a.kcur + row, __half2float(hv), e_q);
     } else {
         (a.kc + (int64_t)l * a.cache_layer_elems)[(((int64_t)hh * (a.hs >> 2) + (e >> 2)) * a.seq_len + pos) * 4 + (e & 3)] = out;
         tag_store(a.kcur + row, out, e_q);
@@ -1339,6 +1349,9 @@ __device__ __forceinline__ double tag_wait_f64(const u64 *p, unsigned epoch, boo
     return __longlong_as_double((long long)(((unsigned long long)(unsigned)hi << 32) | (unsigned long long)(unsigned)lo));
 }
 
+// H16: the cache holds fp16 elements (K as [n_kv][hs/8][seq_len][8], V rows of hs halves): a lane reads eight
+// elements per 16-byte load; hs is then a multiple of 32.
+template <bool H16>
 __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e_in, unsigned e_out) {
     layer = uni(layer), pos = uni(pos), e_in = uni(e_in), e_out = uni(e_out);
     const FlowArgs &a = c_flow;
@@ -1347,8 +1360,8 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     if (h >= a.n_heads) return true;
     const int hs = a.hs, seq_len = a.seq_len, np = pos + 1;
     const int kvh = h / (a.n_heads / a.n_kv_heads);
-    const float *kc = a.kc + (int64_t)layer * a.cache_layer_elems;
-    const float *vc = a.vc + (int64_t)layer * a.cache_layer_elems;
+    const float *kc = (const float *)((const char *)a.kc + (int64_t)layer * a.cache_layer_elems * (H16 ? 2 : 4));
+    const float *vc = (const float *)((const char *)a.vc + (int64_t)layer * a.cache_layer_elems * (H16 ? 2 : 4));
     // this member's run of timesteps [lo, hi): runs are multiples of 64 long, the last members' may be empty
     const int C = (((np + G - 1) / G) + 63) & ~63;
     const int lo = min(np, j * C), hi = min(np, lo + C), nj = hi - lo;
@@ -1405,7 +1418,31 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         for (int t0 = lo; t0 < hi; t0 += 256) {
             const int t = t0 + tl;
             double acc = 0.0;
-            if (t < hi) {
+            if (H16) {
+                if (t < hi) {
+                    const int per8 = hs >> 5;  // 16-byte groups of eight elements per quarter
+                    const int64_t kg = ((int64_t)kvh * (hs >> 3) + part * per8) * seq_len + t;
+                    const float *kl = s_kcur + part * (hs >> 2);
+                    Half8 kv[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        if (u < per8) {
+                            if (t == pos) {
+#pragma unroll
+                                for (int c = 0; c < 8; c++) kv[u].v[c] = kl[8 * u + c];
+                            } else {
+                                kv[u] = ldg_nt_h8(kc, kg + (int64_t)u * seq_len);
+                            }
+                        }
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        if (u < per8) {
+                            const double *qq = s_q + part * (hs >> 2) + 8 * u;
+#pragma unroll
+                            for (int c = 0; c < 8; c++) acc = fma(qq[c], (double)kv[u].v[c], acc);
+                        }
+                }
+            } else if (t < hi) {
                 const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
                 const float4 *kl = (const float4 *)s_kcur + part * per;
                 float4 kv[8];
@@ -1475,7 +1512,48 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     // (the 16-byte groups of a row are mapped onto n4p lanes, the next power of two; lanes beyond n4 idle)
     const int n4 = hs >> 2, n4p = n4 <= 8 ? 8 : (n4 <= 16 ? 16 : 32);
     const int ngrp = blockDim.x / n4p;
-    {
+    if (H16) {
+        // thread = (group i8 of eight head dimensions, timestep group of 64); four loads in flight
+        const int n8 = hs >> 3, i8 = tid & 15, grp = tid >> 4, ng = blockDim.x >> 4;
+        const bool v_lane = i8 < n8;
+        double acc[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
+        for (int t0 = lo + grp; t0 < hi; t0 += 4 * ng) {
+            Half8 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int t = t0 + u * ng;
+#pragma unroll
+                for (int c = 0; c < 8; c++) v[u].v[c] = 0.f;
+                if (t < hi && v_lane) {
+                    if (t == pos) {
+#pragma unroll
+                        for (int c = 0; c < 8; c++) v[u].v[c] = s_vcur[8 * i8 + c];
+                    } else {
+                        v[u] = ldg_nt_h8(vc, ((int64_t)kvh * seq_len + t) * n8 + i8);
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int t = t0 + u * ng;
+                if (t < hi) {
+                    const double p = (double)(s_att[t - lo] / sf);
+#pragma unroll
+                    for (int c = 0; c < 8; c++) acc[c] = fma(p, (double)v[u].v[c], acc[c]);
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            acc[c] += __shfl_xor(acc[c], 16, WAVE);
+            acc[c] += __shfl_xor(acc[c], 32, WAVE);
+        }
+        if ((tid & 63) < n8) {
+            const int wv = tid >> 6;
+#pragma unroll
+            for (int c = 0; c < 8; c++) s_r[wv * hs + 8 * i8 + c] = acc[c];
+        }
+    } else {
         const int i4 = tid & (n4p - 1), grp = tid / n4p;
         const bool v_lane = i4 < n4;
         const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
@@ -1652,8 +1730,9 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                             : flow_stage<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, nw, tok);
             } else if (kind == 1) {
                 // (a long cache is shared by all the workgroups of a head, a short one read by one of them)
-                if (is_att || pos >= FLOW_ATT_SHORT) {
-                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_split(l, pos, e_q, e_att)
+                if (is_att || pos >= FLOW_ATT_SHORT || (MIXED && a.kv16)) {
+                    const bool fine = (MIXED && a.kv16) ? flow_attention_split<true>(l, pos, e_q, e_att)
+                                      : pos >= FLOW_ATT_SHORT ? flow_attention_split<false>(l, pos, e_q, e_att)
                                       : (MIXED && a.hs == 96) ? flow_attention_short<96>(l, att_h, pos, e_q, e_att)
                                       : a.hs == 128 ? flow_attention_short<128>(l, att_h, pos, e_q, e_att)
                                       : a.hs == 64  ? flow_attention_short<64>(l, att_h, pos, e_q, e_att)
@@ -1682,7 +1761,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             else
                 flow_reg_arrived(rp);
             FTL();
-            if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
+            if (kind == 0 && is_att && pos < FLOW_ATT_SHORT && !(MIXED && a.kv16)) flow_touch_cache(l, att_h, pos);
             if constexpr (MIXED) {
                 // rows of dim inputs padded to whole pieces: the q8_K blocks beyond dim are zero (d = 0, no quants)
                 if (kind != 3 && a.dim_pad > a.dim) {
@@ -1901,7 +1980,7 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
                             : flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, nw, tok);
             } else if (kind == 1) {
                 if (is_att || pos >= FLOW_ATT_SHORT) {
-                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_split(l, pos, e_q, e_att)
+                    const bool fine = pos >= FLOW_ATT_SHORT ? flow_attention_split<false>(l, pos, e_q, e_att)
                                       : a.hs == 128 ? flow_attention_short<128>(l, att_h, pos, e_q, e_att)
                                       : a.hs == 64  ? flow_attention_short<64>(l, att_h, pos, e_q, e_att)
                                                     : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
@@ -2088,6 +2167,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     {
         bool all_f32 = cls_type == L2H_TYPE_F32;
         for (int i = 0; i < n_layer_types; i++) all_f32 = all_f32 && layer_types[i] == L2H_TYPE_F32;
+        if (all_f32 && a.kv16) return no("fp32 models keep an fp32 cache in this kernel");
         if (all_f32) {  // rows of fp32 weights, read where they lie: a row is one "piece"
             if (a.dim % 4 != 0 || a.hidden % 4 != 0 || a.dim > 4096 || a.hidden > 4096)
                 return no("fp32 models: dim and hidden_dim must be multiples of 4, at most 4096");
@@ -2130,6 +2210,10 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     if (a.hidden > 14336 || a.dim_pad > 4096) return no("dim above 4096 or hidden_dim above 14336");
     if (a.n_heads > grid || (a.hs != 32 && a.hs != 64 && a.hs != 96 && a.hs != 128)) return no("head size must be 32, 64, 96 or 128");
     if (a.hs == 96) a.mixed = 1;
+    if (a.kv16) {  // (set by the caller) the fp16 cache is read by the typed-piece instantiation's attention only
+        if (a.hs % 32 != 0) return no("an fp16 cache needs a head size that is a multiple of 32");
+        a.mixed = 1;
+    }
     // the split attention of long caches: q, the partial sums, one member's run of scores, k and v of the position, G numbers
     const int G = grid / a.n_heads;
     if (G < 1 || a.hs % G != 0 || G > 64) return no("head size must be a multiple of workgroups / heads");

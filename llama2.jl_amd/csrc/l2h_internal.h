@@ -159,6 +159,7 @@ struct FlowArgs {
     unsigned int gen0, spin_limit;
     unsigned int *abort_flag;
     int dim, hidden, hs, n_heads, n_kv_heads, kv_dim, seq_len, n_layers, vocab, neox;
+    int kv16;     // the KV cache holds fp16 elements (typed-piece instantiation of the kernel only)
     int dim_pad;  // dim rounded up to whole pieces (2048): rows of dim inputs are padded with zero super-blocks in the streams
     float theta_scale;
     FlowGeom qkv, wo, w13, w2, cls;

@@ -30,6 +30,14 @@ CASES = {
                                   rope_freq_base=10000.0, rope_is_neox=False)),
     "q5km_long": ("PLAN_Q5_K_M", dict(dim=512, hidden_dim=768, n_layers=2, n_heads=8, n_kv_heads=2, vocab_size=600,
                                       seq_len=1280, rope_freq_base=10000.0, rope_is_neox=False)),
+    # shapes that the streaming kernel takes (launch path 3): its long-cache attention reads the fp16 cache at every
+    # position; head sizes 128 with GQA, 96 (the Phi-3 widths) and 64
+    "flow_q4_hs128": ("PLAN_Q4_K", dict(dim=2048, hidden_dim=2048, n_layers=2, n_heads=16, n_kv_heads=4, vocab_size=600,
+                                        seq_len=128, rope_freq_base=500000.0, rope_is_neox=False)),
+    "flow_phi3_hs96": ("PLAN_Q4_K", dict(dim=3072, hidden_dim=2048, n_layers=2, n_heads=32, n_kv_heads=32, vocab_size=512,
+                                         seq_len=128, rope_freq_base=10000.0, rope_is_neox=True)),
+    "flow_q5km_hs64": ("PLAN_Q5_K_M", dict(dim=4096, hidden_dim=2048, n_layers=2, n_heads=64, n_kv_heads=16, vocab_size=600,
+                                           seq_len=128, rope_freq_base=10000.0, rope_is_neox=False)),
 }
 
 
@@ -40,8 +48,8 @@ def test_fp16_cache_matches_oracle(pkg, orc, case):
     lm = _model(pkg, plan, **kw)
     cfg = lm.config
     dev = lm.device(kv_fp16=True)
-    assert dev.path == 1
-    om = orc.model_from_language_model(lm, nthreads=8)
+    assert dev.path == (3 if case.startswith("flow_") else 1)
+    om = orc.model_from_language_model(lm, nthreads=16)
     mode = orc.GPU_SPEC | orc.KV16
     prompt = synth.seeded_prompt(5, 6, cfg.vocab_size)
     ids, logits = dev.generate_greedy(prompt, 40, want_logits=True)
@@ -97,10 +105,10 @@ def test_fp16_cache_limits(pkg):
     plan, kw = "PLAN_Q4_K", dict(dim=2048, hidden_dim=2048, n_layers=1, n_heads=16, n_kv_heads=4, vocab_size=300,
                                  seq_len=64, rope_freq_base=10000.0, rope_is_neox=False)
     lm = _model(pkg, plan, **kw)
-    with pytest.raises(pkg.L2HError):  # the one-launch-per-token kernels read fp32 caches
-        DeviceModel(lm.config, lm.weights, path=3, kv_fp16=True)
-    dev = DeviceModel(lm.config, lm.weights, kv_fp16=True)  # automatic choice: falls to path 1
-    assert dev.path == 1
+    with pytest.raises(pkg.L2HError):  # the persistent kernel with grid barriers reads fp32 caches
+        DeviceModel(lm.config, lm.weights, path=2, kv_fp16=True)
+    dev = DeviceModel(lm.config, lm.weights, kv_fp16=True)  # automatic choice: the streaming kernel
+    assert dev.path == 3
     with pytest.raises(pkg.L2HError):  # the batched prompt pass writes an fp32 cache
         dev.prefill(synth.seeded_prompt(1, 8, 300), 0)
     dev.close()
