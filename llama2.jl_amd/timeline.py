@@ -68,6 +68,17 @@ def main():
         d = np.diff(med[i0 - 1:i0 + per])
         print("layer 1: %.2f us = " % (med[i0 + per - 1] - med[i0 - 1]) +
               " ".join("%s:%.2f" % (names[i0 + k].rsplit(" ", 1)[0].replace(" ", "/"), d[k]) for k in range(per)))
+    # inside the attention of layer 2 (short caches): five stamps per head, relative to the moment the head's
+    # workgroup finished its q|k|v epilogue
+    if n_layers >= 3:
+        t0 = tl[:, 0].min()
+        a_us = (buf[n_wg * 64:n_wg * 64 + cfg.n_heads * 16].reshape(cfg.n_heads, 16) - t0) * 0.01
+        i_fin = names.index("qkv fin l2")
+        wg_of = [h * stride + h % stride for h in range(cfg.n_heads)]
+        rel = a_us[:, :5] - us[wg_of, i_fin][:, None]
+        labels = ("entered", "q, k, v and the keys there", "scores and maximum", "softmax", "values summed")
+        print("attention of layer 2, us after the workgroup's q|k|v epilogue (median over the heads): " +
+              ", ".join("%s %.2f" % (lab, float(np.median(rel[:, k]))) for k, lab in enumerate(labels)))
     dev.close()
 
 
