@@ -1896,39 +1896,72 @@ __device__ __noinline__ bool flow_stage_xf(const void *src, int K, const float *
     return true;
 }
 
-// the rows of one phase for one workgroup: a wavefront takes a contiguous run of the workgroup's rows, two at a
+// The rows of one phase for one workgroup: a wavefront takes a contiguous run of the workgroup's rows, two at a
 // time; partial sums in the layout the epilogues expect (a row is one "piece": four doubles, the sums of 16 lanes
-// each; CLS: one double per row)
-template <bool CLS>
-__device__ __forceinline__ void flow_loop_f32(const FlowGeom &g, int kind, int layer, int wg, int K) {
+// each; CLS: one double per row).  The weights do not depend on the phase's input: the first FLOW_F32_PRE 16-byte
+// loads per lane of the run's first two rows are requested before the wait for it (flow_f32_request), so that their
+// latency passes during the wait (layer phases have one or two rows per wavefront: usually all of their bytes).
+#define FLOW_F32_PRE 2
+struct F32Pre {
+    f32x4v w[2][FLOW_F32_PRE];
+};
+__device__ __forceinline__ const float4 *flow_f32_row(const FlowGeom &g, bool cls, int kind, int layer, int wg, int lr, int K) {
     const FlowArgs &a = c_flow;
+    const int L = wg * g.rpw + lr;
+    int seg, row;
+    flow_row_src(cls ? 1 : kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
+    const int wi = cls ? 7 : (kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 + seg : 6)));
+    return (const float4 *)(a.f_w[wi] + (cls ? (int64_t)0 : (int64_t)layer * a.f_stride[wi]) + (int64_t)row * K);
+}
+template <bool CLS>
+__device__ __forceinline__ void flow_f32_request(F32Pre &pre, const FlowGeom &g, int kind, int layer, int wg, int K) {
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    if (cnt <= 0) return;
+    const int n4 = K >> 2;
+#pragma unroll
+    for (int r = 0; r < 2; r++) {
+        const f32x4v *w4 = (const f32x4v *)flow_f32_row(g, CLS, kind, layer, wg, start + min(r, cnt - 1), K);
+#pragma unroll
+        for (int u = 0; u < FLOW_F32_PRE; u++)
+            if (lane + 64 * u < n4) pre.w[r][u] = __builtin_nontemporal_load(w4 + lane + 64 * u);
+    }
+}
+template <bool CLS>
+__device__ __forceinline__ void flow_loop_f32(const F32Pre &pre, const FlowGeom &g, int kind, int layer, int wg, int K) {
     int lane = threadIdx.x & 63;
     asm volatile("" : "+v"(lane));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     const float4 *x4 = (const float4 *)s_act;
     const int n4 = K >> 2;
+#define F32_FMA4(ACC_, W_, X_)                       \
+    ACC_ = fma((double)W_.x, (double)X_.x, ACC_);    \
+    ACC_ = fma((double)W_.y, (double)X_.y, ACC_);    \
+    ACC_ = fma((double)W_.z, (double)X_.z, ACC_);    \
+    ACC_ = fma((double)W_.w, (double)X_.w, ACC_)
     for (int i = 0; i < cnt; i += 2) {
-        const float4 *w4[2];
-#pragma unroll
-        for (int r = 0; r < 2; r++) {
-            const int L = wg * g.rpw + start + min(i + r, cnt - 1);
-            int seg, row;
-            flow_row_src(CLS ? 1 : kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
-            const int wi = CLS ? 7 : (kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 + seg : 6)));
-            w4[r] = (const float4 *)(a.f_w[wi] + (CLS ? (int64_t)0 : (int64_t)layer * a.f_stride[wi]) + (int64_t)row * K);
-        }
+        const float4 *wa4 = flow_f32_row(g, CLS, kind, layer, wg, start + i, K);
+        const float4 *wb4 = flow_f32_row(g, CLS, kind, layer, wg, start + min(i + 1, cnt - 1), K);
         double acc0 = 0.0, acc1 = 0.0;
-        for (int j = lane; j < n4; j += 64) {
-            const float4 wa = ldg_nt_f4(w4[0] + j), wb = ldg_nt_f4(w4[1] + j), xv = x4[j];
-            acc0 = fma((double)wa.x, (double)xv.x, acc0);
-            acc0 = fma((double)wa.y, (double)xv.y, acc0);
-            acc0 = fma((double)wa.z, (double)xv.z, acc0);
-            acc0 = fma((double)wa.w, (double)xv.w, acc0);
-            acc1 = fma((double)wb.x, (double)xv.x, acc1);
-            acc1 = fma((double)wb.y, (double)xv.y, acc1);
-            acc1 = fma((double)wb.z, (double)xv.z, acc1);
-            acc1 = fma((double)wb.w, (double)xv.w, acc1);
+        int j0 = 0;
+        if (i == 0) {  // the run's first two rows: their first loads were requested before the wait
+#pragma unroll
+            for (int u = 0; u < FLOW_F32_PRE; u++)
+                if (lane + 64 * u < n4) {
+                    const float4 xv = x4[lane + 64 * u];
+                    const f32x4v wa = pre.w[0][u], wb = pre.w[1][u];
+                    F32_FMA4(acc0, wa, xv);
+                    F32_FMA4(acc1, wb, xv);
+                }
+            j0 = 64 * FLOW_F32_PRE;
+        }
+        for (int j = j0 + lane; j < n4; j += 64) {
+            const float4 wa = ldg_nt_f4(wa4 + j), wb = ldg_nt_f4(wb4 + j), xv = x4[j];
+            F32_FMA4(acc0, wa, xv);
+            F32_FMA4(acc1, wb, xv);
         }
         if (CLS) {
             const double v0 = wave_sum_f64_dpp(acc0), v1 = wave_sum_f64_dpp(acc1);
@@ -1942,6 +1975,7 @@ __device__ __forceinline__ void flow_loop_f32(const FlowGeom &g, int kind, int l
             if (i + 1 < cnt) s_part[4 * (start + i + 1) + (lane >> 4)] = v1;
         }
     }
+#undef F32_FMA4
 }
 
 __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
@@ -1974,6 +2008,10 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
         for (int kind = 0; kind < 4; kind++) {
             bool ok;
             const FlowGeom g = flow_geom(a, kind);
+            const int K = kind == 3 ? a.hidden : a.dim;
+            F32Pre pre;
+            // (after the attention where this workgroup runs one: its loads would wait behind these)
+            if (kind != 1) flow_f32_request<false>(pre, g, kind, l, wg, K);
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
                 ok = l == 0 ? flow_stage_xf<PRO_RMSNORM, SRC_EMB>(nullptr, a.dim, nw, tok)
@@ -1986,6 +2024,7 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
                                                     : flow_attention_short<32>(l, att_h, pos, e_q, e_att);
                     if (!uni((int)fine)) return;
                 }
+                flow_f32_request<false>(pre, g, kind, l, wg, K);
                 ok = flow_stage_xf<PRO_QUANT, SRC_BARE>(a.xo + (int64_t)(e_att & 1u) * a.dim, a.dim, nullptr, tok);
             } else if (kind == 2) {
                 ok = flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_b, a.dim, a.rms_ffn + (int64_t)l * a.norm_stride, tok);
@@ -1996,7 +2035,7 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
             unsigned oldw = 0;
             if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = bare_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
             if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
-            flow_loop_f32<false>(g, kind, l, wg, kind == 3 ? a.hidden : a.dim);
+            flow_loop_f32<false>(pre, g, kind, l, wg, K);
             if (kind == 0)
                 flow_finish_qkv(l, wg, pos, e_q);
             else if (kind == 1)
@@ -2009,8 +2048,10 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
     }
     // ---- final rmsnorm (:309) + classifier (:312) ----
     const unsigned e_fin = E0 + 5u * (unsigned)a.n_layers, e_cls = e_fin + 1;
+    F32Pre pre;
+    flow_f32_request<true>(pre, a.cls, 4, 0, wg, a.dim);
     if (!uni(flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, a.rms_final, tok))) return;
-    flow_loop_f32<true>(a.cls, 4, 0, wg, a.dim);
+    flow_loop_f32<true>(pre, a.cls, 4, 0, wg, a.dim);
     flow_finish_cls(wg, e_cls);
     if (wg == 0) flow_pick_token(nwg, e_cls);
 }
