@@ -1832,8 +1832,11 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
 // Activations stay fp32 in LDS (no q8_K), products are exact in fp64 and summed in fp64, as in matvec_f32_kernel.
 // ------------------------------------------------------------------------------------------
 // the input vector of a phase -> fp32 in this workgroup's LDS; K <= 4096 and a multiple of 4
+#ifndef XF_INLINE
+#define XF_INLINE __noinline__
+#endif
 template <int PRO, int SRC>
-__device__ __noinline__ bool flow_stage_xf(const void *src, int K, const float *normw, int tok) {
+__device__ XF_INLINE bool flow_stage_xf(const void *src, int K, const float *normw, int tok) {
     src = uni(src), K = uni(K), normw = uni(normw), tok = uni(tok);
     const FlowArgs &a = c_flow;
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1896,22 +1899,28 @@ __device__ __noinline__ bool flow_stage_xf(const void *src, int K, const float *
     return true;
 }
 
-// The rows of one phase for one workgroup: a wavefront takes a contiguous run of the workgroup's rows, two at a
-// time; partial sums in the layout the epilogues expect (a row is one "piece": four doubles, the sums of 16 lanes
-// each; CLS: one double per row).  The weights do not depend on the phase's input: the first FLOW_F32_PRE 16-byte
-// loads per lane of the run's first two rows are requested before the wait for it (flow_f32_request), so that their
-// latency passes during the wait (layer phases have one or two rows per wavefront: usually all of their bytes).
+// The rows of one phase for one workgroup.  A row is cut into ppr slices of K / ppr inputs (a "piece", chosen so that a
+// slice is at most 512 floats where K allows: two 16-byte loads per lane), and a wavefront takes a contiguous run of
+// the workgroup's pieces, two at a time; partial sums in the layout the epilogues expect (four doubles per piece,
+// the sums of 16 lanes each; CLS: one double per piece).  The weights do not depend on the phase's input: the first
+// FLOW_F32_PRE 16-byte loads per lane of the run's first two pieces are requested before the wait for it
+// (flow_f32_request), so that their latency passes during the wait (layer phases have one or two pieces per
+// wavefront: usually all of their bytes).
 #define FLOW_F32_PRE 2
 struct F32Pre {
     f32x4v w[2][FLOW_F32_PRE];
 };
-__device__ __forceinline__ const float4 *flow_f32_row(const FlowGeom &g, bool cls, int kind, int layer, int wg, int lr, int K) {
+// piece j of the workgroup -> its floats (n4 groups of four)
+__device__ __forceinline__ const float4 *flow_f32_piece(const FlowGeom &g, bool cls, int kind, int layer, int wg, int j, int K,
+                                                        int &x_off4) {
     const FlowArgs &a = c_flow;
+    const int lr = j / g.ppr, part = j - lr * g.ppr;
     const int L = wg * g.rpw + lr;
     int seg, row;
     flow_row_src(cls ? 1 : kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row);
     const int wi = cls ? 7 : (kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 + seg : 6)));
-    return (const float4 *)(a.f_w[wi] + (cls ? (int64_t)0 : (int64_t)layer * a.f_stride[wi]) + (int64_t)row * K);
+    x_off4 = part * ((K / g.ppr) >> 2);
+    return (const float4 *)(a.f_w[wi] + (cls ? (int64_t)0 : (int64_t)layer * a.f_stride[wi]) + (int64_t)row * K) + x_off4;
 }
 template <bool CLS>
 __device__ __forceinline__ void flow_f32_request(F32Pre &pre, const FlowGeom &g, int kind, int layer, int wg, int K) {
@@ -1920,10 +1929,11 @@ __device__ __forceinline__ void flow_f32_request(F32Pre &pre, const FlowGeom &g,
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
     if (cnt <= 0) return;
-    const int n4 = K >> 2;
+    const int n4 = (K / g.ppr) >> 2;
 #pragma unroll
     for (int r = 0; r < 2; r++) {
-        const f32x4v *w4 = (const f32x4v *)flow_f32_row(g, CLS, kind, layer, wg, start + min(r, cnt - 1), K);
+        int xo;
+        const f32x4v *w4 = (const f32x4v *)flow_f32_piece(g, CLS, kind, layer, wg, start + min(r, cnt - 1), K, xo);
 #pragma unroll
         for (int u = 0; u < FLOW_F32_PRE; u++)
             if (lane + 64 * u < n4) pre.w[r][u] = __builtin_nontemporal_load(w4 + lane + 64 * u);
@@ -1935,33 +1945,34 @@ __device__ __forceinline__ void flow_loop_f32(const F32Pre &pre, const FlowGeom 
     asm volatile("" : "+v"(lane));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
-    const float4 *x4 = (const float4 *)s_act;
-    const int n4 = K >> 2;
+    const int n4 = (K / g.ppr) >> 2;
 #define F32_FMA4(ACC_, W_, X_)                       \
     ACC_ = fma((double)W_.x, (double)X_.x, ACC_);    \
     ACC_ = fma((double)W_.y, (double)X_.y, ACC_);    \
     ACC_ = fma((double)W_.z, (double)X_.z, ACC_);    \
     ACC_ = fma((double)W_.w, (double)X_.w, ACC_)
     for (int i = 0; i < cnt; i += 2) {
-        const float4 *wa4 = flow_f32_row(g, CLS, kind, layer, wg, start + i, K);
-        const float4 *wb4 = flow_f32_row(g, CLS, kind, layer, wg, start + min(i + 1, cnt - 1), K);
+        int xa, xb;
+        const float4 *wa4 = flow_f32_piece(g, CLS, kind, layer, wg, start + i, K, xa);
+        const float4 *wb4 = flow_f32_piece(g, CLS, kind, layer, wg, start + min(i + 1, cnt - 1), K, xb);
+        const float4 *xa4 = (const float4 *)s_act + xa, *xb4 = (const float4 *)s_act + xb;
         double acc0 = 0.0, acc1 = 0.0;
         int j0 = 0;
-        if (i == 0) {  // the run's first two rows: their first loads were requested before the wait
+        if (i == 0) {  // the run's first two pieces: their first loads were requested before the wait
 #pragma unroll
             for (int u = 0; u < FLOW_F32_PRE; u++)
                 if (lane + 64 * u < n4) {
-                    const float4 xv = x4[lane + 64 * u];
+                    const float4 xv = xa4[lane + 64 * u], yv = xb4[lane + 64 * u];
                     const f32x4v wa = pre.w[0][u], wb = pre.w[1][u];
                     F32_FMA4(acc0, wa, xv);
-                    F32_FMA4(acc1, wb, xv);
+                    F32_FMA4(acc1, wb, yv);
                 }
             j0 = 64 * FLOW_F32_PRE;
         }
         for (int j = j0 + lane; j < n4; j += 64) {
-            const float4 wa = ldg_nt_f4(wa4 + j), wb = ldg_nt_f4(wb4 + j), xv = x4[j];
+            const float4 wa = ldg_nt_f4(wa4 + j), wb = ldg_nt_f4(wb4 + j), xv = xa4[j], yv = xb4[j];
             F32_FMA4(acc0, wa, xv);
-            F32_FMA4(acc1, wb, xv);
+            F32_FMA4(acc1, wb, yv);
         }
         if (CLS) {
             const double v0 = wave_sum_f64_dpp(acc0), v1 = wave_sum_f64_dpp(acc1);
@@ -1983,6 +1994,16 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = blockIdx.x, nwg = gridDim.x;
     (void)wave;
+#ifdef L2H_TIMELINE
+    int tl_n = 0;
+#define XTL()                                                                                   \
+    do {                                                                                        \
+        if (a.timeline && tid == 0 && tl_n < 64) a.timeline[wg * 64 + tl_n++] = wall_clock64(); \
+    } while (0)
+#else
+#define XTL()
+#endif
+    XTL();
     // ---- this step's token, position and RoPE angles (reference src/inference.jl:122-127) ----
     const int pos = a.ctl->pos;
     const int tok = a.ctl->step < a.ctl->n_prompt ? a.prompt[a.ctl->step] : a.ctl->last_argmax;
@@ -2032,10 +2053,12 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
                 ok = flow_stage_xf<PRO_QUANT, SRC_BARE>(a.hbw + (int64_t)(e_w13 & 1u) * a.hidden, a.hidden, nullptr, tok);
             }
             if (!uni(ok)) return;
+            XTL();
             unsigned oldw = 0;
             if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = bare_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
             if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
             flow_loop_f32<false>(pre, g, kind, l, wg, K);
+            XTL();
             if (kind == 0)
                 flow_finish_qkv(l, wg, pos, e_q);
             else if (kind == 1)
@@ -2044,6 +2067,7 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
                 flow_finish_w13(wg, e_w13);
             else
                 flow_finish_resid(3, wg, oldw);
+            XTL();
         }
     }
     // ---- final rmsnorm (:309) + classifier (:312) ----
@@ -2054,6 +2078,7 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
     flow_loop_f32<true>(pre, a.cls, 4, 0, wg, a.dim);
     flow_finish_cls(wg, e_cls);
     if (wg == 0) flow_pick_token(nwg, e_cls);
+#undef XTL
 }
 
 // ------------------------------------------------------------------------------------------
@@ -2191,7 +2216,15 @@ static FlowGeom make_geom(int64_t n_rows, int64_t K, int type, int grid) {
     int rpw = (int)((n_rows + grid - 1) / grid);
     rpw += rpw & 1;
     g.rpw = rpw;
-    g.ppr = type == L2H_TYPE_F32 ? 1 : (int)(K / 256) / (type == L2H_TYPE_Q6_K ? 16 : 8);
+    if (type == L2H_TYPE_F32) {
+        // fp32 rows: slices of at most 512 floats where K allows it (1, 2, 4 or 8 slices of a multiple of 4 floats):
+        // two loads per lane, which flow_f32_request covers
+        int ppr = 1;
+        while (ppr < 8 && K / ppr > 512 && K % (8 * ppr) == 0) ppr *= 2;
+        g.ppr = ppr;
+    } else {
+        g.ppr = (int)(K / 256) / (type == L2H_TYPE_Q6_K ? 16 : 8);
+    }
     return g;
 }
 
@@ -2225,7 +2258,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
             a.cls = make_geom(a.vocab, a.dim, L2H_TYPE_F32, grid);
             const FlowGeom *gs[5] = {&a.qkv, &a.wo, &a.w13, &a.w2, &a.cls};
             for (const FlowGeom *g : gs)
-                if (g->rpw > FLOW_MAX_ROWS || g->rpw > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
+                if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
                     return no("too many rows per workgroup");
             if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
             a.f32 = 1;
