@@ -454,3 +454,42 @@ def test_streaming_kernel_soak_against_per_phase_path(pkg, case, reps, n_new):
         assert np.array_equal(a_logits.view(np.uint32), b_logits.view(np.uint32)), rep
     fast.close()
     slow.close()
+
+
+SHAPES = [
+    # (plan, dim, hidden, layers, heads, kv heads, vocab, neox): row counts that do not divide by the workgroups, odd
+    # vocabularies, one and many KV heads, every form of the kernel
+    ("PLAN_Q4_K", 2048, 6144, 1, 16, 16, 5001, False),
+    ("PLAN_Q4_K_S", 4096, 2048, 2, 32, 4, 999, False),
+    ("PLAN_Q4_K", 2048, 2048, 3, 64, 8, 257, True),
+    ("PLAN_Q5_K_M", 4096, 4096, 1, 32, 32, 1031, True),
+    (dict(emb=12, output=14, wq=14, wk=14, wv=14, wo=14, w1=14, w3=14, w2=14), 4096, 2048, 2, 64, 8, 300, False),
+    ("PLAN_Q4_K", 3072, 4096, 1, 32, 8, 777, False),
+    ("PLAN_F32", 512, 708, 2, 8, 2, 1001, False),
+    ("PLAN_F32", 1024, 2048, 1, 16, 16, 130, True),
+]
+
+
+@pytest.mark.parametrize("shape", range(len(SHAPES)))
+def test_streaming_kernel_other_shapes_against_per_phase_path(pkg, shape):
+    """Shapes off the benchmark's: the streaming kernel's split of rows over workgroups and wavefronts, its typed
+    pieces and its fp32 form against the per-phase path, tokens and final logits bit for bit (the per-phase path is
+    the one the oracle tests pin at many shapes)."""
+    from llama2_jl_amd import synth
+    from llama2_jl_amd.inference import DeviceModel
+    plan, dim, hidden, layers, heads, kv, vocab, neox = SHAPES[shape]
+    lm = _model(pkg, plan, dim=dim, hidden_dim=hidden, n_layers=layers, n_heads=heads, n_kv_heads=kv, vocab_size=vocab,
+                seq_len=320, rope_freq_base=10000.0, rope_is_neox=neox)
+    fast = DeviceModel(lm.config, lm.weights, path=3)
+    slow = DeviceModel(lm.config, lm.weights, path=1)
+    assert fast.path == 3 and slow.path == 1
+    for rep, n_new in enumerate((24, 300)):  # the second run crosses into the long-cache attention
+        prompt = synth.seeded_prompt(50 + rep, 3 + 4 * rep, vocab)
+        fast.reset()
+        slow.reset()
+        a_ids, a_logits = fast.generate_greedy(prompt, n_new, want_logits=True)
+        b_ids, b_logits = slow.generate_greedy(prompt, n_new, want_logits=True)
+        assert np.asarray(a_ids).tolist() == np.asarray(b_ids).tolist(), (shape, rep)
+        assert np.array_equal(a_logits.view(np.uint32), b_logits.view(np.uint32)), (shape, rep)
+    fast.close()
+    slow.close()
