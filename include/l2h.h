@@ -100,9 +100,11 @@ int l2h_model_set_kv_type(l2h_model *m, int kv_type);
 /* How transformer! is launched (before finalize): 0 = automatic (3 where the model fits it, else 1),
  * 1 = one kernel per phase (recorded once, replayed per token), 2 = a persistent kernel per token
  * with grid barriers between the phases, 3 = the streaming kernel per token (per-wavefront weight
- * streams fetched ahead into LDS, activations exchanged as epoch-tagged words; needs q4_K layer
- * matrices, a q4_K or q6_K classifier, dim and hidden_dim multiples of 2048, a short cache).
- * 2 and 3 are an error at finalize if the model does not fit.  All paths compute the same
+ * streams fetched ahead into LDS, activations exchanged as epoch-tagged words; needs q4_K, q5_K or
+ * q6_K layer matrices with a q4_K or q6_K classifier, dim 2048, 3072 or 4096 and hidden_dim a multiple
+ * of 2048 up to 14336 -- or a model of fp32 matrices with dim and hidden_dim up to 4096 in multiples of
+ * 4 -- and a head size of 32, 64, 96 or 128; any cache length).
+ * 2 and 3 are an error at finalize if the model does not fit; l2h_model_path_reason then tells why.  All paths compute the same
  * arithmetic and give the same results.  No counterpart in the reference.  l2h_model_path reports
  * the choice after finalize (1, 2 or 3). */
 int l2h_model_set_path(l2h_model *m, int path);
