@@ -37,8 +37,11 @@ WORKLOADS = {
     "8b-q5km": ("PLAN_Q5_K_M", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
                                     vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
     # the same shape with the tensor mix of a Q4_K_S file as llama.cpp is said to write it: attn_v and ffn_down of the
-    # first four layers q5_K (the streaming kernel takes all-q4_K layers only: this runs on launch path 1)
+    # first four layers q5_K (typed pieces in the streaming kernel)
     "8b-q4ks-file": ("plan_q4_k_s_file", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
+                                              vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
+    # and with that of a Q4_K_M file: attn_v and ffn_down q6_K in about half of the layers
+    "8b-q4km-file": ("plan_q4_k_m_file", dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8,
                                               vocab_size=128256, seq_len=512, rope_freq_base=500000.0, rope_is_neox=False), 32),
     "llama2c-f32": ("PLAN_F32", dict(dim=512, hidden_dim=1376, n_layers=8, n_heads=8, n_kv_heads=8, vocab_size=32000,
                                      seq_len=1024, rope_freq_base=10000.0, rope_is_neox=False), 16),

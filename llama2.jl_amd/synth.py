@@ -29,6 +29,16 @@ def plan_q4_k_s_file(n_layers, n_first=None):
     return dict(PLAN_Q4_K_S, wv=per_layer, w2=per_layer)
 
 
+def plan_q4_k_m_file(n_layers):
+    """The tensor mix llama.cpp's quantizer is said to give a Q4_K_M file (not checked against a real file here): q4_K
+    layers in which attn_v and ffn_down are q6_K for the layers its "use more bits" rule picks (the first and the last
+    eighth, and every third layer in between), q6_K output."""
+    def more_bits(i):
+        return i < n_layers // 8 or i >= 7 * n_layers // 8 or (i - n_layers // 8) % 3 == 2
+    per_layer = [TYPE_Q6_K if more_bits(l) else TYPE_Q4_K for l in range(n_layers)]
+    return dict(PLAN_Q4_K_S, wv=per_layer, w2=per_layer)
+
+
 def _threads():
     return max(1, min(16, os.cpu_count() or 1))
 

@@ -1,7 +1,7 @@
 """Where the time of one token goes inside the streaming decode kernel (launch path 3).
 
     python llama2.jl_amd/build.py --timeline          # builds llama2.jl_amd/libl2hip_tl.so (-DL2H_TIMELINE)
-    python llama2.jl_amd/timeline.py [n_layers]       # on the GPU; prints the table
+    python llama2.jl_amd/timeline.py [n_layers [plan]] # on the GPU; prints the table (plan: a name from synth.py, default PLAN_Q4_K_S)
 
 In the profiling build thread 0 of every workgroup stamps the 100 MHz wall clock at the phase boundaries
 of the first layers of a launch (after staging a phase's input, after the wait for the ring's pieces, at
@@ -31,9 +31,10 @@ def main():
     spec.loader.exec_module(pkg)
     from llama2_jl_amd import _lib, synth
     n_layers = int(sys.argv[1]) if len(sys.argv) > 1 else 4
+    plan = getattr(synth, sys.argv[2]) if len(sys.argv) > 2 else synth.PLAN_Q4_K_S  # e.g. PLAN_Q5_K_M: typed pieces
     cfg = pkg.ModelConfig(dim=4096, hidden_dim=14336, n_layers=n_layers, n_heads=32, n_kv_heads=8, vocab_size=128256,
                           seq_len=512, rope_freq_base=500000.0)
-    lm = synth.synthetic_model(cfg, synth.PLAN_Q4_K_S, seed=1)
+    lm = synth.synthetic_model(cfg, plan, seed=1)
     dev = lm.device(path=3)
     dev.generate_greedy(synth.seeded_prompt(1, 32, cfg.vocab_size), 8)
     lib = _lib.lib()
