@@ -68,8 +68,12 @@ function set_tensor!(m::DeviceModel, role, layer, A)
     check(m.ctx.handle, rc)
 end
 
-"Upload the weights of a Llama2.jl `LanguageModel` once; the copy stays resident in HBM."
-function DeviceModel(model::LanguageModel; ctx::Context = Context(), seq_len::Integer = model.config.seq_len)
+"""
+Upload the weights of a Llama2.jl `LanguageModel` once; the copy stays resident in HBM.  `kv_fp16 = true` keeps
+the KV cache in Float16 (rows rounded when appended; the reference's cache is Float32, `src/inference.jl:62-70`).
+"""
+function DeviceModel(model::LanguageModel; ctx::Context = Context(), seq_len::Integer = model.config.seq_len,
+                     kv_fp16::Bool = false)
     c = model.config
     cfg = L2HConfig(c.dim, c.hidden_dim, c.n_layers, c.n_heads, c.n_kv_heads, c.vocab_size, seq_len,
                     c.rope_freq_base, c.rope_is_neox ? 1 : 0)
@@ -88,9 +92,14 @@ function DeviceModel(model::LanguageModel; ctx::Context = Context(), seq_len::In
             set_tensor!(m, role, l - 1, A)
         end
     end
+    kv_fp16 && check(ctx.handle, ccall((:l2h_model_set_kv_type, lib), Cint, (Ptr{Cvoid}, Cint), m.handle, 1))
     check(ctx.handle, ccall((:l2h_model_finalize, lib), Cint, (Ptr{Cvoid},), m.handle))
     return m
 end
+
+"Which of the library's launch paths decodes this model (3 = the one-launch-per-token streaming kernel), and why not 3."
+launch_path(m::DeviceModel) = Int(ccall((:l2h_model_path, lib), Cint, (Ptr{Cvoid},), m.handle))
+launch_path_reason(m::DeviceModel) = unsafe_string(ccall((:l2h_model_path_reason, lib), Cstring, (Ptr{Cvoid},), m.handle))
 
 reset!(m::DeviceModel) = check(m.ctx.handle, ccall((:l2h_state_reset, lib), Cint, (Ptr{Cvoid},), m.handle))
 
