@@ -317,6 +317,23 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
     float xv[4][4];
     float wv0[4];
     bool ok = true;
+    // one q8_K block of this wavefront: quantized and put into LDS
+    auto quantize_block = [&](int r, const float (&x4)[4]) {
+        const int b = wave + r * FLOW_NW;
+        uint32_t packed;
+        int bsum;
+        float d;
+        q8k_quantize_wave(x4, packed, bsum, d);
+        ((uint32_t *)s_qs)[64 * b + lane] = packed;
+        if ((lane & 3) == 0) s_bs[16 * b + (lane >> 2)] = (int16_t)bsum;
+        if (lane == 0) s_d[b] = d;
+    };
+    // A vector that is only quantized (no norm over the whole of it) is quantized block by block as the blocks become
+    // complete, while the words of slower producers are still being waited for: the q8_K area is free by now (its last
+    // readers, the previous phase's loops, ended before that phase's epilogue), and of the 2.4 µs that the 56 blocks of the
+    // SwiGLU vector take, most then lies inside the wait.
+    constexpr bool early = !rms && SRC == SRC_BARE;
+    unsigned done = 0u;  // (bit r: block r is in LDS)
     // the norm weights are requested before the wait for the input: their latency passes meanwhile
     if (rms && rounds > 0) {
         const float4 t = *(const float4 *)(normw + 256 * wave + 4 * lane);
@@ -351,6 +368,17 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
                 if (!(FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3)))
                     POLL_BARE4(w0, w1, w2, w3, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW, pb + 768 * FLOW_NW);
                 all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
+            }
+            if (early) {
+                const u32x4v wr[4] = {w0, w1, w2, w3};
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (r < rounds && !(done & (1u << r)) && __ballot(!FULL(wr[r])) == 0ull) {
+                        const float x4[4] = {__uint_as_float(wr[r].x), __uint_as_float(wr[r].y), __uint_as_float(wr[r].z),
+                                             __uint_as_float(wr[r].w)};
+                        quantize_block(r, x4);
+                        done |= 1u << r;
+                    }
             }
 #undef FULL
             if (__ballot(!all) == 0ull) break;
@@ -394,18 +422,10 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
 #pragma unroll
         for (int k = 0; k < 4; k++) xv[0][k] = wv0[k] * (ss * xv[0][k]);
     }
+    if (!early) {
 #pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const int b = wave + r * FLOW_NW;
-        if (r < rounds && (SRC == SRC_BARE || r == 0)) {
-            uint32_t packed;
-            int bsum;
-            float d;
-            q8k_quantize_wave(xv[r], packed, bsum, d);
-            ((uint32_t *)s_qs)[64 * b + lane] = packed;
-            if ((lane & 3) == 0) s_bs[16 * b + (lane >> 2)] = (int16_t)bsum;
-            if (lane == 0) s_d[b] = d;
-        }
+        for (int r = 0; r < 4; r++)
+            if (r < rounds && (SRC == SRC_BARE || r == 0)) quantize_block(r, xv[r]);
     }
     __syncthreads();
     return true;
