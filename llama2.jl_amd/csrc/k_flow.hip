@@ -1396,6 +1396,16 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     u64 *x_part = a.att_x + (int64_t)a.n_heads * G * 3 + ((int64_t)h * G) * hs * 2;
     const int tid = threadIdx.x;
     bool ok = true;
+#ifdef L2H_TIMELINE
+    int stl = 0;  // profiling build: member 0 of every head stamps the steps of layer 2
+#define STL()                                                                                                         \
+    do {                                                                                                              \
+        if (a.timeline && tid == 0 && j == 0 && layer == 2 && stl < 16) a.timeline[256 * 64 + h * 16 + stl++] = wall_clock64(); \
+    } while (0)
+#else
+#define STL()
+#endif
+    STL();
     __syncthreads();  // the activation area is free
     if (tid < 3 * hs) {
         const int which = tid / hs, i = tid % hs;
@@ -1428,15 +1438,18 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         return false;                                                                                              \
     }
     SPLIT_CHECK();
+    STL();
     const float scale = sqrtf((float)hs);
     float mx = -INFINITY;
-    // scores: thread = (timestep tl of a block of 256, quarter of the head dimension); the quarter's 16-byte loads
-    // are all in flight at once; quarters are added in order (fp64)
+    // (a cache row that only one head reads is read once per token: loaded with the non-temporal hint)
+    const bool once = a.n_heads == a.n_kv_heads;
+    // scores: a wavefront takes 16 timesteps at a time, lane = (timestep p16, quarter of the head dimension); the
+    // quarter's 16-byte loads are all in flight at once; the quarters are added in order (fp64) through lane exchanges,
+    // so that the wavefronts run through their timesteps without meeting
     {
-        const int tl = tid & 255, part = tid >> 8, per = hs >> 4;  // hs is a multiple of 16, at most 128
-        double *s_sp = s_r;                                        // [4][256]
-        for (int t0 = lo; t0 < hi; t0 += 256) {
-            const int t = t0 + tl;
+        const int lane = tid & 63, wv = tid >> 6, p16 = lane & 15, part = lane >> 4, per = hs >> 4;  // hs: a multiple of 16, at most 128
+        for (int t0 = lo + 16 * wv; t0 < hi; t0 += 16 * FLOW_NW) {
+            const int t = t0 + p16;
             double acc = 0.0;
             if (H16) {
                 if (t < hi) {
@@ -1468,7 +1481,7 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                 float4 kv[8];
 #pragma unroll
                 for (int u = 0; u < 8; u++)
-                    if (u < per) kv[u] = t == pos ? kl[u] : kp[(int64_t)u * seq_len];
+                    if (u < per) kv[u] = t == pos ? kl[u] : (once ? ldg_nt_f4(kp + (int64_t)u * seq_len) : kp[(int64_t)u * seq_len]);
 #pragma unroll
                 for (int u = 0; u < 8; u++)
                     if (u < per) {
@@ -1479,18 +1492,16 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                         acc = fma(qq[3], (double)kv[u].w, acc);
                     }
             }
-            s_sp[part * 256 + tl] = acc;
-            __syncthreads();
+            const double a1 = __shfl(acc, p16 + 16, WAVE), a2 = __shfl(acc, p16 + 32, WAVE), a3 = __shfl(acc, p16 + 48, WAVE);
             if (part == 0 && t < hi) {
-                const double v = ((s_sp[tl] + s_sp[256 + tl]) + s_sp[512 + tl]) + s_sp[768 + tl];
-                const float sc = (float)v / scale;
+                const float sc = (float)(((acc + a1) + a2) + a3) / scale;
                 s_att[t - lo] = sc;
                 mx = fmaxf(mx, sc);
             }
-            __syncthreads();
         }
     }
     mx = block_max_f32(mx, s_redf);
+    STL();
     if (tid == 0) tag_store(x_max + j, mx, e_out);
     if (tid < G) {  // the largest score of the head: every member's
         const u64 *p = x_max + tid;
@@ -1509,6 +1520,7 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     if (!ok) s_flag = 1;
     __syncthreads();
     SPLIT_CHECK();
+    STL();
     float gmx = -INFINITY;
     for (int k = 0; k < G; k++) gmx = fmaxf(gmx, (float)s_x[k]);
     double sum = 0.0;
@@ -1518,11 +1530,13 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         sum += (double)e;
     }
     sum = block_sum_f64(sum, s_red);  // (ends with every thread past the reads of s_x above)
+    STL();
     if (tid == 0) tag_store_f64(x_sum + 2 * j, sum, e_out);
     if (tid < G) s_x[tid] = tag_wait_f64(x_sum + 2 * tid, e_out, ok);
     if (!ok) s_flag = 1;
     __syncthreads();
     SPLIT_CHECK();
+    STL();
     double tot = 0.0;
     for (int k = 0; k < G; k++) tot += s_x[k];
     const float sf = (float)tot;  // softmax!'s sum (reference src/inference.jl:169-174)
@@ -1578,16 +1592,21 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         const bool v_lane = i4 < n4;
         const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
         double acc[4] = {0.0, 0.0, 0.0, 0.0};
-        for (int t0 = lo + grp; t0 < hi; t0 += 4 * ngrp) {
-            float4 v[4];
+#ifndef FLOW_VD
+#define FLOW_VD 4
+#endif
+        constexpr int VD = FLOW_VD;
+        for (int t0 = lo + grp; t0 < hi; t0 += VD * ngrp) {
+            float4 v[VD];
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < VD; u++) {
                 const int t = t0 + u * ngrp;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (t < hi && v_lane) v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : vp[(int64_t)t * n4];
+                if (t < hi && v_lane)
+                    v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : (once ? ldg_nt_f4(vp + (int64_t)t * n4) : vp[(int64_t)t * n4]);
             }
 #pragma unroll
-            for (int u = 0; u < 4; u++) {
+            for (int u = 0; u < VD; u++) {
                 const int t = t0 + u * ngrp;
                 if (t < hi) {
                     const double p = (double)(s_att[t - lo] / sf);
@@ -1608,6 +1627,7 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         }
     }
     __syncthreads();
+    STL();
     if (tid < hs) {
         double acc = 0.0;
         for (int k = 0; k < FLOW_NW; k++) acc += s_r[k * hs + tid];
@@ -1625,6 +1645,7 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
     __syncthreads();
     SPLIT_CHECK();
 #undef SPLIT_CHECK
+    STL();
     if (tid < per_m) {
         double acc = 0.0;
         for (int m = 0; m < G; m++) acc += s_r[tid * G + m];
@@ -1633,6 +1654,8 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         bare_store(a.xo + (int64_t)((e_out & 1u) ^ 1u) * a.dim + (int64_t)h * hs + el, FLOW_EMPTY);
     }
     __syncthreads();
+    STL();
+#undef STL
     return true;
 }
 
