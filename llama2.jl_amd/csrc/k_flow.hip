@@ -1278,11 +1278,13 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
         for (int u = 0; u < NV; u++) {
             const int tv = grp + u * ngrp;
             v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (v_lane) {
-                if (tv < pos) v[u] = vp[(int64_t)tv * n4];
-                else if (tv == pos) v[u] = ((const float4 *)s_vcur)[i4];
-            }
+            if (v_lane && tv < pos) v[u] = vp[(int64_t)tv * n4];
         }
+        // (the current position's row comes from LDS, after all the loads are out: a choice between the two sources at
+        // each load makes the compiler wait for every load in turn)
+#pragma unroll
+        for (int u = 0; u < NV; u++)
+            if (v_lane && grp + u * ngrp == pos) v[u] = ((const float4 *)s_vcur)[i4];
         // the quarters are added in order (fp64)
         const double a1 = __shfl(acc, p16 + 16, WAVE), a2 = __shfl(acc, p16 + 32, WAVE), a3 = __shfl(acc, p16 + 48, WAVE);
         if (part == 0 && t < np) sc = (float)(((acc + a1) + a2) + a3) / scale;
@@ -1459,14 +1461,14 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                     Half8 kv[4];
 #pragma unroll
                     for (int u = 0; u < 4; u++)
-                        if (u < per8) {
-                            if (t == pos) {
+                        if (u < per8) kv[u] = ldg_nt_h8(kc, kg + (int64_t)u * seq_len);
+                    if (t == pos) {  // (replaced afterwards: see the fp32 rows below)
+#pragma unroll
+                        for (int u = 0; u < 4; u++)
+                            if (u < per8)
 #pragma unroll
                                 for (int c = 0; c < 8; c++) kv[u].v[c] = kl[8 * u + c];
-                            } else {
-                                kv[u] = ldg_nt_h8(kc, kg + (int64_t)u * seq_len);
-                            }
-                        }
+                    }
 #pragma unroll
                     for (int u = 0; u < 4; u++)
                         if (u < per8) {
@@ -1479,9 +1481,17 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                 const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
                 const float4 *kl = (const float4 *)s_kcur + part * per;
                 float4 kv[8];
+                // (all of a lane's loads are requested before anything waits for one: the current position's row, which
+                // comes from LDS, replaces what was loaded for it afterwards — a choice between the two sources at the
+                // load itself makes the compiler wait for every load in turn)
 #pragma unroll
                 for (int u = 0; u < 8; u++)
-                    if (u < per) kv[u] = t == pos ? kl[u] : (once ? ldg_nt_f4(kp + (int64_t)u * seq_len) : kp[(int64_t)u * seq_len]);
+                    if (u < per) kv[u] = once ? ldg_nt_f4(kp + (int64_t)u * seq_len) : kp[(int64_t)u * seq_len];
+                if (t == pos) {
+#pragma unroll
+                    for (int u = 0; u < 8; u++)
+                        if (u < per) kv[u] = kl[u];
+                }
 #pragma unroll
                 for (int u = 0; u < 8; u++)
                     if (u < per) {
@@ -1558,15 +1568,14 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                 const int t = t0 + u * ng;
 #pragma unroll
                 for (int c = 0; c < 8; c++) v[u].v[c] = 0.f;
-                if (t < hi && v_lane) {
-                    if (t == pos) {
-#pragma unroll
-                        for (int c = 0; c < 8; c++) v[u].v[c] = s_vcur[8 * i8 + c];
-                    } else {
-                        v[u] = ldg_nt_h8(vc, ((int64_t)kvh * seq_len + t) * n8 + i8);
-                    }
-                }
+                if (t < hi && v_lane) v[u] = ldg_nt_h8(vc, ((int64_t)kvh * seq_len + t) * n8 + i8);
             }
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+                if (t0 + u * ng == pos && v_lane) {
+#pragma unroll
+                    for (int c = 0; c < 8; c++) v[u].v[c] = s_vcur[8 * i8 + c];
+                }
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int t = t0 + u * ng;
@@ -1602,12 +1611,12 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
             for (int u = 0; u < VD; u++) {
                 const int t = t0 + u * ngrp;
                 v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (t < hi && v_lane)
-                    v[u] = t == pos ? *(const float4 *)(s_vcur + 4 * i4) : (once ? ldg_nt_f4(vp + (int64_t)t * n4) : vp[(int64_t)t * n4]);
+                if (t < hi && v_lane) v[u] = once ? ldg_nt_f4(vp + (int64_t)t * n4) : vp[(int64_t)t * n4];
             }
 #pragma unroll
             for (int u = 0; u < VD; u++) {
                 const int t = t0 + u * ngrp;
+                if (t == pos && v_lane) v[u] = *(const float4 *)(s_vcur + 4 * i4);  // (see the scores)
                 if (t < hi) {
                     const double p = (double)(s_att[t - lo] / sf);
                     acc[0] = fma(p, (double)v[u].x, acc[0]);
