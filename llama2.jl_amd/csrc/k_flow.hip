@@ -1459,10 +1459,14 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
                     const int64_t kg = ((int64_t)kvh * (hs >> 3) + part * per8) * seq_len + t;
                     const float *kl = s_kcur + part * (hs >> 2);
                     Half8 kv[4];
+                    h8_bits kb[4];  // (all loads first, then the widening: see the fp32 rows below)
+                    // (no branch around a load: a group beyond the head size repeats group 0)
+#pragma unroll
+                    for (int u = 0; u < 4; u++) kb[u] = ldg_nt_h8_bits(kc, kg + (int64_t)(u < per8 ? u : 0) * seq_len);
 #pragma unroll
                     for (int u = 0; u < 4; u++)
-                        if (u < per8) kv[u] = ldg_nt_h8(kc, kg + (int64_t)u * seq_len);
-                    if (t == pos) {  // (replaced afterwards: see the fp32 rows below)
+                        if (u < per8) kv[u] = h8_widen(kb[u]);
+                    if (t == pos) {
 #pragma unroll
                         for (int u = 0; u < 4; u++)
                             if (u < per8)
@@ -1563,13 +1567,15 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
         double acc[8] = {0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0};
         for (int t0 = lo + grp; t0 < hi; t0 += 4 * ng) {
             Half8 v[4];
+            h8_bits vb[4];
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int t = t0 + u * ng;
-#pragma unroll
-                for (int c = 0; c < 8; c++) v[u].v[c] = 0.f;
-                if (t < hi && v_lane) v[u] = ldg_nt_h8(vc, ((int64_t)kvh * seq_len + t) * n8 + i8);
+                vb[u] = (h8_bits){0u, 0u, 0u, 0u};
+                if (t < hi && v_lane) vb[u] = ldg_nt_h8_bits(vc, ((int64_t)kvh * seq_len + t) * n8 + i8);
             }
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = h8_widen(vb[u]);
 #pragma unroll
             for (int u = 0; u < 4; u++)
                 if (t0 + u * ng == pos && v_lane) {

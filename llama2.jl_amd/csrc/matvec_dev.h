@@ -23,10 +23,13 @@ __device__ __forceinline__ float4 ldg_nt_f4(const float4 *p) {
 struct Half8 {
     float v[8];
 };
-// 8 consecutive fp16 elements (group g of 16 bytes), widened to fp32 (exact)
-__device__ __forceinline__ Half8 ldg_nt_h8(const void *base, int64_t g) {
-    typedef unsigned int u32x4v_ __attribute__((ext_vector_type(4)));
-    const u32x4v_ t = __builtin_nontemporal_load((const u32x4v_ *)base + g);
+// 8 consecutive fp16 elements (group g of 16 bytes): the load, and the widening to fp32 (exact).  Separate, so that a
+// caller can request several groups before it waits for the first.
+typedef unsigned int h8_bits __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ h8_bits ldg_nt_h8_bits(const void *base, int64_t g) {
+    return __builtin_nontemporal_load((const h8_bits *)base + g);
+}
+__device__ __forceinline__ Half8 h8_widen(const h8_bits t) {
     Half8 r;
     r.v[0] = half_bits_to_float((uint16_t)(t.x & 0xFFFF));
     r.v[1] = half_bits_to_float((uint16_t)(t.x >> 16));
@@ -38,6 +41,7 @@ __device__ __forceinline__ Half8 ldg_nt_h8(const void *base, int64_t g) {
     r.v[7] = half_bits_to_float((uint16_t)(t.w >> 16));
     return r;
 }
+__device__ __forceinline__ Half8 ldg_nt_h8(const void *base, int64_t g) { return h8_widen(ldg_nt_h8_bits(base, g)); }
 // element i of a cache <- v (fp16: rounded to nearest even)
 __device__ __forceinline__ void st_kv(void *base, int64_t i, float v, bool h16) {
     if (h16)
