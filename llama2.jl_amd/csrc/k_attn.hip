@@ -131,10 +131,14 @@ __global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, con
         // fp16 cache: 16-byte groups of eight elements, hs / 32 of them per quarter (hs a multiple of 32, at most 128)
         const int per8 = hs >> 5;
         const int64_t kg = ((int64_t)kvh * (hs >> 3) + part * per8) * seq_len + t;
+        // (all loads are requested before one is waited for: no branch around a load — a group beyond the head size
+        // repeats group 0 — and the widening to fp32 comes after the last request)
+        h8_bits kb[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) kb[u] = ldg_nt_h8_bits(kc, kg + (int64_t)(u < per8 ? u : 0) * seq_len);
         Half8 kv[4];
 #pragma unroll
-        for (int u = 0; u < 4; u++)
-            if (u < per8) kv[u] = ldg_nt_h8(kc, kg + (int64_t)u * seq_len);
+        for (int u = 0; u < 4; u++) kv[u] = h8_widen(kb[u]);
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < 4; u++) {
@@ -152,8 +156,7 @@ __global__ __launch_bounds__(256) void attn_scores4_kernel(const double *qd, con
         const int64_t kg = ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;  // group of four elements
         float4 kv[8];
 #pragma unroll
-        for (int u = 0; u < 8; u++)
-            if (u < per) kv[u] = ldg_nt_f4((const float4 *)kc + kg + (int64_t)u * seq_len);
+        for (int u = 0; u < 8; u++) kv[u] = ldg_nt_f4((const float4 *)kc + kg + (int64_t)(u < per ? u : 0) * seq_len);
         __syncthreads();
 #pragma unroll
         for (int u = 0; u < 8; u++) {
@@ -258,13 +261,15 @@ __global__ __launch_bounds__(256) void attn_av4_kernel(const float *att, const d
             }
             Half8 v[4];
             const int64_t vg = ((int64_t)kvh * seq_len + t0) * n8 + i8;
+            h8_bits vb[4];  // (loads first, widening after the last request)
 #pragma unroll
             for (int u = 0; u < 4; u++) {
                 const int l = tg + 16 * u;
-#pragma unroll
-                for (int c = 0; c < 8; c++) v[u].v[c] = 0.f;
-                if (active && l < nt) v[u] = ldg_nt_h8(vc, vg + (int64_t)l * n8);
+                vb[u] = (h8_bits){0u, 0u, 0u, 0u};
+                if (active && l < nt) vb[u] = ldg_nt_h8_bits(vc, vg + (int64_t)l * n8);
             }
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = h8_widen(vb[u]);
             __syncthreads();
 #pragma unroll
             for (int u = 0; u < 4; u++) {
