@@ -52,7 +52,7 @@ __constant__ __attribute__((aligned(16))) unsigned char c_flow_raw[(sizeof(FlowA
 __shared__ __attribute__((aligned(16))) unsigned char s_ring[FLOW_NW * FLOW_D * FLOW_SLOT];
 // activation area: q8_K input of the running phase in the first 16 KiB, then the per-piece partial sums
 // and the row values; attention (between two matvec phases) uses the whole area for itself
-__shared__ uint4 s_act[FLOW_ACT_BYTES / 16];
+__shared__ uint4 s_act[(FLOW_ACT_BYTES + 2048) / 16];  // (+ 2 KiB behind it: the last two of flow_stage's raw blocks)
 #define s_part ((double *)((unsigned char *)s_act + 16384))
 #define s_val ((float *)((unsigned char *)s_act + 16384 + FLOW_MAX_PIECES * 8))
 __shared__ float s_rope[256];
@@ -315,8 +315,21 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
     const int rounds = nb > wave ? (nb - wave + FLOW_NW - 1) / FLOW_NW : 0;  // q8_K blocks of this wavefront
     constexpr bool rms = PRO == PRO_RMSNORM;
     float xv[4][4];
-    float wv0[4];
+    float nw16[16];
     bool ok = true;
+    // A vector that is normalised first (K <= 4096: at most one block per wavefront) is waited for by all sixteen
+    // wavefronts, a block each, which also form the sum of squares; its raw values then go through LDS to the first four
+    // wavefronts, which normalise and quantise four blocks each, a block per row of 16 lanes (q8k_quantize_rows16): with a
+    // block per wavefront the sixteen of them spent 1.3 us in that arithmetic, four to a SIMD.  Block b waits in the part
+    // of the activation area that nothing else uses while a dim-long vector is staged — except that the last block of
+    // each of the four wavefronts waits where that same wavefront's quants go (it reads before it writes), and the last
+    // two of the others behind the activation area.
+    auto raw_of = [&](int b) -> float * {
+        const int w = b >> 2, r = b & 3, i = 3 * w + r;
+        const int at = r == 3 ? 256 * w : (i < 10 ? 1024 + 256 * i : FLOW_ACT_BYTES / 4 + 256 * (i - 10));
+        return (float *)s_act + at;
+    };
+    const int row_b = 4 * wave + (lane >> 4), g16 = lane & 15;  // (rms, first four wavefronts: block and group of this lane)
     // one q8_K block of this wavefront: quantized and put into LDS
     auto quantize_block = [&](int r, const float (&x4)[4]) {
         const int b = wave + r * FLOW_NW;
@@ -335,12 +348,16 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
     constexpr bool early = !rms && SRC == SRC_BARE;
     unsigned done = 0u;  // (bit r: block r is in LDS)
     // the norm weights are requested before the wait for the input: their latency passes meanwhile
-    if (rms && rounds > 0) {
-        const float4 t = *(const float4 *)(normw + 256 * wave + 4 * lane);
-        wv0[0] = t.x;
-        wv0[1] = t.y;
-        wv0[2] = t.z;
-        wv0[3] = t.w;
+    if (rms && wave < 4) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            // (a row without a block works on block 0's numbers and stores nothing)
+            const float4 t = *(const float4 *)(normw + 256 * (row_b < nb ? row_b : 0) + 16 * g16 + 4 * q);
+            nw16[4 * q] = t.x;
+            nw16[4 * q + 1] = t.y;
+            nw16[4 * q + 2] = t.z;
+            nw16[4 * q + 3] = t.w;
+        }
     }
     if (SRC == SRC_EMB) {
         if (rounds > 0)
@@ -406,6 +423,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
         }
         acc = wave_sum_f64_dpp(acc);
         if (lane == 0) s_red[wave] = acc;
+        if (rounds > 0) *(float4 *)(raw_of(wave) + 4 * lane) = make_float4(xv[0][0], xv[0][1], xv[0][2], xv[0][3]);
     }
     __syncthreads();
     if (s_flag) {
@@ -413,16 +431,35 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
         return false;
     }
     if (rms) {
-        double t = 0.0;
-        for (int w = 0; w < FLOW_NW; w++) t += s_red[w];
-        float ss = (float)t;
-        ss /= (float)K;
-        ss += 1e-5f;
-        ss = 1.0f / sqrtf(ss);
+        if (wave < 4) {
+            double t = 0.0;
+            for (int w = 0; w < FLOW_NW; w++) t += s_red[w];
+            float ss = (float)t;
+            ss /= (float)K;
+            ss += 1e-5f;
+            ss = 1.0f / sqrtf(ss);
+            const bool there = row_b < nb;
+            const float *xr = raw_of(there ? row_b : 0) + 16 * g16;
+            float v[16];
 #pragma unroll
-        for (int k = 0; k < 4; k++) xv[0][k] = wv0[k] * (ss * xv[0][k]);
-    }
-    if (!early) {
+            for (int q = 0; q < 4; q++) {
+                const float4 x4 = *(const float4 *)(xr + 4 * q);
+                v[4 * q] = nw16[4 * q] * (ss * x4.x);
+                v[4 * q + 1] = nw16[4 * q + 1] * (ss * x4.y);
+                v[4 * q + 2] = nw16[4 * q + 2] * (ss * x4.z);
+                v[4 * q + 3] = nw16[4 * q + 3] * (ss * x4.w);
+            }
+            q8k_u32x4 packed;
+            int bsum;
+            float d;
+            q8k_quantize_rows16(v, packed, bsum, d);
+            if (there) {
+                ((q8k_u32x4 *)s_qs)[16 * row_b + g16] = packed;
+                s_bs[16 * row_b + g16] = (int16_t)bsum;
+                if (g16 == 0) s_d[row_b] = d;
+            }
+        }
+    } else if (!early) {
 #pragma unroll
         for (int r = 0; r < 4; r++)
             if (r < rounds && (SRC == SRC_BARE || r == 0)) quantize_block(r, xv[r]);
