@@ -59,6 +59,16 @@ __shared__ float s_rope[256];
 __shared__ double s_red[16];
 __shared__ float s_redf[16];
 __shared__ int s_flag;
+#ifdef L2H_TIMELINE
+// profiling build: flow_stage's own stamps (thread 0 of one workgroup, one layer) go to a.timeline[s_tl_fine++]
+__shared__ int s_tl_fine;
+#define STG()                                                                                          \
+    do {                                                                                               \
+        if (threadIdx.x == 0 && a.timeline && s_tl_fine >= 0) a.timeline[s_tl_fine++] = wall_clock64(); \
+    } while (0)
+#else
+#define STG()
+#endif
 __shared__ __attribute__((aligned(16))) unsigned char s_sink[256];  // target of fetches made only to warm the L2
 
 __device__ __forceinline__ void tag_store(u64 *p, float v, unsigned epoch) {
@@ -317,6 +327,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
     float xv[4][4];
     float nw16[16];
     bool ok = true;
+    STG();  // entered
     // A vector that is normalised first (K <= 4096: at most one block per wavefront) is waited for by all sixteen
     // wavefronts, a block each, which also form the sum of squares; its raw values then go through LDS to the first four
     // wavefronts, which normalise and quantise four blocks each, a block per row of 16 lanes (q8k_quantize_rows16): with a
@@ -386,6 +397,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
                     POLL_BARE4(w0, w1, w2, w3, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW, pb + 768 * FLOW_NW);
                 all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
             }
+            if (spins == 0) STG();  // the first poll is back
             if (early) {
                 const u32x4v wr[4] = {w0, w1, w2, w3};
 #pragma unroll
@@ -405,6 +417,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
                 break;
             }
         }
+        STG();  // this wavefront's words are all there
         const u32x4v ws[4] = {w0, w1, w2, w3};
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -426,6 +439,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
         if (rounds > 0) *(float4 *)(raw_of(wave) + 4 * lane) = make_float4(xv[0][0], xv[0][1], xv[0][2], xv[0][3]);
     }
     __syncthreads();
+    STG();  // every wavefront's are
     if (s_flag) {
         if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         return false;
@@ -464,7 +478,9 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
         for (int r = 0; r < 4; r++)
             if (r < rounds && (SRC == SRC_BARE || r == 0)) quantize_block(r, xv[r]);
     }
+    STG();  // this wavefront's blocks are in LDS
     __syncthreads();
+    STG();  // everybody's
     return true;
 }
 
@@ -1819,6 +1835,9 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
             const FlowGeom g = flow_geom(a, kind);
             const int n_reg = MIXED ? 0 : uni(flow_reg_pieces(g, wg, wave));
             if (!MIXED && kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
+#ifdef L2H_TIMELINE
+            if (tid == 0) s_tl_fine = ((int)gridDim.x > 101 && wg == 101 && l == 2) ? 256 * 64 + 512 + kind * 8 : -1;
+#endif
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;
                 ok = l == 0 ? flow_stage<PRO_RMSNORM, SRC_EMB>(nullptr, a.dim, nw, tok)

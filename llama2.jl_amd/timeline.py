@@ -8,8 +8,9 @@ of the first layers of a launch (after staging a phase's input, after the wait f
 the end of its own streaming loop, when the whole workgroup has finished it, after the epilogue).  The
 script decodes a few tokens of a model with the benchmark's widths, reads the stamps of the last launch
 and prints, per boundary, the minimum / median / maximum over the workgroups, the step from the previous
-boundary (median), and a one-line summary of a steady-state layer.  Numbers are microseconds since the
-first workgroup started."""
+boundary (median), a one-line summary of a steady-state layer, the steps inside the attention of one layer
+and the steps inside the staging function of one workgroup.  Numbers are microseconds since the first
+workgroup started."""
 import ctypes
 import importlib.util
 import os
@@ -80,6 +81,18 @@ def main():
         labels = ("entered", "q, k, v and the keys there", "scores and maximum", "softmax", "values summed")
         print("attention of layer 2, us after the workgroup's q|k|v epilogue (median over the heads): " +
               ", ".join("%s %.2f" % (lab, float(np.median(rel[:, k]))) for k, lab in enumerate(labels)))
+    # inside the staging function (workgroup 101, layer 2): six stamps per phase, relative to the moment the last
+    # workgroup finished the epilogue of the phase before
+    if n_layers >= 3 and n_wg > 101:
+        fine = buf[n_wg * 64 + 512:n_wg * 64 + 512 + 32].reshape(4, 8)
+        t0 = tl[:, 0].min()
+        before = {"qkv": "w2 fin l1", "wo": "qkv fin l2", "w13": "wo fin l2", "w2": "w13 fin l2"}
+        labels = ("entered", "first poll back", "its words there", "all wavefronts' there", "its blocks quantised", "all quantised")
+        for k, ph in enumerate(PHASES):
+            last = float(us[:, names.index(before[ph])].max())
+            f = (fine[k][:6] - t0) * 0.01 - last
+            print("staging for %-3s (workgroup 101, layer 2), us after the last workgroup's previous epilogue: " % ph +
+                  ", ".join("%s %+.2f" % (lab, float(v)) for lab, v in zip(labels, f)))
     dev.close()
 
 
