@@ -310,8 +310,21 @@ __device__ __forceinline__ void flow_drain(Ring &r) {
 // SRC: where the input comes from
 #define SRC_EMB 0     // the embedding row of `tok`
 #define SRC_BARE 2    // fp32 words; a word is there when it is not FLOW_EMPTY
-// The embedding and norm weights come with vectors of dim <= 4096 only (one q8_K block per wavefront);
-// the words of the hidden vector take up to four rounds.
+#define FULL(V_) (V_.x != FLOW_EMPTY && V_.y != FLOW_EMPTY && V_.z != FLOW_EMPTY && V_.w != FLOW_EMPTY)
+// Four q8_K blocks per wavefront throughout (q8k_quantize_rows16): a block per row of 16 lanes, a group of 16 values per
+// lane.  With a block per wavefront — sixteen wavefronts, four to a SIMD, each through its own chain of reductions and
+// divisions for 256 values — the 56 blocks of the hidden vector took 2.4 us of every workgroup's vector pipes, most of it
+// after the last word had arrived, and the 16 blocks of a dim-long vector 1.3 us.
+//
+// A vector that is only quantised (attention output, SwiGLU output): wavefront w waits for blocks 4w .. 4w+3 itself, a
+// lane for its 16 words (four 16-byte loads), and quantises them when all are there; one barrier.
+//
+// A vector that is normalised first (the embedding and norm weights come with dim <= 4096 only: at most 16 blocks) is
+// waited for by all sixteen wavefronts, a block each, which also form the sum of squares; its raw values then go through
+// LDS to the first four wavefronts, which normalise and quantise.  Block b waits in the part of the activation area
+// that nothing else uses while a dim-long vector is staged — except that the last block of each of the four wavefronts
+// waits where that same wavefront's quants go (it reads before it writes), and the last two of the others behind the
+// activation area.
 template <int PRO, int SRC>
 __device__ __noinline__ bool flow_stage(const void *src, int K, const float *normw, int tok) {
     src = uni(src), K = uni(K), normw = uni(normw), tok = uni(tok);
@@ -321,130 +334,125 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
     float *s_d = (float *)(s_qs + 14336 + 1792);
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nb = K >> 8;
-    static_assert(STAGE_MAX_ROUNDS == 4, "four rounds below");
-    const int rounds = nb > wave ? (nb - wave + FLOW_NW - 1) / FLOW_NW : 0;  // q8_K blocks of this wavefront
     constexpr bool rms = PRO == PRO_RMSNORM;
-    float xv[4][4];
-    float nw16[16];
+    static_assert(rms || SRC == SRC_BARE, "a vector that is only quantised arrives as bare words");
+    const int row_b = 4 * wave + (lane >> 4), g16 = lane & 15;  // block and group of this lane where a row is a block
+    const bool there = row_b < nb;  // (a row without a block works on block 0's numbers and stores nothing)
     bool ok = true;
     STG();  // entered
-    // A vector that is normalised first (K <= 4096: at most one block per wavefront) is waited for by all sixteen
-    // wavefronts, a block each, which also form the sum of squares; its raw values then go through LDS to the first four
-    // wavefronts, which normalise and quantise four blocks each, a block per row of 16 lanes (q8k_quantize_rows16): with a
-    // block per wavefront the sixteen of them spent 1.3 us in that arithmetic, four to a SIMD.  Block b waits in the part
-    // of the activation area that nothing else uses while a dim-long vector is staged — except that the last block of
-    // each of the four wavefronts waits where that same wavefront's quants go (it reads before it writes), and the last
-    // two of the others behind the activation area.
-    auto raw_of = [&](int b) -> float * {
-        const int w = b >> 2, r = b & 3, i = 3 * w + r;
-        const int at = r == 3 ? 256 * w : (i < 10 ? 1024 + 256 * i : FLOW_ACT_BYTES / 4 + 256 * (i - 10));
-        return (float *)s_act + at;
-    };
-    const int row_b = 4 * wave + (lane >> 4), g16 = lane & 15;  // (rms, first four wavefronts: block and group of this lane)
-    // one q8_K block of this wavefront: quantized and put into LDS
-    auto quantize_block = [&](int r, const float (&x4)[4]) {
-        const int b = wave + r * FLOW_NW;
-        uint32_t packed;
+    auto quads_store = [&](const float (&v)[16]) {
+        q8k_u32x4 packed;
         int bsum;
         float d;
-        q8k_quantize_wave(x4, packed, bsum, d);
-        ((uint32_t *)s_qs)[64 * b + lane] = packed;
-        if ((lane & 3) == 0) s_bs[16 * b + (lane >> 2)] = (int16_t)bsum;
-        if (lane == 0) s_d[b] = d;
+        q8k_quantize_rows16(v, packed, bsum, d);
+        if (there) {
+            ((q8k_u32x4 *)s_qs)[16 * row_b + g16] = packed;
+            s_bs[16 * row_b + g16] = (int16_t)bsum;
+            if (g16 == 0) s_d[row_b] = d;
+        }
     };
-    // A vector that is only quantized (no norm over the whole of it) is quantized block by block as the blocks become
-    // complete, while the words of slower producers are still being waited for: the q8_K area is free by now (its last
-    // readers, the previous phase's loops, ended before that phase's epilogue), and of the 2.4 µs that the 56 blocks of the
-    // SwiGLU vector take, most then lies inside the wait.
-    constexpr bool early = !rms && SRC == SRC_BARE;
-    unsigned done = 0u;  // (bit r: block r is in LDS)
-    // the norm weights are requested before the wait for the input: their latency passes meanwhile
-    if (rms && wave < 4) {
+    if constexpr (!rms) {
+        if (4 * wave < nb) {
+            u32x4v w0 = {FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY}, w1 = w0, w2 = w0, w3 = w0;
+            const unsigned *pb = (const unsigned *)src + 256 * (there ? row_b : 0) + 16 * g16;
+            unsigned spins = 0;
+            for (;;) {
+                // (a lane that has all its words does not ask again: waiting for a slow producer costs little traffic)
+                if (!(FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3))) POLL_BARE4(w0, w1, w2, w3, pb, pb + 4, pb + 8, pb + 12);
+                const bool all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
+                if (spins == 0) STG();  // the first poll is back
+                if (__ballot(!all) == 0ull) break;
+                if (++spins > a.spin_limit ||
+                    ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                    ok = false;
+                    break;
+                }
+            }
+            STG();  // this wavefront's words are all there
+            const u32x4v ws[4] = {w0, w1, w2, w3};
+            float v[16];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            // (a row without a block works on block 0's numbers and stores nothing)
-            const float4 t = *(const float4 *)(normw + 256 * (row_b < nb ? row_b : 0) + 16 * g16 + 4 * q);
-            nw16[4 * q] = t.x;
-            nw16[4 * q + 1] = t.y;
-            nw16[4 * q + 2] = t.z;
-            nw16[4 * q + 3] = t.w;
+            for (int q = 0; q < 4; q++) {
+                v[4 * q] = __uint_as_float(ws[q].x);
+                v[4 * q + 1] = __uint_as_float(ws[q].y);
+                v[4 * q + 2] = __uint_as_float(ws[q].z);
+                v[4 * q + 3] = __uint_as_float(ws[q].w);
+            }
+            quads_store(v);
         }
-    }
-    if (SRC == SRC_EMB) {
-        if (rounds > 0)
-#pragma unroll
-            for (int k = 0; k < 4; k++) xv[0][k] = dequant_elem(a.emb, tok, 256 * wave + 4 * lane + k);
+        if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
+        STG();  // this wavefront's blocks are in LDS
+        __syncthreads();
+        STG();  // everybody's
+        if (s_flag) {
+            if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return false;
+        }
+        return true;
     } else {
-        unsigned spins = 0;
-        // round r in w<r>; all start as "not there"
-        u32x4v w0 = {FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY}, w1 = w0, w2 = w0, w3 = w0;
-        const unsigned *pb = (const unsigned *)src + 256 * wave + 4 * lane;
-        for (;;) {
-            bool all = true;
-            // (a lane that has all its words does not ask again: waiting for a slow producer costs little traffic)
-#define FULL(V_) (V_.x != FLOW_EMPTY && V_.y != FLOW_EMPTY && V_.z != FLOW_EMPTY && V_.w != FLOW_EMPTY)
-            if (rounds == 1) {
+        const bool mine = wave < nb;  // this wavefront waits for block `wave`
+        float xv[4] = {0.f, 0.f, 0.f, 0.f};
+        float nw16[16];
+        auto raw_of = [&](int b) -> float * {
+            const int w = b >> 2, r = b & 3, i = 3 * w + r;
+            const int at = r == 3 ? 256 * w : (i < 10 ? 1024 + 256 * i : FLOW_ACT_BYTES / 4 + 256 * (i - 10));
+            return (float *)s_act + at;
+        };
+        // the norm weights are requested before the wait for the input: their latency passes meanwhile
+        if (wave < 4) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                // (a global load: through a plain pointer it would be a flat one, which the LDS waits below would wait for)
+                typedef float f32x4v __attribute__((ext_vector_type(4)));
+                const f32x4v t = *(const AS1 f32x4v *)(normw + 256 * (there ? row_b : 0) + 16 * g16 + 4 * q);
+                nw16[4 * q] = t.x;
+                nw16[4 * q + 1] = t.y;
+                nw16[4 * q + 2] = t.z;
+                nw16[4 * q + 3] = t.w;
+            }
+        }
+        if (SRC == SRC_EMB) {
+            if (mine)
+#pragma unroll
+                for (int k = 0; k < 4; k++) xv[k] = dequant_elem(a.emb, tok, 256 * wave + 4 * lane + k);
+        } else if (mine) {
+            unsigned spins = 0;
+            u32x4v w0 = {FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY, FLOW_EMPTY};
+            const unsigned *pb = (const unsigned *)src + 256 * wave + 4 * lane;
+            for (;;) {
                 if (!FULL(w0)) POLL_BARE1(w0, pb);
-                all = FULL(w0);
-            } else if (rounds == 2) {
-                if (!(FULL(w0) && FULL(w1))) POLL_BARE2(w0, w1, pb, pb + 256 * FLOW_NW);
-                all = FULL(w0) && FULL(w1);
-            } else if (rounds == 3) {
-                if (!(FULL(w0) && FULL(w1) && FULL(w2))) POLL_BARE3(w0, w1, w2, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW);
-                all = FULL(w0) && FULL(w1) && FULL(w2);
-            } else if (rounds == 4) {
-                if (!(FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3)))
-                    POLL_BARE4(w0, w1, w2, w3, pb, pb + 256 * FLOW_NW, pb + 512 * FLOW_NW, pb + 768 * FLOW_NW);
-                all = FULL(w0) && FULL(w1) && FULL(w2) && FULL(w3);
+                const bool all = FULL(w0);
+                if (spins == 0) STG();  // the first poll is back
+                if (__ballot(!all) == 0ull) break;
+                if (++spins > a.spin_limit ||
+                    ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+                    ok = false;
+                    break;
+                }
             }
-            if (spins == 0) STG();  // the first poll is back
-            if (early) {
-                const u32x4v wr[4] = {w0, w1, w2, w3};
+            STG();  // this wavefront's words are all there
+            xv[0] = __uint_as_float(w0.x);
+            xv[1] = __uint_as_float(w0.y);
+            xv[2] = __uint_as_float(w0.z);
+            xv[3] = __uint_as_float(w0.w);
+        }
+        if (!ok) s_flag = 1;
+        {  // rmsnorm! (reference src/inference.jl:102-110)
+            double acc = 0.0;
+            if (mine) {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (r < rounds && !(done & (1u << r)) && __ballot(!FULL(wr[r])) == 0ull) {
-                        const float x4[4] = {__uint_as_float(wr[r].x), __uint_as_float(wr[r].y), __uint_as_float(wr[r].z),
-                                             __uint_as_float(wr[r].w)};
-                        quantize_block(r, x4);
-                        done |= 1u << r;
-                    }
+                for (int k = 0; k < 4; k++) acc = fma((double)xv[k], (double)xv[k], acc);
             }
-#undef FULL
-            if (__ballot(!all) == 0ull) break;
-            if (++spins > a.spin_limit ||
-                ((spins & 63) == 0 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-                ok = false;
-                break;
-            }
+            acc = wave_sum_f64_dpp(acc);
+            if (lane == 0) s_red[wave] = acc;
+            if (mine) *(float4 *)(raw_of(wave) + 4 * lane) = make_float4(xv[0], xv[1], xv[2], xv[3]);
         }
-        STG();  // this wavefront's words are all there
-        const u32x4v ws[4] = {w0, w1, w2, w3};
-#pragma unroll
-        for (int r = 0; r < 4; r++) {
-            xv[r][0] = __uint_as_float(ws[r].x);
-            xv[r][1] = __uint_as_float(ws[r].y);
-            xv[r][2] = __uint_as_float(ws[r].z);
-            xv[r][3] = __uint_as_float(ws[r].w);
+        __syncthreads();
+        STG();  // every wavefront's are
+        if (s_flag) {
+            if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return false;
         }
-    }
-    if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
-    if (rms) {  // rmsnorm! (reference src/inference.jl:102-110)
-        double acc = 0.0;
-        if (rounds > 0) {
-#pragma unroll
-            for (int k = 0; k < 4; k++) acc = fma((double)xv[0][k], (double)xv[0][k], acc);
-        }
-        acc = wave_sum_f64_dpp(acc);
-        if (lane == 0) s_red[wave] = acc;
-        if (rounds > 0) *(float4 *)(raw_of(wave) + 4 * lane) = make_float4(xv[0][0], xv[0][1], xv[0][2], xv[0][3]);
-    }
-    __syncthreads();
-    STG();  // every wavefront's are
-    if (s_flag) {
-        if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        return false;
-    }
-    if (rms) {
         if (wave < 4) {
             double t = 0.0;
             for (int w = 0; w < FLOW_NW; w++) t += s_red[w];
@@ -452,7 +460,6 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
             ss /= (float)K;
             ss += 1e-5f;
             ss = 1.0f / sqrtf(ss);
-            const bool there = row_b < nb;
             const float *xr = raw_of(there ? row_b : 0) + 16 * g16;
             float v[16];
 #pragma unroll
@@ -463,26 +470,15 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
                 v[4 * q + 2] = nw16[4 * q + 2] * (ss * x4.z);
                 v[4 * q + 3] = nw16[4 * q + 3] * (ss * x4.w);
             }
-            q8k_u32x4 packed;
-            int bsum;
-            float d;
-            q8k_quantize_rows16(v, packed, bsum, d);
-            if (there) {
-                ((q8k_u32x4 *)s_qs)[16 * row_b + g16] = packed;
-                s_bs[16 * row_b + g16] = (int16_t)bsum;
-                if (g16 == 0) s_d[row_b] = d;
-            }
+            quads_store(v);
         }
-    } else if (!early) {
-#pragma unroll
-        for (int r = 0; r < 4; r++)
-            if (r < rounds && (SRC == SRC_BARE || r == 0)) quantize_block(r, xv[r]);
+        STG();  // this wavefront's blocks are in LDS
+        __syncthreads();
+        STG();  // everybody's
+        return true;
     }
-    STG();  // this wavefront's blocks are in LDS
-    __syncthreads();
-    STG();  // everybody's
-    return true;
 }
+#undef FULL
 
 // ------------------------------------------------------------------------------------------
 // the arithmetic of one phase for one workgroup: pieces from the ring x q8_K activations in LDS

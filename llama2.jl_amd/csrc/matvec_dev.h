@@ -471,20 +471,19 @@ __device__ __forceinline__ void q8k_quantize_rows16(const float (&v)[16], q8k_u3
     }
     const bool zero = rmax == 0.0f;
     const float iscale = zero ? 0.0f : -127.0f / bmx;
-    int sum = 0;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
 #pragma unroll
     for (int b = 0; b < 16; b++) {
         int q = (int)rintf(iscale * v[b]);
         q = q < 127 ? q : 127;
-        sum += (int)(int8_t)q;
         w[b >> 2] |= ((uint32_t)(q & 0xFF)) << (8 * (b & 3));
     }
     packed.x = w[0];
     packed.y = w[1];
     packed.z = w[2];
     packed.w = w[3];
-    bsum = sum;
+    // the group's sum of the quants as stored (int8): four signed byte dot products with ones
+    bsum = sdot4(w[3], 0x01010101u, sdot4(w[2], 0x01010101u, sdot4(w[1], 0x01010101u, sdot4(w[0], 0x01010101u, 0))));
     d = zero ? 0.0f : 1.0f / iscale;
 }
 

@@ -87,10 +87,13 @@ def main():
         fine = buf[n_wg * 64 + 512:n_wg * 64 + 512 + 32].reshape(4, 8)
         t0 = tl[:, 0].min()
         before = {"qkv": "w2 fin l1", "wo": "qkv fin l2", "w13": "wo fin l2", "w2": "w13 fin l2"}
-        labels = ("entered", "first poll back", "its words there", "all wavefronts' there", "its blocks quantised", "all quantised")
         for k, ph in enumerate(PHASES):
+            # (a vector that is normalised has a barrier of its own after the wait; one that is only quantised has not)
+            labels = (("entered", "first poll back", "its words there", "all wavefronts' there", "its blocks quantised",
+                       "all quantised") if ph in ("qkv", "w13") else
+                      ("entered", "first poll back", "its words there", "its blocks quantised", "all quantised"))
             last = float(us[:, names.index(before[ph])].max())
-            f = (fine[k][:6] - t0) * 0.01 - last
+            f = (fine[k][:len(labels)] - t0) * 0.01 - last
             print("staging for %-3s (workgroup 101, layer 2), us after the last workgroup's previous epilogue: " % ph +
                   ", ".join("%s %+.2f" % (lab, float(v)) for lab, v in zip(labels, f)))
     dev.close()
