@@ -1289,7 +1289,9 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
     const int p16 = lane & 15, part = lane >> 4, t = 16 * wave + p16;
     const int i4 = tid & (n4p - 1), grp = tid / n4p;
     const bool v_lane = n4p == n4 || i4 < n4;
-    float4 kv[per], v[NV];
+    typedef float f32x4v __attribute__((ext_vector_type(4)));  // (one 128-bit register: a struct's four floats get split up)
+    float4 kv[per];
+    f32x4v v[NV];
     {
         const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
 #pragma unroll
@@ -1322,18 +1324,18 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
             }
         }
         // the values are requested now (the keys' registers are free): they arrive during the softmax
-        const float4 *vp = (const float4 *)(vc + (int64_t)kvh * seq_len * hs) + i4;
+        // (No lane-dependent branch around a load and no choice of source at it: either makes the compiler wait for the
+        // loads one by one.  A wavefront skips the loads none of whose timesteps is in the cache — a scalar branch — and
+        // within a load a lane without a row, or beyond the head size, reads row 0; what the lane really sums is picked
+        // after the softmax, when the loads have long landed.)
+        const f32x4v *vp0 = (const f32x4v *)(vc + (int64_t)kvh * seq_len * hs) + (v_lane ? i4 : 0);
+        const int grp0 = (wave * 64) / n4p;  // the wavefront's first timestep group
 #pragma unroll
         for (int u = 0; u < NV; u++) {
             const int tv = grp + u * ngrp;
-            v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (v_lane && tv < pos) v[u] = vp[(int64_t)tv * n4];
+            v[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
+            if (grp0 + u * ngrp < pos) v[u] = vp0[(int64_t)(tv < pos ? tv : 0) * n4];
         }
-        // (the current position's row comes from LDS, after all the loads are out: a choice between the two sources at
-        // each load makes the compiler wait for every load in turn)
-#pragma unroll
-        for (int u = 0; u < NV; u++)
-            if (v_lane && grp + u * ngrp == pos) v[u] = ((const float4 *)s_vcur)[i4];
         // the quarters are added in order (fp64)
         const double a1 = __shfl(acc, p16 + 16, WAVE), a2 = __shfl(acc, p16 + 32, WAVE), a3 = __shfl(acc, p16 + 48, WAVE);
         if (part == 0 && t < np) sc = (float)(((acc + a1) + a2) + a3) / scale;
@@ -1361,6 +1363,8 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
 #pragma unroll
         for (int u = 0; u < NV; u++) {
             const int tv = grp + u * ngrp;
+            if (tv == pos) v[u] = ((const f32x4v *)s_vcur)[v_lane ? i4 : 0];  // (the current position's row comes from LDS)
+            if (!v_lane) v[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
             if (tv < np) {
                 const double p = s_p[tv];
                 acc[0] = fma(p, (double)v[u].x, acc[0]);
