@@ -1267,6 +1267,23 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
 #define ATL()
 #endif
     ATL();
+    // scores: lane = (timestep p16 of the wavefront's 16, quarter of the head dimension);
+    // values: thread = (16-byte group i4 of the head dimension, timestep group grp), timesteps grp + u * ngrp
+    const int p16 = lane & 15, part = lane >> 4, t = 16 * wave + p16;
+    const int i4 = tid & (n4p - 1), grp = tid / n4p;
+    const bool v_lane = n4p == n4 || i4 < n4;
+    typedef float f32x4v __attribute__((ext_vector_type(4)));  // (one 128-bit register: a struct's four floats get split up)
+    f32x4v kv[per], v[NV];
+    // The keys are requested first of all, before the wait for q: a wavefront none of whose timesteps is in the cache skips
+    // them (a scalar branch), a lane beyond the cache reads timestep 0 and does not use it.
+    {
+        const f32x4v *kp = (const f32x4v *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + (t < pos ? t : 0);
+#pragma unroll
+        for (int u = 0; u < per; u++) {
+            kv[u] = f32x4v{0.f, 0.f, 0.f, 0.f};
+            if (16 * wave < pos) kv[u] = kp[(int64_t)u * seq_len];
+        }
+    }
     __syncthreads();  // the activation area is free
     if (tid < 3 * hs) {
         const int which = tid / hs, i = tid % hs;
@@ -1284,20 +1301,6 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
         s_q[tid] = tag_val(w);  // s_q, s_kcur, s_vcur lie one behind the other
     }
     if (!ok) s_flag = 1;
-    // scores: lane = (timestep p16 of the wavefront's 16, quarter of the head dimension);
-    // values: thread = (16-byte group i4 of the head dimension, timestep group grp), timesteps grp + u * ngrp
-    const int p16 = lane & 15, part = lane >> 4, t = 16 * wave + p16;
-    const int i4 = tid & (n4p - 1), grp = tid / n4p;
-    const bool v_lane = n4p == n4 || i4 < n4;
-    typedef float f32x4v __attribute__((ext_vector_type(4)));  // (one 128-bit register: a struct's four floats get split up)
-    float4 kv[per];
-    f32x4v v[NV];
-    {
-        const float4 *kp = (const float4 *)kc + ((int64_t)kvh * (hs >> 2) + part * per) * seq_len + t;
-#pragma unroll
-        for (int u = 0; u < per; u++)
-            if (t < pos) kv[u] = kp[(int64_t)u * seq_len];
-    }
     __syncthreads();
     if (s_flag) {
         if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1307,7 +1310,7 @@ __device__ __noinline__ bool flow_attention_short(int layer, int h, int pos, uns
     // the current position's key and value are in LDS, the earlier ones came from the cache
     if (t == pos) {
 #pragma unroll
-        for (int u = 0; u < per; u++) kv[u] = ((const float4 *)s_kcur)[part * per + u];
+        for (int u = 0; u < per; u++) kv[u] = ((const f32x4v *)s_kcur)[part * per + u];
     }
     const float scale = sqrtf((float)hs);
     float sc = -INFINITY;
