@@ -1009,13 +1009,25 @@ __device__ __forceinline__ void flow_row_values(int n_local, int ppr) {
 
 // the same for one row, straight from the partial sums (the layer epilogues: one barrier instead of two)
 __device__ __forceinline__ float flow_row_value4(int lr, int ppr) {
+    const double *q4 = s_part + 4 * lr * ppr;
     double v = 0.0;
-    for (int p = 0; p < ppr; p++) {
-        const double *q4 = s_part + 4 * (lr * ppr + p);
-        v += (q4[0] + q4[1]) + (q4[2] + q4[3]);
+    // (the quarter sums of up to four pieces are read before any is added: one LDS latency per four pieces, not per piece)
+    for (int p0 = 0; p0 < ppr; p0 += 4) {
+        double q[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (p0 + i < ppr) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) q[i][k] = q4[4 * (p0 + i) + k];
+            }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            if (p0 + i < ppr) v += (q[i][0] + q[i][1]) + (q[i][2] + q[i][3]);
     }
     return (float)v;
 }
+// the value of the row next to this thread's (tid ^ 1), which that thread has just formed in the same way
+__device__ __forceinline__ float flow_pair_value(float own) { return dpp_f32<DPP_QUAD_SWAP1>(own); }
 
 // ---- epilogues -------------------------------------------------------------------------------
 // (The layer epilogues are inlined: a function waits before it returns for its stores to be acknowledged,
@@ -1034,7 +1046,8 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
     const int L = wg * a.qkv.rpw + tid;
     int seg, row;
     flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row, ANY_HS);
-    const float val = flow_row_value4(tid, a.qkv.ppr), other = flow_row_value4(tid ^ 1, a.qkv.ppr);
+    // (rows come in pairs and a workgroup's run of them is even, so the partner's thread is here too)
+    const float val = flow_row_value4(tid, a.qkv.ppr), other = flow_pair_value(val);
     const int hs_log = 31 - __builtin_clz(a.hs);  // (a power of two unless ANY_HS)
     const int hh = ANY_HS ? row / a.hs : row >> hs_log, e = ANY_HS ? row - hh * a.hs : row & (a.hs - 1);
     if (seg == 2) {
@@ -1096,8 +1109,10 @@ __device__ __noinline__ unsigned flow_w13_word(int wg) {
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
     __syncthreads();
-    if (tid >= n_local || (tid & 1)) return 0u;
-    return bare_of(swiglu_val(flow_row_value4(tid, a.w13.ppr), flow_row_value4(tid + 1, a.w13.ppr)));
+    if (tid >= n_local) return 0u;
+    const float own = flow_row_value4(tid, a.w13.ppr), next = flow_pair_value(own);  // (w1 row u | w3 row u, threads 2u | 2u+1)
+    if (tid & 1) return 0u;
+    return bare_of(swiglu_val(own, next));
 }
 __device__ __forceinline__ void flow_finish_w13(int wg, unsigned e_out) {
     const FlowArgs &a = c_flow;
