@@ -26,9 +26,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
 # HBM traffic of the dominant kernel per launch, from rocprofv3 --pmc runs of this script (FETCH_SIZE x 2.000 KiB +
 # WRITE_SIZE x 1.000 KiB per unit, the factors a plain read of known size gave in the same runs):
 #   (workload, launch path 1): per matvec launch, 31.23 MB read + 0.04 MB written (profiles/pmc_fetch_write_bench_8b-q4ks.md)
-#   (workload, launch path 3): per token launch, 4489.4 MB read + 9.3 MB written (profiles/pmc_fetch_write_bench_8b-q4ks_streaming.md);
+#   (workload, launch path 3): per token launch, 4486.3 MB read + 9.3 MB written (profiles/pmc_fetch_write_bench_8b-q4ks_streaming.md);
 #   8b-q5km: 5755.5 MB read + 9.3 MB written (profiles/kernel_stats_bench_8b-q5km.md)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4498700000, ("8b-q5km", 3): 5764800000}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4495700000, ("8b-q5km", 3): 5764800000}
 
 WORKLOADS = {
     # name: (plan, config kwargs, prompt length)
