@@ -168,7 +168,10 @@ int l2h_state_read(l2h_model *m, int which, float *host, int64_t n);
 
 /* ---- single operators (each is the device form of one reference function) ----------- */
 /* quantize x[n] (n % 256 == 0) to block_q8_K records (src/kquants.jl:37-42: f32 d,
- * i8 qs[256], i16 bsums[16]; 292 bytes each) with llama.cpp's quantize_row_q8_K rule. */
+ * i8 qs[256], i16 bsums[16]; 292 bytes each) with llama.cpp's quantize_row_q8_K rule.
+ * The library holds two forms of this quantizer (a block per wavefront in the per-phase
+ * kernels, four blocks per wavefront in the streaming kernel); the call runs both and
+ * fails with L2H_EHIP if their outputs differ. */
 int l2h_quantize_q8k(l2h_ctx *ctx, const float *x, int64_t n, void *out_blocks);
 /* dequantize!(y, x) (src/kquants.jl:44,70,186,322): nb blocks -> 256*nb floats
  * (F32: nb elements copied). */

@@ -1417,13 +1417,30 @@ extern "C" int l2h_quantize_q8k(l2h_ctx *ctx, const float *x, int64_t n, void *o
     std::vector<void *> tr;
     int rc = q8_alloc(ctx, n, &q, &tr);
     if (rc) return rc;
+    // The library has two forms of this quantizer: a block per wavefront (the per-phase kernels' prologue) and four
+    // blocks per wavefront (the streaming kernel's staging).  Both run here and must agree byte for byte.
+    Q8Dev q2;
+    std::vector<void *> tr2;
+    rc = q8_alloc(ctx, n, &q2, &tr2);
+    if (rc) {
+        (void)hipFree(tr[0]);
+        return rc;
+    }
     hipError_t e = k_stage_dump(ctx->stream, dx.as<float>(), nullptr, n, PRO_QUANT, q, nullptr);
+    if (e == hipSuccess) e = k_quantize_rows16(ctx->stream, dx.as<float>(), n, q2);
     if (e == hipSuccess) e = hipStreamSynchronize(ctx->stream);
-    if (e == hipSuccess)
+    if (e == hipSuccess) {
+        const size_t bytes = (size_t)(n / QK_K) * 292;
+        std::vector<unsigned char> other(bytes);
         rc = q8_pack_blocks(ctx, q, n, out_blocks);
-    else
+        if (rc == L2H_OK) rc = q8_pack_blocks(ctx, q2, n, other.data());
+        if (rc == L2H_OK && memcmp(other.data(), out_blocks, bytes) != 0)
+            rc = set_err(ctx, L2H_EHIP, "the two forms of the q8_K quantizer disagree");
+    } else {
         rc = set_err(ctx, L2H_EHIP, "quantize failed: %s", hipGetErrorString(e));
+    }
     (void)hipFree(tr[0]);
+    (void)hipFree(tr2[0]);
     return rc;
 }
 

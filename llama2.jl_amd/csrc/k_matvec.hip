@@ -184,6 +184,33 @@ __global__ __launch_bounds__(1024) void stage_dump_kernel(PhaseArgs a, int64_t n
     }
 }
 
+// quantize_row_q8_K with four blocks per wavefront, a block per row of 16 lanes: the form in which the streaming decode
+// kernel stages its inputs (q8k_quantize_rows16); the stand-alone quantizer runs it beside the one-block-per-wavefront
+// form and compares, so that its tests pin both
+__global__ __launch_bounds__(64) void quantize_rows16_kernel(const float *x, int64_t nb, Q8Dev out) {
+    const int lane = threadIdx.x, g = lane & 15;
+    const int64_t b = 4 * (int64_t)blockIdx.x + (lane >> 4);
+    const bool there = b < nb;  // (a row without a block works on zeros and stores nothing)
+    float v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) v[k] = there ? x[256 * b + 16 * g + k] : 0.0f;
+    q8k_u32x4 packed;
+    int bsum;
+    float d;
+    q8k_quantize_rows16(v, packed, bsum, d);
+    if (there) {
+        ((q8k_u32x4 *)out.qs)[16 * b + g] = packed;
+        out.bsums[16 * b + g] = (int16_t)bsum;
+        if (g == 0) out.d[b] = d;
+    }
+}
+
+hipError_t k_quantize_rows16(hipStream_t s, const float *x, int64_t n, Q8Dev q8_out) {
+    const int64_t nb = n / 256;
+    hipLaunchKernelGGL(quantize_rows16_kernel, dim3((unsigned)((nb + 3) / 4)), dim3(64), 0, s, x, nb, q8_out);
+    return hipGetLastError();
+}
+
 hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64_t n, int pro, Q8Dev q8_out,
                         float *f32_out) {
     PhaseArgs a{};

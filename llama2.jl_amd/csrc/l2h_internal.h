@@ -217,6 +217,8 @@ hipError_t k_mega_bind(hipStream_t s, const PhaseArgs *ph);
 hipError_t k_mega_launch(hipStream_t s, const MegaArgs &g, int t_qkv, int t_wo, int t_w13, int t_w2, int t_out, int grid,
                          size_t lds);
 hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64_t n, int pro, Q8Dev q8_out, float *f32_out);
+// the same quantization in the streaming decode kernel's form (four blocks per wavefront)
+hipError_t k_quantize_rows16(hipStream_t s, const float *x, int64_t n, Q8Dev q8_out);
 hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
 // kv16: the caches hold fp16 elements (needs head_size <= 128, a multiple of 16)
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,

@@ -51,6 +51,25 @@ def _q8_cases(rng):
         x[256 * b + i] = m if b % 2 else -m
         x[256 * b + j] = -m if b % 2 else m
     cases["ties"] = x
+    # the same with many blocks and with both holders inside one group of 16, in neighbouring groups, or far apart (the
+    # streaming kernel's form of the quantizer searches a lane's 16 values by a tree and a block's 16 lanes by ballot)
+    x = rng.uniform(-1, 1, 256 * 66).astype(np.float32)  # (66 blocks: the last group of four is half filled)
+    for b in range(66):
+        m = np.float32(2.0 + 0.25 * b)
+        g = int(rng.integers(0, 16))
+        if b % 3 == 0:
+            i, j = sorted(rng.choice(16, 2, replace=False) + 16 * g)
+        elif b % 3 == 1:
+            i, j = 16 * g + int(rng.integers(0, 16)), 16 * ((g + 1) % 16) + int(rng.integers(0, 16))
+            i, j = min(i, j), max(i, j)
+        else:
+            i, j = sorted(rng.choice(256, 2, replace=False))
+        x[256 * b + i] = m if b % 2 else -m
+        x[256 * b + j] = -m if b % 2 else m
+        if b % 5 == 0:  # a third holder, later still
+            k = int(rng.integers(j, 256))
+            x[256 * b + k] = m
+    cases["ties_many"] = x
     x = np.zeros(512, np.float32)
     x[:256] = (np.arange(256) - 127.5) / 127.0  # exact half-way products iscale*x = k + 0.5
     x[0] = -1.0
