@@ -465,6 +465,7 @@ SHAPES = [
     ("PLAN_Q5_K_M", 4096, 4096, 1, 32, 32, 1031, True),
     (dict(emb=12, output=14, wq=14, wk=14, wv=14, wo=14, w1=14, w3=14, w2=14), 4096, 2048, 2, 64, 8, 300, False),
     ("PLAN_Q4_K", 3072, 4096, 1, 32, 8, 777, False),
+    ("PLAN_Q4_K", 1536, 2048, 2, 16, 4, 333, False),  # six q8_K blocks per dim-long vector: a group of four half filled
     ("PLAN_F32", 512, 708, 2, 8, 2, 1001, False),
     ("PLAN_F32", 1024, 2048, 1, 16, 16, 130, True),
 ]
