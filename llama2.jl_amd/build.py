@@ -1,23 +1,12 @@
 """Builds libl2hip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
 
-Usage:  python llama2.jl_amd/build.py [--timeline | --microbench]
+Usage:  python llama2.jl_amd/build.py [--timeline]
 The objects are compiled in parallel (one hipcc per source file) and linked into
 llama2.jl_amd/libl2hip.so.  hipcc cross-compiles: no GPU is needed to build.
 
 --timeline builds llama2.jl_amd/libl2hip_tl.so instead: the same library with -DL2H_TIMELINE, in which the
 streaming decode kernel stamps the wall clock at every phase boundary (llama2.jl_amd/timeline.py prints
 the table).  The product library is not touched.
-
---microbench builds nine stand-alone programs into llama2.jl_amd/build_mb/ (csrc/microbench/): `stream` (how fast
-256 x 16 wavefronts read bytes in the access patterns of the streaming decode kernel), `loop` (that kernel's q4_K
-piece loop alone, with and without its fetches), `exchange` (one "every workgroup reads the whole vector"
-hand-over through device memory), `tile` (the q4_K arithmetic with a lane per super-block instead of a lane per 32
-weights, operands resident in LDS), `dma_rate` (how fast 1, 2, 4, 8 or 16 wavefronts per CU stream with
-global_load_lds alone), `l2share` (what a workgroup gains when another one of its XCD, or of another XCD, has just
-read the same bytes), `prefetch` (a model of a decode layer in which some workgroups of every XCD only pull the
-weight streams towards the caches ahead of the others), `pollmix` (how long a poll of uncached memory takes while
-its own wavefront, its CU's other wavefronts, or other CUs stream) and `pingpong` (the one-way latency of a word
-handed from one workgroup to another).  Each prints a table; run them on the GPU without arguments.
 """
 import concurrent.futures
 import os
@@ -85,23 +74,6 @@ def build(force=True, verbose=True, timeline=False):
     return lib
 
 
-def build_microbench(verbose=True):
-    out = os.path.join(HERE, "build_mb")
-    os.makedirs(out, exist_ok=True)
-    for name in ("stream", "loop", "exchange", "tile", "dma_rate", "l2share", "prefetch", "pollmix", "pingpong"):
-        exe = os.path.join(out, name)
-        cmd = [_hipcc(), os.path.join(CSRC, "microbench", name + ".hip"), "-o", exe, "-O3", "-std=c++17", "-ffp-contract=off",
-               "-I", os.path.join(ROOT, "include"), "-I", CSRC] + DEVICE
-        r = subprocess.run(cmd, capture_output=True, text=True)
-        if r.returncode != 0:
-            raise RuntimeError("hipcc failed on %s:\n%s" % (name, r.stdout + r.stderr))
-        if verbose:
-            print("built", exe)
-
-
 if __name__ == "__main__":
-    if "--microbench" in sys.argv[1:]:
-        build_microbench()
-    else:
-        build(force=True, timeline="--timeline" in sys.argv[1:])
+    build(force=True, timeline="--timeline" in sys.argv[1:])
     sys.exit(0)
