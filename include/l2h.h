@@ -100,10 +100,16 @@ int l2h_model_set_kv_type(l2h_model *m, int kv_type);
 /* How transformer! is launched (before finalize): 0 = automatic (3 where the model fits it, else 1),
  * 1 = one kernel per phase (recorded once, replayed per token), 2 = a persistent kernel per token
  * with grid barriers between the phases, 3 = the streaming kernel per token (per-wavefront weight
- * streams fetched ahead into LDS, activations exchanged as epoch-tagged words; needs q4_K, q5_K or
- * q6_K layer matrices with a q4_K or q6_K classifier, dim 2048, 3072 or 4096 and hidden_dim a multiple
- * of 2048 up to 14336 -- or a model of fp32 matrices with dim and hidden_dim up to 4096 in multiples of
- * 4 -- and a head size of 32, 64, 96 or 128; any cache length).
+ * streams fetched ahead into LDS, activations exchanged as epoch-tagged words).  Path 3 takes
+ *   - q4_K, q5_K or q6_K layer matrices (w1 and w3 of a layer of one type) with a q4_K or q6_K classifier:
+ *     dim a multiple of 256, at most 4096, and either a multiple of 2048 or at most a quarter below one
+ *     (1536..2048, 3072..4096; a q6_K classifier needs the multiple of 2048 above dim to be 4096);
+ *     hidden_dim a multiple of 2048 up to 14336; head size 32, 64, 96 or 128; fp32 or fp16 cache;
+ *   - models whose matrices are all fp32: dim and hidden_dim multiples of 4, at most 4096; head size 32, 64
+ *     or 128; fp32 cache;
+ *   in both cases n_heads <= 256, a head size that is a multiple of 256 / n_heads, and a cache length that fits
+ *   the attention's LDS area (with head size 128: about 2 400 positions times 256 / n_heads, e.g. 19 000
+ *   for 32 heads).
  * 2 and 3 are an error at finalize if the model does not fit; l2h_model_path_reason then tells why.  All paths compute the same
  * arithmetic and give the same results.  No counterpart in the reference.  l2h_model_path reports
  * the choice after finalize (1, 2 or 3). */
@@ -171,7 +177,9 @@ int l2h_state_read(l2h_model *m, int which, float *host, int64_t n);
  * i8 qs[256], i16 bsums[16]; 292 bytes each) with llama.cpp's quantize_row_q8_K rule.
  * The library holds two forms of this quantizer (a block per wavefront in the per-phase
  * kernels, four blocks per wavefront in the streaming kernel); the call runs both and
- * fails with L2H_EHIP if their outputs differ. */
+ * fails with L2H_EHIP if their outputs differ.  x must be finite (L2H_EINVAL otherwise: the
+ * rule's "first element of largest magnitude" is undefined for a NaN); inside the decode
+ * kernels a non-finite activation gives unspecified quants but no fault. */
 int l2h_quantize_q8k(l2h_ctx *ctx, const float *x, int64_t n, void *out_blocks);
 /* dequantize!(y, x) (src/kquants.jl:44,70,186,322): nb blocks -> 256*nb floats
  * (F32: nb elements copied). */

@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <cmath>
 
 #include <algorithm>
 #include <mutex>
@@ -780,7 +781,13 @@ static int flow_setup(l2h_model *m) {
     int64_t total = 0;
     FlowTypedTables tt;
     FlowTypedDev typed;
-    std::vector<void *> tmp;  // tables that only the repack kernels read
+    // tables that only the repack kernels read: freed on every way out of this function
+    struct TmpTables {
+        std::vector<void *> v;
+        ~TmpTables() {
+            for (void *p : v) (void)hipFree(p);
+        }
+    } tmp;
     int rc;
     if (a.mixed) {
         k_flow_typed_tables(a, types.data(), cls_type, grid, tt);
@@ -789,7 +796,7 @@ static int flow_setup(l2h_model *m) {
         auto up = [&](const void *src, size_t bytes, const void **dst) -> int {
             void *v = nullptr;
             HIPCHK(ctx, hipMalloc(&v, std::max<size_t>(bytes, 16)));
-            tmp.push_back(v);
+            tmp.v.push_back(v);
             HIPCHK(ctx, hipMemcpy(v, src, bytes, hipMemcpyHostToDevice));
             *dst = v;
             return L2H_OK;
@@ -797,10 +804,8 @@ static int flow_setup(l2h_model *m) {
         if ((rc = up(tt.piece_base.data(), tt.piece_base.size() * 8, (const void **)&typed.piece_base)) ||
             (rc = up(tt.cls_off.data(), tt.cls_off.size() * 8, (const void **)&typed.cls_off)) ||
             (rc = up(tt.piece_off.data(), tt.piece_off.size() * 8, (const void **)&typed.piece_off)) ||
-            (rc = up(tt.piece_tag.data(), tt.piece_tag.size() * 2, (const void **)&typed.piece_tag))) {
-            for (void *v : tmp) (void)hipFree(v);
+            (rc = up(tt.piece_tag.data(), tt.piece_tag.size() * 2, (const void **)&typed.piece_tag)))
             return rc;
-        }
         unsigned int *wt = nullptr;
         if ((rc = dalloc(m, &wt, (int64_t)tt.wave_types.size(), false))) return rc;
         HIPCHK(ctx, hipMemcpy(wt, tt.wave_types.data(), tt.wave_types.size() * 4, hipMemcpyHostToDevice));
@@ -827,7 +832,6 @@ static int flow_setup(l2h_model *m) {
     }
     if (!a.f32) HIPCHK(ctx, k_flow_repack(ctx->stream, a, stream, off_dev, 4, 0, &m->glob[L2H_OUTPUT], 1, grid, cls_type, typed));
     HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
-    for (void *v : tmp) HIPCHK(ctx, hipFree(v));
     a.stream = stream;
     a.wave_off = off_dev;
     // the exchanged words live in uncached memory, zeroed like any other allocation
@@ -1409,6 +1413,9 @@ extern "C" int l2h_quantize_q8k(l2h_ctx *ctx, const float *x, int64_t n, void *o
     if (!ctx || !x || !out_blocks) return set_err(ctx, L2H_EINVAL, "l2h_quantize_q8k: NULL argument");
     if (n < 0 || n % QK_K != 0) return set_err(ctx, L2H_EINVAL, "n = %lld is not a multiple of 256", (long long)n);
     if (n == 0) return L2H_OK;
+    // the rule's "first element of largest magnitude" has no meaning for a NaN, and an infinite extreme gives a scale of 0
+    for (int64_t i = 0; i < n; i++)
+        if (!std::isfinite(x[i])) return set_err(ctx, L2H_EINVAL, "x[%lld] is not finite", (long long)i);
     HIPCHK(ctx, hipSetDevice(ctx->device));
     DevBuf dx;
     HIPCHK(ctx, dx.alloc((size_t)n * 4));

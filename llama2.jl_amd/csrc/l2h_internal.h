@@ -220,7 +220,7 @@ hipError_t k_stage_dump(hipStream_t s, const float *x, const float *normw, int64
 // the same quantization in the streaming decode kernel's form (four blocks per wavefront)
 hipError_t k_quantize_rows16(hipStream_t s, const float *x, int64_t n, Q8Dev q8_out);
 hipError_t k_rope_only(hipStream_t s, float *x, int head_size, int n_heads, int pos, float theta_scale, int neox);
-// kv16: the caches hold fp16 elements (needs head_size <= 128, a multiple of 16)
+// kv16: the caches hold fp16 elements (needs head_size <= 128, a multiple of 32)
 hipError_t k_attention(hipStream_t s, const double *qd, const float *kc, const float *vc, float *att, double *pd,
                        double *part, float *out, const DecodeCtl *ctl, int head_size, int n_heads,
                        int n_kv_heads, int seq_len, int kv16);

@@ -420,7 +420,8 @@ __device__ __forceinline__ void q8k_quantize_wave(const float v[4], uint32_t &pa
     }
     const float wmax = wave_max_f32_dpp(amax);
     // lowest lane whose own extreme reaches the block's: its first such element is the block's first
-    const unsigned long long holders = __ballot(amax == wmax);
+    // (no lane holds it only where the block has a NaN: lane 0 then stands in, so that `first` is always a lane)
+    const unsigned long long held = __ballot(amax == wmax), holders = held | (unsigned long long)(held == 0ull);
     const int first = __builtin_ctzll(holders);
     const float bmx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx), first));
     // an all-zero block gives q = 0, d = 0 (no branch: several blocks' code can then be interleaved)
@@ -460,12 +461,14 @@ __device__ __forceinline__ void q8k_quantize_rows16(const float (&v)[16], q8k_u3
     rmax = fmaxf(rmax, dpp_f32<DPP_ROW_HALF_MIRROR>(rmax));
     rmax = fmaxf(rmax, dpp_f32<DPP_ROW_MIRROR>(rmax));
     // lowest lane of the row whose own extreme reaches the block's: its first such element is the block's first
-    // (on the scalar unit, a row at a time; a row's set is never empty: its maximum is some lane's)
+    // (on the scalar unit, a row at a time; a row's set is empty only where the block has a NaN: the row's lane 0 then
+    // stands in, so that `first` is always a lane of the row)
     const unsigned long long holders = __ballot(amax == rmax);
     float bmx = 0.0f;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-        const int first = 16 * r + __builtin_ctz((unsigned)(holders >> (16 * r)) & 0xFFFFu);
+        const unsigned row = (unsigned)(holders >> (16 * r)) & 0xFFFFu;
+        const int first = 16 * r + __builtin_ctz(row | (unsigned)(row == 0u));
         const float m = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx), first));
         bmx = (int)(threadIdx.x & 48u) == 16 * r ? m : bmx;
     }

@@ -77,9 +77,11 @@ def dummy_tokenizer(vocab_size):
     return BPETokenizer(toks[:vocab_size], [0.0] * vocab_size, 1, 2)
 
 
-def synthetic_model(config, plan, seed=1234, sigma=0.02, share_classifier=False):
+def synthetic_model(config, plan, seed=1234, sigma=0.02, share_classifier=False, norm_spread=0.2):
     """Random-init model of the given shape; stream ids are (layer, role) so any tensor can be
-    regenerated alone."""
+    regenerated alone.  The norm weights are seeded uniform(1 - norm_spread, 1 + norm_spread), different in
+    every layer and tensor, so that a wrong layer's or the wrong tensor's norm weights change the result;
+    norm_spread=0 gives all ones (what the benchmark configurations specify)."""
     c = config
     hs = c.dim // c.n_heads
     kv_dim = hs * c.n_kv_heads
@@ -88,17 +90,23 @@ def synthetic_model(config, plan, seed=1234, sigma=0.02, share_classifier=False)
         t = plan[role]
         return make_matrix(seed, stream, ne1, ne0, t[layer] if isinstance(t, (list, tuple)) else t, sigma)
 
+    def norm(stream):
+        if norm_spread == 0:
+            return np.ones(c.dim, np.float32)
+        rng = np.random.default_rng([seed, 7919, stream])
+        return rng.uniform(1.0 - norm_spread, 1.0 + norm_spread, c.dim).astype(np.float32)
+
     emb = mat(1, c.vocab_size, c.dim, "emb")
     layers = []
     for l in range(c.n_layers):
         s = 100 + 16 * l
         layers.append(TransformerLayerWeights(
-            rms_att_weight=np.ones(c.dim, np.float32), rms_ffn_weight=np.ones(c.dim, np.float32),
+            rms_att_weight=norm(s + 7), rms_ffn_weight=norm(s + 8),
             wq=mat(s + 0, c.dim, c.dim, "wq", l), wk=mat(s + 1, kv_dim, c.dim, "wk", l), wv=mat(s + 2, kv_dim, c.dim, "wv", l),
             wo=mat(s + 3, c.dim, c.dim, "wo", l), w1=mat(s + 4, c.hidden_dim, c.dim, "w1", l),
             w2=mat(s + 5, c.dim, c.hidden_dim, "w2", l), w3=mat(s + 6, c.hidden_dim, c.dim, "w3", l)))
     output = emb if share_classifier else mat(2, c.vocab_size, c.dim, "output")
-    weights = TransformerWeights(emb, layers, np.ones(c.dim, np.float32), output)
+    weights = TransformerWeights(emb, layers, norm(3), output)
     return LanguageModel(c, dummy_tokenizer(c.vocab_size), weights)
 
 

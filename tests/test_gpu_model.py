@@ -118,8 +118,8 @@ def test_distance_to_reference_float_arithmetic(pkg, orc, case):
     if plan == "PLAN_F32":
         assert errs.max() <= 1e-5 and agree == len(fed)
     else:
-        # the q8_K step: 8 bits per activation, about 0.7 % RMS per matvec
-        assert errs.max() <= 0.15
+        # the q8_K step: 8 bits per activation, about 0.7 % RMS per matvec; observed 0.02-0.05 and 39-44 of 45 positions
+        assert errs.max() <= 0.08 and agree >= 0.7 * len(fed)
     dev.close()
     om.close()
 
@@ -393,11 +393,26 @@ def test_temperature_sampling_on_device(pkg, rng):
         dev.sample_token(1.0, 1.0)
 
 
+# Prompt pass (bf16 products of float activations) against sequential decode (q8_K activations, integer products) at
+# full depth: two roundings of the same sums whose difference grows with the layers (0.02-0.05 of the largest value
+# after 2 layers, about 0.2 after 32: observed 0.195 / 0.184 / 0.149 for logits / K / V, root mean square 0.19 / 0.17 /
+# 0.17; the oracle's own two arithmetics differ by as much at this depth, see test_q4ks_full_size_against_oracle).
+# Bounds: largest difference relative to the largest value, and root-mean-square difference relative to the
+# root-mean-square value.
+PF_SEQ_TOL, PF_SEQ_RMS_TOL = 0.3, 0.3
+
+
+def _rms_rel(a, b):
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    return float(np.sqrt(np.mean((a - b) ** 2)) / max(1e-30, np.sqrt(np.mean(b ** 2))))
+
+
 def test_full_size_model_launch_paths_agree(pkg):
     """The benchmark's model at its full size (Llama-3-8B shape: 32 layers, vocabulary 128256, q4_K layers, q6_K
     output), too large for the CPU oracle to follow in a test: the two launch paths that share no kernel
     code beyond the arithmetic helpers must give the same 128 greedy tokens and bit-identical final logits,
-    and the prompt pass must leave the same logits and cache with and without its bf16 weight copy."""
+    the prompt pass must leave the same logits and cache with and without its bf16 weight copy, and what it leaves
+    must agree (to bf16 accuracy) with decoding the same 2048 tokens one by one."""
     from llama2_jl_amd import synth
     kw = dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8, vocab_size=128256, seq_len=512,
               rope_freq_base=500000.0, rope_is_neox=False)
@@ -423,6 +438,19 @@ def test_full_size_model_launch_paths_agree(pkg):
             assert pf[0][1] == pf[1][1]
             assert np.array_equal(pf[0][0], pf[1][0])
             assert np.array_equal(pf[0][2], pf[1][2]) and np.array_equal(pf[0][3], pf[1][3])
+            # the prompt pass against the state the token loop leaves (src/inference.jl:349-358: the reference feeds a
+            # prompt token by token): the same 2048 tokens decoded one after the other, last logits and the last
+            # layer's cache rows.  bf16 products of float activations against q8_K integer products: two roundings of
+            # the same sums, 32 layers deep -- a tolerance, the observed values are printed.
+            dev.reset()
+            _, seq_logits = dev.generate_greedy(long_prompt, 1, want_logits=True)
+            sk, sv = dev.kv_read(31, 0, 2048)
+            e_l, e_k, e_v = _rel(pf[0][0], seq_logits), _rel(pf[0][2], sk), _rel(pf[0][3], sv)
+            r_l, r_k, r_v = _rms_rel(pf[0][0], seq_logits), _rms_rel(pf[0][2], sk), _rms_rel(pf[0][3], sv)
+            print("\n[full size] 2048-position prompt pass vs the same tokens decoded one by one: logits rel diff max %.3g "
+                  "rms %.3g, layer-31 K max %.3g rms %.3g, V max %.3g rms %.3g; same next token: %s"
+                  % (e_l, r_l, e_k, r_k, e_v, r_v, pf[0][1] == int(np.argmax(seq_logits))))
+            assert max(e_l, e_k, e_v) <= PF_SEQ_TOL and max(r_l, r_k, r_v) <= PF_SEQ_RMS_TOL
         dev.close()
         del dev, lm
     assert got[1][0].tolist() == got[3][0].tolist()

@@ -86,6 +86,16 @@ def test_quantize_q8k_bit_exact(pkg, orc, rng):
         assert got.tobytes() == want.tobytes(), name
 
 
+def test_quantize_q8k_rejects_non_finite_input(pkg):
+    """NaN or infinity in the input: an argument error, checked on the host before anything runs."""
+    for bad in (np.nan, np.inf, -np.inf):
+        x = np.ones(512, np.float32)
+        x[300] = bad
+        with pytest.raises(pkg.L2HError) as ei:
+            pkg.quantize_q8_K(x)
+        assert ei.value.code == -1 and "not finite" in str(ei.value)  # L2H_EINVAL
+
+
 @pytest.mark.parametrize("typ", [Q4, Q5, Q6])
 @pytest.mark.parametrize("ne0,ne1", [(256, 5), (768, 67), (4096, 130), (14336, 9)])
 def test_matmul_kquant(pkg, orc, rng, typ, ne0, ne1):

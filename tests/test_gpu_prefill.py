@@ -129,6 +129,39 @@ def test_prefill_longer_than_one_chunk(pkg, orc):
     assert err <= LOGIT_TOL and _rel(k, rk) <= KV_TOL and _rel(v, rv) <= KV_TOL
 
 
+def test_prefill_headline_widths_against_token_loop(pkg, orc):
+    """The prompt pass at the headline's widths (dim 4096, hidden 14336, 32 / 8 heads of 128, q4_K layers; K = 4096 and
+    14336 in the products), two layers deep and with a small vocabulary so that the oracle's token loop finishes in
+    seconds, 320 positions (w1|w3 then runs as the launch that mixes 256 x 256 and 256 x 128 tiles): every layer's K/V
+    rows and the last logits against the oracle, at the same tolerances as the small shapes; with and without the
+    bf16 weight copy."""
+    from llama2_jl_amd import synth
+    kw = dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8, vocab_size=2048, seq_len=336,
+              rope_freq_base=500000.0, rope_is_neox=False)
+    lm = _model(pkg, "PLAN_Q4_K_S", **kw)
+    n = 320
+    prompt = synth.seeded_prompt(13, n, kw["vocab_size"])
+    om = orc.model_from_language_model(lm, nthreads=16)
+    om.reset()
+    ref = _oracle_run(orc, om, prompt)
+    dev = lm.device()
+    for on in (True, False):
+        dev.set_prefill_copy(on)
+        dev.reset()
+        logits, nxt = dev.prefill(prompt, 0)
+        e = _rel(logits, ref)
+        ekv = 0.0
+        for layer in range(2):
+            k, v = dev.kv_read(layer, 0, n)
+            rk, rv = om.kv_read(layer, 0, n)
+            ekv = max(ekv, _rel(k, rk), _rel(v, rv))
+        print("\n[headline widths, bf16 copy %s] prefill vs token loop: logits rel err %.3g, K/V rel err %.3g" % (on, e, ekv))
+        assert e <= LOGIT_TOL and ekv <= KV_TOL
+    dev.set_prefill_copy(True)
+    dev.close()
+    om.close()
+
+
 def test_prefill_argument_checks(pkg):
     plan, kw = CASES["f32"]
     lm = _model(pkg, plan, **kw)

@@ -123,6 +123,40 @@ def test_q5km_full_size_against_oracle(pkg, orc):
     assert np.array_equal(a_logits.view(np.uint32), b_logits.view(np.uint32))
 
 
+def test_q4ks_full_size_against_oracle(pkg, orc):
+    """Configuration 2, the headline, at its full size (32 layers, vocabulary 128256, q4_K layers, q6_K output): the
+    oracle follows it for a 4-token prompt and 6 greedy tokens on the library's own choice of launch path (the
+    streaming kernel)."""
+    from llama2_jl_amd import synth
+    kw = dict(dim=4096, hidden_dim=14336, n_layers=32, n_heads=32, n_kv_heads=8, vocab_size=128256, seq_len=512,
+              rope_freq_base=500000.0, rope_is_neox=False)
+    lm = _model(pkg, "PLAN_Q4_K_S", 35, **kw)
+    prompt = synth.seeded_prompt(6, 4, kw["vocab_size"])
+    dev = lm.device()
+    assert dev.path == 3
+    om = orc.model_from_language_model(lm, nthreads=16)
+    ids, logits = dev.generate_greedy(prompt, 6, want_logits=True)
+    ref_ids, ref_logits = om.generate_greedy(prompt, 6, orc.GPU_SPEC)
+    print("\n[Q4_K_S, full size, launch path 3] logits rel err %.3g" % _rel(logits, ref_logits))
+    assert ids.tolist() == ref_ids.tolist()
+    assert _rel(logits, ref_logits) <= 1e-3
+    # How far the q8_K step moves a random-weight model of this depth, for scale (the prompt pass multiplies float
+    # activations, and tests/test_gpu_model.py compares it with sequential decode at this size): the oracle's two
+    # arithmetics fed the same nine tokens, logits at the last position.
+    fed = list(prompt) + [int(t) for t in ref_ids[:5]]
+    last = {}
+    for mode in (orc.GPU_SPEC, orc.REFERENCE):
+        om.reset()
+        for pos, tok in enumerate(fed):
+            last[mode] = om.forward(int(tok), pos, mode)
+    a, b = last[orc.GPU_SPEC].astype(np.float64), last[orc.REFERENCE].astype(np.float64)
+    rms = float(np.sqrt(np.mean((a - b) ** 2)) / np.sqrt(np.mean(b ** 2)))
+    print("[Q4_K_S, full size] oracle with q8_K activations vs with float activations, 32 layers, position 8: logits rel "
+          "diff max %.3g, rms %.3g" % (_rel(last[orc.GPU_SPEC], last[orc.REFERENCE]), rms))
+    om.close()
+    dev.close()
+
+
 def test_phi3_full_size_against_oracle(pkg, orc):
     """Configuration 4 at its full size (32 layers) with its 4096-long cache, 3840 rows pre-filled: six greedy
     tokens from position 3840 against the oracle."""
