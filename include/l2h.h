@@ -122,7 +122,11 @@ const char *l2h_model_path_reason(l2h_model *m);
 /* Launch paths 2 and 3 wait on the device for other workgroups' results; every such wait gives up after
  * `spins` polls (default 2^20 on path 3, about a second), upon which all workgroups leave the kernel and
  * the call that launched it returns L2H_EHIP; the model stays usable (l2h_state_reset, then decode
- * again).  This sets the bound for path 3 (after finalize).  No counterpart in the reference. */
+ * again).  A model whose path the library chose itself (l2h_model_set_path 0) runs on path 1 from
+ * then on, and l2h_model_path / l2h_model_path_reason say so: a GPU that another process shares cannot
+ * hold all of path 3's workgroups at once, and every token would end that way.  A model for which
+ * path 3 was asked for keeps it.  This sets the bound for path 3 (after finalize).  No counterpart in
+ * the reference. */
 int l2h_model_set_wait_limit(l2h_model *m, unsigned int spins);
 /* l2h_prefill keeps a bf16 copy of the layer matrices (2 bytes per weight, made at its first call
  * when that fits beside 2 GiB of free device memory) and multiplies from it; on = 0 makes it

@@ -943,6 +943,25 @@ static hipError_t enqueue_token(l2h_model *m) {
     return hipSuccess;
 }
 
+// Records the launch sequence of one token (launch path 1); positions and tokens are read from the
+// control block on the device, so the recording is replayed unchanged for every step.
+static int record_token(l2h_model *m) {
+    l2h_ctx *ctx = m->ctx;
+    if (m->exec || getenv("L2H_NO_GRAPH")) return L2H_OK;
+    HIPCHK(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeGlobal));
+    hipError_t e = enqueue_token(m);
+    hipGraph_t g = nullptr;
+    hipError_t e2 = hipStreamEndCapture(ctx->stream, &g);
+    if (e != hipSuccess || e2 != hipSuccess) {
+        if (g) (void)hipGraphDestroy(g);
+        return set_err(ctx, L2H_EHIP, "recording the token launch sequence failed: %s",
+                       hipGetErrorString(e != hipSuccess ? e : e2));
+    }
+    m->graph = g;
+    HIPCHK(ctx, hipGraphInstantiate(&m->exec, m->graph, nullptr, nullptr, 0));
+    return L2H_OK;
+}
+
 extern "C" int l2h_model_finalize(l2h_model *m) {
     if (!m) return L2H_EINVAL;
     l2h_ctx *ctx = m->ctx;
@@ -993,21 +1012,7 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
     if ((rc = mega_setup(m))) return rc;
     if ((rc = flow_setup(m))) return rc;
 
-    // Record the launch sequence of one token; positions and tokens are read from the
-    // control block on the device, so the recording is replayed unchanged for every step.
-    if (!m->mega && !m->flow && !getenv("L2H_NO_GRAPH")) {
-        HIPCHK(ctx, hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeGlobal));
-        hipError_t e = enqueue_token(m);
-        hipGraph_t g = nullptr;
-        hipError_t e2 = hipStreamEndCapture(ctx->stream, &g);
-        if (e != hipSuccess || e2 != hipSuccess) {
-            if (g) (void)hipGraphDestroy(g);
-            return set_err(ctx, L2H_EHIP, "recording the token launch sequence failed: %s",
-                           hipGetErrorString(e != hipSuccess ? e : e2));
-        }
-        m->graph = g;
-        HIPCHK(ctx, hipGraphInstantiate(&m->exec, m->graph, nullptr, nullptr, 0));
-    }
+    if (!m->mega && !m->flow && (rc = record_token(m))) return rc;
     m->finalized = true;
     return L2H_OK;
 }
@@ -1043,6 +1048,20 @@ static int mega_check(l2h_model *m) {
         HIPCHK(m->ctx, hipMemset(m->flow_args.x_a, 0xFF, (size_t)m->c.dim * 4));
         HIPCHK(m->ctx, hipMemset(m->flow_args.x_b, 0xFF, (size_t)m->c.dim * 4));
         HIPCHK(m->ctx, hipMemset(m->flow_args.xo, 0xFF, 2 * (size_t)m->c.dim * 4));
+        // Where the library chose this path itself, the following calls run one kernel per phase: a launch whose
+        // workgroups are not all resident at once (another process on the GPU) would give up at every token.  A
+        // caller that asked for path 3 keeps it.
+        if (m->path_request == 0) {
+            const int rc = record_token(m);
+            if (rc == L2H_OK) {
+                m->flow = false;
+                m->flow_why = "a wait of the streaming kernel ran into its limit (are its workgroups resident at once?); "
+                              "the model now runs one kernel per phase";
+                if (g_flow_bound == m) g_flow_bound = nullptr;
+                return set_err(m->ctx, L2H_EHIP, "streaming decode kernel: a wait for activations timed out; the model "
+                                                 "runs on launch path 1 from now on");
+            }
+        }
         return set_err(m->ctx, L2H_EHIP, "streaming decode kernel: a wait for activations timed out");
     }
     if (!m->mega) return L2H_OK;

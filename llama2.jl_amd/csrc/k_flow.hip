@@ -88,6 +88,11 @@ __device__ __forceinline__ float tag_val(u64 w) { return __uint_as_float((unsign
 // back into word i of the other: every reader of that one finished with it a phase ago, and it is the
 // same thread that writes word i of either.
 #define FLOW_EMPTY 0xFFFFFFFFu
+// A barrier that orders the workgroup's LDS traffic only.  __syncthreads() also waits for every request to memory that
+// the wavefront has under way, the fetches into its ring included; nothing that passes between the wavefronts of a
+// workgroup where this one stands goes through memory.
+// (In the staging function and the layer epilogues: 769 against 766 tok/s on the headline model.)
+__device__ __forceinline__ void flow_barrier_lds() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 __device__ __forceinline__ unsigned bare_load(const unsigned *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -382,7 +387,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
         }
         if (!ok) s_flag = 1;  // zero since the start of the kernel; a kernel that sets it ends
         STG();  // this wavefront's blocks are in LDS
-        __syncthreads();
+        flow_barrier_lds();
         STG();  // everybody's
         if (s_flag) {
             if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -447,7 +452,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
             if (lane == 0) s_red[wave] = acc;
             if (mine) *(float4 *)(raw_of(wave) + 4 * lane) = make_float4(xv[0], xv[1], xv[2], xv[3]);
         }
-        __syncthreads();
+        flow_barrier_lds();
         STG();  // every wavefront's are
         if (s_flag) {
             if (threadIdx.x == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -473,7 +478,7 @@ __device__ __noinline__ bool flow_stage(const void *src, int K, const float *nor
             quads_store(v);
         }
         STG();  // this wavefront's blocks are in LDS
-        __syncthreads();
+        flow_barrier_lds();
         STG();  // everybody's
         return true;
     }
@@ -1041,7 +1046,7 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
     const int n_local = flow_n_local(a.qkv, wg);
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));  // (what derives from it is computed here and not kept across the kernel)
-    __syncthreads();
+    flow_barrier_lds();
     if (tid >= n_local) return;
     const int L = wg * a.qkv.rpw + tid;
     int seg, row;
@@ -1091,7 +1096,7 @@ __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned ol
     const int n_local = flow_n_local(g, wg);
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
-    __syncthreads();
+    flow_barrier_lds();
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
     const float old = bare_read(src + row, oldw);
@@ -1108,7 +1113,7 @@ __device__ __noinline__ unsigned flow_w13_word(int wg) {
     const int n_local = flow_n_local(a.w13, wg);
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
-    __syncthreads();
+    flow_barrier_lds();
     if (tid >= n_local) return 0u;
     const float own = flow_row_value4(tid, a.w13.ppr), next = flow_pair_value(own);  // (w1 row u | w3 row u, threads 2u | 2u+1)
     if (tid & 1) return 0u;

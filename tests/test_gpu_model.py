@@ -322,6 +322,34 @@ def test_streaming_kernel_gives_up_and_recovers(pkg):
         assert np.asarray(got).tolist() == np.asarray(want).tolist()
 
 
+def test_streaming_kernel_gives_up_and_falls_to_the_per_phase_path(pkg):
+    """Where the library chose the streaming kernel itself (path 0), a launch that gave up makes the model run one
+    kernel per phase from then on: a GPU shared with another process would otherwise fail at every token.  The wait
+    bound is forced to zero from the host, so every kernel exits normally; the failing call reports the switch, the
+    following calls give the tokens of the per-phase path (which are the streaming kernel's)."""
+    from llama2_jl_amd import synth
+    plan, kw = FLOW_CASES["all_q4"]
+    lm = _model(pkg, plan, **kw)
+    dev = lm.device()
+    assert dev.path == 3 and dev.path_reason == ""
+    prompt = synth.seeded_prompt(11, 6, lm.config.vocab_size)
+    dev.reset()
+    want = dev.generate_greedy(prompt, 10)
+    dev.set_wait_limit(0)
+    dev.reset()
+    with pytest.raises(pkg.L2HError) as ei:
+        dev.generate_greedy(prompt, 10)
+    assert "launch path 1" in str(ei.value)
+    from llama2_jl_amd import _lib
+    assert _lib.lib().l2h_model_path(dev.handle) == 1
+    assert "one kernel per phase" in _lib.lib().l2h_model_path_reason(dev.handle).decode()
+    for _ in range(2):
+        dev.reset()
+        got = dev.generate_greedy(prompt, 10)
+        assert np.asarray(got).tolist() == np.asarray(want).tolist()
+    dev.close()
+
+
 def test_generate_argument_checks(pkg):
     from llama2_jl_amd import synth
     plan, kw = CASES["f32"]
