@@ -24,11 +24,15 @@ import __graft_entry__ as entry  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
 # HBM traffic of the dominant kernel per launch, from rocprofv3 --pmc runs of this script (FETCH_SIZE x 2.000 KiB +
-# WRITE_SIZE x 1.000 KiB per unit, the factors a plain read of known size gave in the same runs):
-#   (workload, launch path 1): per matvec launch, 31.23 MB read + 0.04 MB written (profiles/pmc_fetch_write_bench_8b-q4ks.md)
-#   (workload, launch path 3): per token launch, 4486.3 MB read + 9.3 MB written (profiles/pmc_fetch_write_bench_8b-q4ks_streaming.md);
-#   8b-q5km: 5755.5 MB read + 9.3 MB written (profiles/kernel_stats_bench_8b-q5km.md)
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4495700000, ("8b-q5km", 3): 5764800000}
+# WRITE_SIZE x 1.000 KiB per unit, the factors a plain read of known size gave in the same runs; the launches of the
+# timed region):
+#   (8b-q4ks, launch path 1): per matvec launch, 31.23 MB read + 0.04 MB written (profiles/pmc_fetch_write_bench_8b-q4ks.md)
+#   launch path 3, per token launch (profiles/pmc_fetch_write_streaming_kernel_all_workloads.md):
+#     8b-q4ks 4500.9 MB read + 9.3 MB written, 8b-q5km 5760.0 + 9.3, phi3-4k 5858.9 + 38.9, llama2c-f32 172.6 + 0.8,
+#     8b-q4ks-prefill (its decode steps at positions 2048 and up) 5021.0 + 67.1
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4510221000, ("8b-q5km", 3): 5769380000,
+                                     ("phi3-4k", 3): 5897871000, ("llama2c-f32", 3): 173480000,
+                                     ("8b-q4ks-prefill", 3): 5088146000}
 
 WORKLOADS = {
     # name: (plan, config kwargs, prompt length)
@@ -242,8 +246,8 @@ def main():
         om.close()
 
     # HBM traffic of the dominant kernel per launch (FETCH_SIZE + WRITE_SIZE, scaled), measured with
-    # rocprofv3 --pmc on this workload: profiles/pmc_fetch_write_bench_8b-q4ks.md
-    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dev.path))
+    # rocprofv3 --pmc on this workload with its fp32 cache (null for a combination that no counter run covers)
+    traffic = MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get((args.workload, dev.path)) if args.kv == "fp32" else None
 
     result = {
         "metric": "decode tok/s, Llama-3-8B-shape Q4_K_S, batch 1; % of HBM-BW roofline",

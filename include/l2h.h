@@ -194,6 +194,12 @@ int l2h_dequantize(l2h_ctx *ctx, int ggml_type, const void *blocks, int64_t nb, 
  * sums the kernel formed: [ne1][ne0/256] int32 each.  k-quant: ne0 <= 16384. */
 int l2h_matmul(l2h_ctx *ctx, int ggml_type, const void *A, int64_t ne0, int64_t ne1, const float *x, float *y,
                int32_t *I_sc, int32_t *I_min);
+/* matmul!(y, A, x) (src/matmul.jl:13-23 as transformer! calls it, src/inference.jl:247-249, 281, 291-292,
+ * 302, 312) with A one of the model's resident matrices: role L2H_TOK_EMB, L2H_OUTPUT or L2H_WQ..L2H_W3 of
+ * `layer` (ignored for the first two).  x[ne0] and y[ne1] are host arrays.  Nothing is uploaded but x: this is
+ * the seam at which the reference's own transformer! runs on device-resident weights (a matrix type whose
+ * matmul! method calls this). */
+int l2h_model_matmul(l2h_model *m, int role, int layer, const float *x, float *y);
 /* rmsnorm!(o, x, weight) (src/inference.jl:102-110). o may alias x. n <= 15360. */
 int l2h_rmsnorm(l2h_ctx *ctx, float *o, const float *x, const float *weight, int64_t n);
 /* rmsnorm! followed by q8_K quantization of the result, exactly as the matvec kernels do it in

@@ -65,6 +65,7 @@ SIGNATURES = {
     "l2h_quantize_q8k": (_I, [_P, _P, _I64, _P]),
     "l2h_dequantize": (_I, [_P, _I, _P, _I64, _P]),
     "l2h_matmul": (_I, [_P, _I, _P, _I64, _I64, _P, _P, _P, _P]),
+    "l2h_model_matmul": (_I, [_P, _I, _I, _P, _P]),
     "l2h_rmsnorm": (_I, [_P, _P, _P, _P, _I64]),
     "l2h_rmsnorm_q8k": (_I, [_P, _P, _P, _I64, _P]),
     "l2h_rope": (_I, [_P, _P, _I, _I, _I, _F, _I]),

@@ -1544,6 +1544,34 @@ extern "C" int l2h_matmul(l2h_ctx *ctx, int type, const void *A, int64_t ne0, in
     return rc;
 }
 
+// matmul!(y, A, x) with A one of the model's resident matrices (uploaded through l2h_model_set_tensor)
+extern "C" int l2h_model_matmul(l2h_model *m, int role, int layer, const float *x, float *y) {
+    if (!m || !x || !y) return set_err(m ? m->ctx : nullptr, L2H_EINVAL, "l2h_model_matmul: NULL argument");
+    l2h_ctx *ctx = m->ctx;
+    if (!m->finalized) return set_err(ctx, L2H_ESTATE, "model not finalized");
+    const bool glob = role == L2H_TOK_EMB || role == L2H_OUTPUT;
+    const bool per_layer = role >= L2H_WQ && role < L2H_N_ROLES;
+    if (!glob && !per_layer) return set_err(ctx, L2H_EINVAL, "role %d is not a matrix", role);
+    if (per_layer && (layer < 0 || layer >= m->c.n_layers)) return set_err(ctx, L2H_EINVAL, "layer %d out of range", layer);
+    const DevTensor &t = glob ? m->glob[role] : m->L(layer, role);
+    HIPCHK(ctx, hipSetDevice(ctx->device));
+    DevBuf dx, dy;
+    HIPCHK(ctx, dx.alloc((size_t)t.ne0 * 4));
+    HIPCHK(ctx, dy.alloc((size_t)t.ne1 * 4));
+    HIPCHK(ctx, hipMemcpy(dx.p, x, (size_t)t.ne0 * 4, hipMemcpyHostToDevice));
+    PhaseArgs a{};
+    a.max_grid = ctx->prop.multiProcessorCount;
+    a.nseg = 1;
+    a.w[0] = t;
+    a.w[0].layer_stride = 0;  // (the tensor of this very layer: no stepping through the role's slab)
+    a.y[0] = dy.as<float>();
+    a.xf = dx.as<float>();
+    HIPCHK(ctx, k_matvec(ctx->stream, a, PRO_QUANT, EPI_STORE));
+    HIPCHK(ctx, hipStreamSynchronize(ctx->stream));
+    HIPCHK(ctx, hipMemcpy(y, dy.p, (size_t)t.ne1 * 4, hipMemcpyDeviceToHost));
+    return L2H_OK;
+}
+
 extern "C" int l2h_rmsnorm(l2h_ctx *ctx, float *o, const float *x, const float *weight, int64_t n) {
     if (!ctx || !o || !x || !weight) return set_err(ctx, L2H_EINVAL, "l2h_rmsnorm: NULL argument");
     if (n <= 0 || n > 15360) return set_err(ctx, L2H_EINVAL, "length %lld outside 1..15360", (long long)n);

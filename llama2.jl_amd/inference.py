@@ -71,6 +71,7 @@ class DeviceModel:
                           config.vocab_size, config.seq_len, float(config.rope_freq_base),
                           1 if config.rope_is_neox else 0)
         self.handle = C.c_void_p()
+        self._shapes = {}
         self.ctx.check(_lib.lib().l2h_model_create(self.ctx.handle, C.byref(cfg), C.byref(self.handle)))
         try:
             self._set(_lib.TOK_EMB, 0, weights.token_embedding_table)
@@ -97,6 +98,7 @@ class DeviceModel:
         else:
             (ne0, ne1), typ, raw = matrix_shape(A), matrix_type(A), matrix_bytes(A)
         self.ctx.check(_lib.lib().l2h_model_set_tensor(self.handle, role, layer, typ, _lib.ptr(raw), ne0, ne1))
+        self._shapes[(role, layer)] = (ne0, ne1)
 
     def close(self):
         if self.handle:
@@ -112,6 +114,17 @@ class DeviceModel:
     # --- RunState operations ---
     def reset(self):
         self.ctx.check(_lib.lib().l2h_state_reset(self.handle))
+
+    def matmul(self, role, layer, x):
+        """matmul!(y, A, x) with A the resident matrix `role` of `layer` (l2h_model_matmul): the seam at which the
+        reference's own transformer! can run on device-resident weights."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        ne0, ne1 = self._shapes[(role, 0 if role < 3 else layer)]
+        if x.size != ne0:
+            raise ValueError("x has %d elements, the matrix expects %d" % (x.size, ne0))
+        y = np.empty(ne1, np.float32)
+        self.ctx.check(_lib.lib().l2h_model_matmul(self.handle, role, layer, _lib.ptr(x), _lib.ptr(y)))
+        return y
 
     def set_wait_limit(self, spins):
         """Bound of the streaming kernel's device-side waits (l2h_model_set_wait_limit)."""

@@ -10,6 +10,7 @@
 module Llama2HIP
 
 using Llama2
+import Llama2
 using Llama2: LanguageModel, ModelConfig, TransformerWeights, TransformerLayerWeights,
               block_q4_K, block_q5_K, block_q6_K, encode
 
@@ -190,6 +191,69 @@ function sample(m::DeviceModel, model::LanguageModel, prompt::String = ""; tempe
     println("-------\nachieved tok/s: ", round(generated_seq_len / (time_ns() - time_start) * 1e9; digits = 2))
     return nothing
 end
+
+# ---- drop-in use: the package's own entry points on device-resident weights ------------------------------------
+#
+# Two seams, both without a changed line in Llama2.jl:
+#
+#  * `DeviceLanguageModel` is a model type of its own for which `Llama2.sample` has a method, so that
+#        model = on_device(load_gguf_model("model.gguf"));  sample(model, "Once upon a time")
+#    reads like the reference's call (src/inference.jl:317-324) and runs the whole token loop on the GPU.
+#  * `DeviceMatrix <: AbstractMatrix` stands in for a weight in the `AbstractMatrix` fields of
+#    `TransformerWeights` / `TransformerLayerWeights` (src/inference.jl:27-48).  `Llama2.matmul!` has a method for it
+#    (the reference dispatches on the matrix type, src/matmul.jl:3-23), so a `LanguageModel` built by
+#    `with_device_matrices` flows through the reference's own `sample` and `transformer!` unchanged: rmsnorm, RoPE and
+#    attention stay on the CPU, every matrix product runs on the resident weights (one vector up, one down per product:
+#    the slow of the two seams, for checking one against the other).
+
+"A weight that lives in a `DeviceModel`: `matmul!` runs on the GPU, everything else (size, indexing) on the host array."
+struct DeviceMatrix{T, A <: AbstractMatrix{T}} <: AbstractMatrix{T}
+    dev::DeviceModel
+    role::Int32
+    layer::Int32          # 0-based, as the C ABI counts
+    host::A
+end
+Base.size(A::DeviceMatrix) = size(A.host)
+Base.getindex(A::DeviceMatrix, i::Int, j::Int) = A.host[i, j]
+Base.getindex(A::DeviceMatrix, ::Colon, j::Int) = A.host[:, j]
+Base.view(A::DeviceMatrix, ::Colon, j::Int) = view(A.host, :, j)
+Base.IndexStyle(::Type{<:DeviceMatrix}) = IndexCartesian()
+
+"`matmul!(y, A, x)` of Llama2.jl (src/matmul.jl:3-23) for a device-resident `A`."
+function Llama2.matmul!(y::AbstractVector{Float32}, A::DeviceMatrix, x::AbstractVector{Float32})
+    xs = x isa Vector{Float32} ? x : collect(x)
+    ys = y isa Vector{Float32} ? y : Vector{Float32}(undef, length(y))
+    check(A.dev.ctx.handle, ccall((:l2h_model_matmul, lib), Cint, (Ptr{Cvoid}, Cint, Cint, Ptr{Float32}, Ptr{Float32}),
+                                  A.dev.handle, A.role, A.layer, xs, ys))
+    ys === y || copyto!(y, ys)
+    return nothing
+end
+
+"A `LanguageModel` whose matrices are `DeviceMatrix`es of `dev`: the reference's `sample(model, prompt)` runs on it as it is."
+function with_device_matrices(model::LanguageModel, dev::DeviceModel = DeviceModel(model))
+    w = model.weights
+    dm(role, layer, A) = DeviceMatrix{eltype(A), typeof(A)}(dev, Int32(role), Int32(layer), A)
+    layers = [TransformerLayerWeights(; rms_att_weight = lw.rms_att_weight, rms_ffn_weight = lw.rms_ffn_weight,
+                                      wq = dm(WQ, l - 1, lw.wq), wk = dm(WK, l - 1, lw.wk), wv = dm(WV, l - 1, lw.wv),
+                                      wo = dm(WO, l - 1, lw.wo), w1 = dm(W1, l - 1, lw.w1), w2 = dm(W2, l - 1, lw.w2),
+                                      w3 = dm(W3, l - 1, lw.w3)) for (l, lw) in enumerate(w.layers)]
+    weights = TransformerWeights(; token_embedding_table = w.token_embedding_table, layers = layers,
+                                 rms_final_weight = w.rms_final_weight, output_weight = dm(OUTPUT, 0, w.output_weight))
+    return LanguageModel(model.config, model.tokenizer, weights)
+end
+
+"A loaded model together with its resident copy: what `sample` takes in place of a `LanguageModel`."
+struct DeviceLanguageModel{TOK}
+    host::LanguageModel{TOK}
+    dev::DeviceModel
+end
+on_device(model::LanguageModel; kwargs...) = DeviceLanguageModel(model, DeviceModel(model; kwargs...))
+# (config, tokenizer and weights read as on a LanguageModel)
+Base.getproperty(m::DeviceLanguageModel, name::Symbol) =
+    name === :host || name === :dev ? getfield(m, name) : getproperty(getfield(m, :host), name)
+
+"`sample(model, prompt; ...)` of Llama2.jl (src/inference.jl:317-395), the token loop on the GPU."
+Llama2.sample(m::DeviceLanguageModel, prompt::String = ""; kwargs...) = sample(m.dev, m.host, prompt; kwargs...)
 
 # ---- the single operators (each one seam of src/inference.jl / src/matmul.jl; host arrays in, host arrays out) ----
 

@@ -350,6 +350,32 @@ def test_streaming_kernel_gives_up_and_falls_to_the_per_phase_path(pkg):
     dev.close()
 
 
+@pytest.mark.parametrize("case", ["q4ks_gqa", "q5km", "f32"])
+def test_resident_matrix_matmul(pkg, orc, rng, case):
+    """l2h_model_matmul: matmul!(y, A, x) on a matrix that lives in the model (the seam at which the reference's own
+    transformer! runs on device-resident weights) equals l2h_matmul on the same host matrix bit for bit, for every
+    matrix role, layers other than the first included (each has its own place in its role's slab)."""
+    from llama2_jl_amd import _lib, kquants
+    plan, kw = CASES[case]
+    lm = _model(pkg, plan, **kw)
+    dev = lm.device()
+    w = lm.weights
+    last = lm.config.n_layers - 1
+    mats = [(_lib.TOK_EMB, 0, w.token_embedding_table), (_lib.OUTPUT, 0, w.output_weight)]
+    for name, role in (("wq", _lib.WQ), ("wk", _lib.WK), ("wv", _lib.WV), ("wo", _lib.WO), ("w1", _lib.W1), ("w2", _lib.W2),
+                       ("w3", _lib.W3)):
+        mats += [(role, 0, getattr(w.layers[0], name)), (role, last, getattr(w.layers[last], name))]
+    for role, layer, A in mats:
+        ne0, _ = kquants.matrix_shape(A)
+        x = rng.standard_normal(ne0).astype(np.float32)
+        got = dev.matmul(role, layer, x)
+        want = kquants.matmul(A, x)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (role, layer)
+    with pytest.raises(pkg.L2HError):
+        dev.matmul(_lib.RMS_ATT, 0, np.zeros(lm.config.dim, np.float32))  # not a matrix
+    dev.close()
+
+
 def test_generate_argument_checks(pkg):
     from llama2_jl_amd import synth
     plan, kw = CASES["f32"]

@@ -106,8 +106,16 @@ def test_julia_binding_matches_the_header():
     defined = set(re.findall(r"(?m)^function\s+([A-Za-z_!0-9]+)\s*\(", code)) | \
         set(re.findall(r"(?m)^([A-Za-z_!0-9]+)\([^\n]*\)\s*=", code))
     for fn in ("Context", "DeviceModel", "set_tensor!", "reset!", "transformer!", "generate", "prefill!", "sample_token",
-               "sample", "matmul!", "dequantize!", "rmsnorm!", "rope!", "softmax!", "argmax_first", "kv_write!"):
+               "sample", "matmul!", "dequantize!", "rmsnorm!", "rope!", "softmax!", "argmax_first", "kv_write!",
+               "with_device_matrices", "on_device"):
         assert fn in defined, "Llama2HIP.%s is not defined" % fn
+    # the drop-in seams: methods added to the reference's own generic functions, with the reference's argument lists
+    # (src/matmul.jl:3-7, src/inference.jl:317-324), a matrix type for the AbstractMatrix fields of the weights
+    # (src/inference.jl:27-48) and the resident-matrix product they rest on
+    assert re.search(r"(?m)^function Llama2\.matmul!\(y::AbstractVector\{Float32\}, A::DeviceMatrix, x::AbstractVector\{Float32\}\)", code)
+    assert re.search(r"(?m)^Llama2\.sample\(m::DeviceLanguageModel, prompt::String = \"\"; kwargs\.\.\.\)", code)
+    assert re.search(r"(?m)^struct DeviceMatrix\{T, A <: AbstractMatrix\{T\}\} <: AbstractMatrix\{T\}", code)
+    assert "l2h_model_matmul" in [m.group(1) for m in calls]
 
 
 def test_no_device_is_an_error_not_a_fallback(pkg):
