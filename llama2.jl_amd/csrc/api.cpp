@@ -226,6 +226,8 @@ struct l2h_model {
     hipGraphExec_t exec = nullptr;
     // persistent decode kernel
     int kv16 = 0;          // 1: the KV cache holds fp16 elements (l2h_model_set_kv_type)
+    bool kv_uncached = false;       // the KV cache lives in uncached memory (see l2h_model_finalize)
+    int flow_steps_per_launch = 1;  // steps of the token loop per launch of the streaming kernel
     int path_request = 0;  // 0 auto, 1 one kernel per phase, 2 persistent kernel, 3 streaming kernel (2, 3: required)
     bool mega = false;
     PhaseArgs mega_ph[5];  // q/k/v, wo, w1+w3, w2 of layer 0 and the classifier, planned for the persistent grid
@@ -861,6 +863,7 @@ static int flow_setup(l2h_model *m) {
         TA(a.att_x, (int64_t)c.n_heads * G * 3 + (int64_t)c.n_heads * G * m->hs * 2);
     }
     TA(a.abort_flag, 1);
+    TA(a.tokw, 8 * 16);  // (eight copies, a 128-byte line each: FLOW_TOK_COPIES in k_flow.hip)
 #undef TA
     a.kc = m->kc;
     a.vc = m->vc;
@@ -880,6 +883,9 @@ static int flow_setup(l2h_model *m) {
     if ((rc = dalloc(m, &m->timeline, (int64_t)grid * 64 + 1024, true))) return rc;
     a.timeline = m->timeline;
 #endif
+    // several steps per launch where the cache is coherent between the steps (L2H_FLOW_STEPS: 1..64, for measurements)
+    m->flow_steps_per_launch = m->kv_uncached ? 8 : 1;
+    if (const char *e = getenv("L2H_FLOW_STEPS")) m->flow_steps_per_launch = std::min(64, std::max(1, atoi(e)));
     m->flow_args = a;
     m->flow_grid = grid;
     m->flow_cls_type = cls_type;
@@ -888,14 +894,16 @@ static int flow_setup(l2h_model *m) {
     return L2H_OK;
 }
 
-static hipError_t flow_launch_token(l2h_model *m) {
+// The streaming kernel runs up to this many steps of the token loop per launch (the next step's token passes from
+// workgroup 0 to the others inside the kernel): what lies between two launches, about 10 us, is paid once per that many tokens.
+static hipError_t flow_launch_tokens(l2h_model *m, int n_tok) {
     if (g_flow_bound != m) {
         hipError_t eb = k_flow_bind(m->ctx->stream, m->flow_args);
         if (eb != hipSuccess) return eb;
         g_flow_bound = m;
     }
-    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, m->flow_cls_type, m->flow_grid, m->flow_args.mixed != 0);
-    if (e == hipSuccess) m->flow_gen += 5u * (unsigned)m->c.n_layers + 2u;
+    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, n_tok, m->flow_cls_type, m->flow_grid, m->flow_args.mixed != 0);
+    if (e == hipSuccess) m->flow_gen += (unsigned)n_tok * (5u * (unsigned)m->c.n_layers + 2u);
     return e;
 }
 
@@ -1000,8 +1008,29 @@ extern "C" int l2h_model_finalize(l2h_model *m) {
         if (m->path_request == 2) return set_err(ctx, L2H_EINVAL, "an fp16 KV cache does not run on launch path 2");
     }
     // (an fp16 cache takes half the floats)
-    DA(m->kc, m->cache_layer_elems * c.n_layers / (m->kv16 ? 2 : 1) + 1, true);
-    DA(m->vc, m->cache_layer_elems * c.n_layers / (m->kv16 ? 2 : 1) + 1, true);
+    // A launch of the streaming kernel that runs several steps of the token loop reads, in a later step, cache rows that
+    // another XCD's workgroups appended in an earlier one: rows in ordinary memory would still sit in the writer's L2
+    // (and stale lines in the reader's), which only the end of a kernel puts right.  Where no two heads share a cache
+    // row (n_kv_heads == n_heads: nothing is read twice, the L2 holds nothing worth keeping) the cache therefore lives
+    // in uncached memory, and such a model decodes several steps per launch; with shared rows it stays in ordinary memory
+    // and every step is a launch.
+    {
+        const char *env = getenv("L2H_KV_UNCACHED");
+        m->kv_uncached = env ? atoi(env) != 0 : (c.n_heads == c.n_kv_heads && (m->path_request == 0 || m->path_request == 3));
+        const int64_t n = m->cache_layer_elems * c.n_layers / (m->kv16 ? 2 : 1) + 1;
+        if (m->kv_uncached) {
+            for (float **p : {&m->kc, &m->vc}) {
+                void *v = nullptr;
+                HIPCHK(ctx, uncached_alloc(ctx->device, (size_t)n * 4, &v));
+                m->uc_allocs.push_back(v);
+                HIPCHK(ctx, hipMemset(v, 0, (size_t)n * 4));
+                *p = (float *)v;
+            }
+        } else {
+            DA(m->kc, n, true);
+            DA(m->vc, n, true);
+        }
+    }
     DA(m->ctl, 1, true);
     DA(m->prompt_dev, c.seq_len, true);
     m->max_out = c.seq_len;
@@ -1021,8 +1050,10 @@ static int run_steps(l2h_model *m, int n) {
     l2h_ctx *ctx = m->ctx;
     for (int i = 0; i < n; i++) {
         if (m->flow) {
-            hipError_t e = flow_launch_token(m);
+            const int n_tok = std::min(n - i, m->flow_steps_per_launch);
+            hipError_t e = flow_launch_tokens(m, n_tok);
             if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "decode kernel launch failed: %s", hipGetErrorString(e));
+            i += n_tok - 1;
         } else if (m->mega) {
             hipError_t e = mega_launch_token(m);
             if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "decode kernel launch failed: %s", hipGetErrorString(e));

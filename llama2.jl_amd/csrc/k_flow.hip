@@ -70,6 +70,8 @@ __shared__ int s_tl_fine;
 #define STG()
 #endif
 __shared__ __attribute__((aligned(16))) unsigned char s_sink[256];  // target of fetches made only to warm the L2
+__shared__ int s_tok;  // the token of a launch's next step (flow_next_token)
+#define FLOW_TOK_COPIES 8
 
 __device__ __forceinline__ void tag_store(u64 *p, float v, unsigned epoch) {
     __hip_atomic_store(p, ((u64)epoch << 32) | (u64)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1166,7 +1168,8 @@ __device__ __noinline__ void flow_finish_cls(int wg, unsigned e_cls) {
 
 // argmax(logits) (:360) over the workgroups' keys and the step bookkeeping of the token loop
 // (:349-386); run by workgroup 0
-__device__ __noinline__ void flow_pick_token(int nwg, unsigned e_cls) {
+// e_next != 0: the launch goes on with another step; the token is handed to all workgroups as a word of that epoch
+__device__ __noinline__ void flow_pick_token(int nwg, unsigned e_cls, unsigned e_next) {
     const FlowArgs &a = c_flow;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     unsigned long long best = 0;
@@ -1213,6 +1216,36 @@ __device__ __noinline__ void flow_pick_token(int nwg, unsigned e_cls) {
     }
     ctl->step += 1;
     ctl->pos += 1;
+    if (e_next)
+        for (int c = 0; c < FLOW_TOK_COPIES; c++) tag_store(a.tokw + 16 * c, __uint_as_float((unsigned)idx), e_next);
+}
+
+// The token of a launch's second and later steps: workgroup 0 publishes it when it has picked (flow_pick_token), and
+// since that takes every workgroup's largest logit, a workgroup that has the word also knows that all others are
+// through the step before (it may write the next step's first activations).  Polled on the scalar path: a scalar load
+// that bypasses the scalar cache does not wait behind the fetches that the rings have just been refilled with, as a
+// vector load would.  The word comes in FLOW_TOK_COPIES copies, a 128-byte line each, and a workgroup's first wavefront
+// polls copy `workgroup % FLOW_TOK_COPIES` for all sixteen (one line is asked by a thirty-second of the chip).  Returns
+// -1 if the wait gave up.
+__device__ __forceinline__ int flow_next_token(unsigned epoch) {
+    const FlowArgs &a = c_flow;
+    if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0) {
+        const u64 *p = a.tokw + 16 * (blockIdx.x % FLOW_TOK_COPIES);
+        int tok = -1;
+        for (unsigned spins = 0; spins <= a.spin_limit; spins++) {
+            u64 w;
+            asm volatile("s_load_dwordx2 %0, %1, 0x0 glc\n\ts_waitcnt lgkmcnt(0)" : "=s"(w) : "s"(p) : "memory");
+            if (tag_is(w, epoch)) {
+                tok = (int)(unsigned)w;
+                break;
+            }
+            if ((spins & 63) == 63 && __hip_atomic_load(a.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
+        if ((threadIdx.x & 63) == 0) s_tok = tok;
+    }
+    flow_barrier_lds();
+    return s_tok;
 }
 
 // The cache lines that head h's attention will read (positions before `pos`) are requested early, while
@@ -1755,22 +1788,52 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
 // ------------------------------------------------------------------------------------------
 // MIXED: the layers' pieces are typed (flow_loop_mixed) and none travel through registers; the classifier's
 // pieces follow them in the stream in their usual form, and the ring starts afresh for them.
+// n_tok: steps of the token loop (reference src/inference.jl:349-386) that this launch runs, one after the other; the
+// epochs of step t start at gen0 + t * (5 * n_layers + 2).
 template <int T_CLS, bool MIXED>
-__global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
+__global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int n_tok) {
     const FlowArgs &a = c_flow;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = blockIdx.x, nwg = gridDim.x;
     unsigned char *ring_base = s_ring + wave * (FLOW_D * FLOW_SLOT);
-
+    // the launch's first step as the control block has it; workgroup 0 advances the block after every step
+    // (flow_pick_token), the others count for themselves
+    const int pos_first = a.ctl->pos, step_first = a.ctl->step, n_prompt = a.ctl->n_prompt, tok_first = a.ctl->last_argmax;
+    if (tid == 0) s_flag = 0;
     Ring r;
-    r.gptr = a.stream + a.wave_off[wg * FLOW_NW + wave];
-    r.lds = (unsigned)(size_t)ring_base;
-    r.issued = r.consumed = r.drain_mark = 0;
-    r.off = 0;
     MRing mr;
     unsigned char *mring_base = s_ring + wave * (FLOWM_D * FLOWM_SLOT);
     const unsigned char *reg_ptr = nullptr;
     RegPieces rp;
+#ifdef L2H_TIMELINE
+    int tl_n = 0;
+#define FTL()                                                                                   \
+    do {                                                                                        \
+        if (a.timeline && tid == 0 && tl_n < 64) a.timeline[wg * 64 + tl_n++] = wall_clock64(); \
+    } while (0)
+#define FTLS()          \
+    do {                \
+        __syncthreads(); \
+        FTL();          \
+    } while (0)
+#else
+#define FTL()
+#define FTLS()
+#endif
+#define LEAVE()        \
+    do {               \
+        flow_drain(r); \
+        return;        \
+    } while (0)
+    // (flow_drain waits for everything this wavefront has requested, whichever ring it went to)
+#pragma nounroll
+  for (int t_step = 0; t_step < n_tok; t_step++) {
+    // the rings start at the head of the streams (their areas are free: the step before ended with a wait for all of
+    // its pieces): requested before the step's token is there
+    r.gptr = a.stream + a.wave_off[wg * FLOW_NW + wave];
+    r.lds = (unsigned)(size_t)ring_base;
+    r.issued = r.consumed = r.drain_mark = 0;
+    r.off = 0;
     if constexpr (MIXED) {
         mr.gptr = r.gptr;
         mr.lds = (unsigned)(size_t)mring_base;
@@ -1794,41 +1857,26 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
                       (int64_t)flow_wave_pieces(a.cls, wg, wave) * (T_CLS == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT));
         flow_top_up_q4(r, ring_base, lane);
     }
-
-#ifdef L2H_TIMELINE
-    int tl_n = 0;
-#define FTL()                                                                                   \
-    do {                                                                                        \
-        if (a.timeline && tid == 0 && tl_n < 64) a.timeline[wg * 64 + tl_n++] = wall_clock64(); \
-    } while (0)
-#define FTLS()          \
-    do {                \
-        __syncthreads(); \
-        FTL();          \
-    } while (0)
-#else
-#define FTL()
-#define FTLS()
-#endif
     FTL();
-#define LEAVE()        \
-    do {               \
-        flow_drain(r); \
-        return;        \
-    } while (0)
-    // (flow_drain waits for everything this wavefront has requested, whichever ring it went to)
 
     // ---- this step's token, position and RoPE angles (reference src/inference.jl:122-127) ----
-    const int pos = a.ctl->pos;
-    const int tok = a.ctl->step < a.ctl->n_prompt ? a.prompt[a.ctl->step] : a.ctl->last_argmax;
-    if (tid == 0) s_flag = 0;
+    const unsigned E0 = gen0 + (unsigned)t_step * (5u * (unsigned)a.n_layers + 2u);
+    const int pos = pos_first + t_step, step = step_first + t_step;
+    int tok = tok_first;
+    if (t_step > 0) {
+        tok = uni(flow_next_token(E0));
+        if (tok < 0) {
+            if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            LEAVE();
+        }
+    }
+    if (step < n_prompt) tok = a.prompt[step];
     if (tid < (a.hs >> 1)) {
         float theta = 1.0f * (float)pos;
         for (int k = 0; k < tid; k++) theta *= a.theta_scale;
         s_rope[2 * tid] = (float)cos((double)theta);
         s_rope[2 * tid + 1] = (float)sin((double)theta);
     }
-    const unsigned E0 = gen0;
     // attention of head h runs on workgroup h * stride + h % stride (spread over the XCDs)
     const int att_stride = nwg / a.n_heads;
     const int att_h = uni(wg / att_stride);
@@ -1958,7 +2006,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0) {
         flow_loop_q4<false, false>(a.cls, r, ring_base, wg, rp, 0);
     flow_finish_cls(wg, e_cls);
     flow_drain(r);
-    if (wg == 0) flow_pick_token(nwg, e_cls);
+    if (wg == 0) flow_pick_token(nwg, e_cls, t_step + 1 < n_tok ? e_cls + 1 : 0u);
+  }
 #undef LEAVE
 }
 
@@ -2126,11 +2175,13 @@ __device__ __forceinline__ void flow_loop_f32(const F32Pre &pre, const FlowGeom 
 #undef F32_FMA4
 }
 
-__global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
+__global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0, int n_tok) {
     const FlowArgs &a = c_flow;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = blockIdx.x, nwg = gridDim.x;
     (void)wave;
+    const int pos_first = a.ctl->pos, step_first = a.ctl->step, n_prompt = a.ctl->n_prompt, tok_first = a.ctl->last_argmax;
+    if (tid == 0) s_flag = 0;
 #ifdef L2H_TIMELINE
     int tl_n = 0;
 #define XTL()                                                                                   \
@@ -2140,18 +2191,27 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
 #else
 #define XTL()
 #endif
+#pragma nounroll
+  for (int t_step = 0; t_step < n_tok; t_step++) {
     XTL();
     // ---- this step's token, position and RoPE angles (reference src/inference.jl:122-127) ----
-    const int pos = a.ctl->pos;
-    const int tok = a.ctl->step < a.ctl->n_prompt ? a.prompt[a.ctl->step] : a.ctl->last_argmax;
-    if (tid == 0) s_flag = 0;
+    const unsigned E0 = gen0 + (unsigned)t_step * (5u * (unsigned)a.n_layers + 2u);
+    const int pos = pos_first + t_step, step = step_first + t_step;
+    int tok = tok_first;
+    if (t_step > 0) {
+        tok = uni(flow_next_token(E0));
+        if (tok < 0) {
+            if (tid == 0) __hip_atomic_store(a.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return;
+        }
+    }
+    if (step < n_prompt) tok = a.prompt[step];
     if (tid < (a.hs >> 1)) {
         float theta = 1.0f * (float)pos;
         for (int k = 0; k < tid; k++) theta *= a.theta_scale;
         s_rope[2 * tid] = (float)cos((double)theta);
         s_rope[2 * tid + 1] = (float)sin((double)theta);
     }
-    const unsigned E0 = gen0;
     const int att_stride = nwg / a.n_heads;
     const int att_h = uni(wg / att_stride);
     const bool is_att = uni((int)(att_h < a.n_heads && wg % att_stride == att_h % att_stride)) != 0;
@@ -2214,7 +2274,8 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0) {
     if (!uni(flow_stage_xf<PRO_RMSNORM, SRC_BARE>(a.x_a, a.dim, a.rms_final, tok))) return;
     flow_loop_f32<true>(pre, a.cls, 4, 0, wg, a.dim);
     flow_finish_cls(wg, e_cls);
-    if (wg == 0) flow_pick_token(nwg, e_cls);
+    if (wg == 0) flow_pick_token(nwg, e_cls, t_step + 1 < n_tok ? e_cls + 1 : 0u);
+  }
 #undef XTL
 }
 
@@ -2562,8 +2623,8 @@ bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed) {
 
 // A plain launch: a cooperative one costs about 20 µs more per token on this stack, and all it would add is the
 // residency check that k_flow_fits makes once.
-hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid, bool mixed) {
-    void *args[] = {&gen0};
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int n_tok, int cls_type, int grid, bool mixed) {
+    void *args[] = {&gen0, &n_tok};
     const void *fn = flow_kernel_fn(cls_type, mixed);
     return hipLaunchKernel(fn, dim3(grid), dim3(1024), args, 0, s);
 }

@@ -158,6 +158,7 @@ struct FlowArgs {
     int max_out;
     unsigned int gen0, spin_limit;
     unsigned int *abort_flag;
+    unsigned long long *tokw;  // {token, epoch} in eight copies, 16 words apart: the token of a launch's next step, from workgroup 0 to all
     int dim, hidden, hs, n_heads, n_kv_heads, kv_dim, seq_len, n_layers, vocab, neox;
     int kv16;     // the KV cache holds fp16 elements (typed-piece instantiation of the kernel only)
     int dim_pad;  // dim rounded up to whole pieces (2048): rows of dim inputs are padded with zero super-blocks in the streams
@@ -196,7 +197,8 @@ struct FlowTypedDev {  // the same on the device, for the repack kernel (null fo
 hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream, const int64_t *wave_off_dev, int kind,
                          int layer, const DevTensor *w, int nw, int grid, int cls_type, const FlowTypedDev &typed);
 hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a);
-hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int cls_type, int grid, bool mixed);
+// one launch runs n_tok steps of the token loop; the epochs of the launch start at gen0 and take 5 * n_layers + 2 per step
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int n_tok, int cls_type, int grid, bool mixed);
 bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed);
 
 // ---- launchers (kernel files) ----------------------------------------------------------------

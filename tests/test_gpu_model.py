@@ -299,6 +299,36 @@ def test_streaming_kernel_long_cache(pkg, orc, rng, case, n_pre, seq_len):
     assert _rel(logits, ref_logits) <= 1e-3
 
 
+@pytest.mark.parametrize("case,steps", [("q4ks_headline_widths", 5), ("q5km_typed", 3), ("f32_rows", 7), ("phi3_widths", 64)])
+def test_several_steps_per_launch(pkg, monkeypatch, case, steps):
+    """One launch of the streaming kernel can run several steps of the token loop (the next token passes from workgroup
+    0 to the others inside the kernel; the cache then lives in uncached memory, so that rows appended in one step are
+    seen by every XCD in the next).  The library does so by itself where no two heads share a cache row; here it is
+    forced for the shapes with shared rows too (L2H_KV_UNCACHED, L2H_FLOW_STEPS: read when the model is finalized), with
+    step counts that do not divide the prompt or the generation: same tokens and final logits as one step per launch
+    and as the per-phase path, over a prompt and 50 generated tokens."""
+    from llama2_jl_amd import synth
+    plan, kw = FLOW_CASES[case]
+    lm = _model(pkg, plan, **kw)
+    prompt = synth.seeded_prompt(23, 9, lm.config.vocab_size)
+    n_new = min(50, lm.config.seq_len - len(prompt))
+    got = []
+    for env in ({"L2H_KV_UNCACHED": "1", "L2H_FLOW_STEPS": str(steps)}, {"L2H_KV_UNCACHED": "0", "L2H_FLOW_STEPS": "1"}, None):
+        for k in ("L2H_KV_UNCACHED", "L2H_FLOW_STEPS"):
+            monkeypatch.delenv(k, raising=False)
+        for k, v in (env or {}).items():
+            monkeypatch.setenv(k, v)
+        lm._device = None
+        dev = lm.device(path=3 if env is not None else 1)
+        assert dev.path == (3 if env is not None else 1)
+        ids, logits = dev.generate_greedy(prompt, n_new, want_logits=True)
+        got.append((np.asarray(ids).tolist(), logits.copy()))
+        dev.close()
+    for other in got[1:]:
+        assert other[0] == got[0][0]
+        assert np.array_equal(other[1].view(np.uint32), got[0][1].view(np.uint32))
+
+
 def test_streaming_kernel_gives_up_and_recovers(pkg):
     """A wait bound of zero makes the first poll that finds a word missing give up: every workgroup leaves
     the kernel, the call fails, and after a reset with the normal bound the model decodes as before (the
