@@ -28,10 +28,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
 # timed region):
 #   (8b-q4ks, launch path 1): per matvec launch, 31.23 MB read + 0.04 MB written (profiles/pmc_fetch_write_bench_8b-q4ks.md)
 #   launch path 3, per token launch (profiles/pmc_fetch_write_streaming_kernel_all_workloads.md):
-#     8b-q4ks 4500.9 MB read + 9.3 MB written, 8b-q5km 5760.0 + 9.3, phi3-4k 5858.9 + 38.9, llama2c-f32 172.6 + 0.8,
+#     8b-q4ks 4500.9 MB read + 9.3 MB written, 8b-q5km 5760.0 + 9.3, phi3-4k 5316.8 + 40.5 (per step: its launches run
+#     eight), llama2c-f32 172.6 + 0.8,
 #     8b-q4ks-prefill (its decode steps at positions 2048 and up) 5021.0 + 67.1
 MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4510221000, ("8b-q5km", 3): 5769380000,
-                                     ("phi3-4k", 3): 5897871000, ("llama2c-f32", 3): 173480000,
+                                     ("phi3-4k", 3): 5357300000, ("llama2c-f32", 3): 173480000,
                                      ("8b-q4ks-prefill", 3): 5088146000}
 
 WORKLOADS = {
@@ -215,6 +216,7 @@ def main():
     bytes_per_launch, launches, avg_launch_us = int(tot_b / max(1, n_launch)), n_launch, tot_us / max(1, n_launch)
     if dev.path == 3:
         kernel_name = "flow_token_kernel (whole token: q4_K/q6_K x q8_K matvecs, attention, argmax)"
+        # (a kernel launch runs dev.steps_per_launch steps of the token loop; bytes, traffic and time are per step)
         bytes_per_launch, launches, avg_launch_us = int(bytes_per_token), 1, ev_ms * 1e3 / K
         achieved = bytes_per_launch / avg_launch_us / 1e3
         log("streaming kernel: %.1f us per launch (HIP events), %.0f GB/s of algorithmic bytes" % (avg_launch_us, achieved))
@@ -266,6 +268,7 @@ def main():
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                      "bytes_per_launch": bytes_per_launch, "launches_per_token": launches,
+                     "token_steps_per_kernel_launch": getattr(dev, "steps_per_launch", 1),
                      "avg_launch_us": round(avg_launch_us, 2), "per_phase_kernels": per_kernel,
                      "measured_stream_read_GBs": round(stream_gbs, 1)},
         "cpu_baseline": cpu,

@@ -115,6 +115,10 @@ int l2h_model_set_kv_type(l2h_model *m, int kv_type);
  * the choice after finalize (1, 2 or 3). */
 int l2h_model_set_path(l2h_model *m, int path);
 int l2h_model_path(l2h_model *m);
+/* Steps of the token loop (src/inference.jl:349-386) that one kernel launch of l2h_generate_greedy runs: 1, or up to 8
+ * on path 3 for a model in which no two heads share a cache row (n_kv_heads == n_heads; the cache then lies in uncached
+ * memory).  No counterpart in the reference. */
+int l2h_model_steps_per_launch(l2h_model *m);
 /* After finalize with the automatic choice: why the streaming kernel (path 3) was not taken, e.g. "layer matrices
  * must be q4_K" for a file whose first layers hold q5_K attn_v / ffn_down tensors; "" when it was taken.  The
  * string lives as long as the model. */

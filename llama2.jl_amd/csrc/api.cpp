@@ -417,6 +417,7 @@ extern "C" const char *l2h_model_path_reason(l2h_model *m) {
     return m->flow_why.c_str();
 }
 
+extern "C" int l2h_model_steps_per_launch(l2h_model *m) { return (m && m->finalized && m->flow) ? m->flow_steps_per_launch : 1; }
 extern "C" int l2h_model_path(l2h_model *m) { return (m && m->finalized) ? (m->flow ? 3 : (m->mega ? 2 : 1)) : 0; }
 
 extern "C" int l2h_model_get_tensor(l2h_model *m, int role, int layer, void *host, int64_t host_bytes) {
@@ -765,7 +766,7 @@ static int flow_setup(l2h_model *m) {
         m->flow_why = "norm weight slabs differ";
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: norm weight slabs differ") : L2H_OK;
     }
-    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount, a.mixed != 0)) {
+    if (!k_flow_fits(cls_type, grid, ctx->prop.multiProcessorCount, flow_form(a))) {
         m->flow_why = "its workgroups do not fit the device at once";
         return required ? set_err(ctx, L2H_EINVAL, "streaming kernel not available: its workgroups do not fit the device at once")
                         : L2H_OK;
@@ -902,7 +903,7 @@ static hipError_t flow_launch_tokens(l2h_model *m, int n_tok) {
         if (eb != hipSuccess) return eb;
         g_flow_bound = m;
     }
-    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, n_tok, m->flow_cls_type, m->flow_grid, m->flow_args.mixed != 0);
+    hipError_t e = k_flow_launch(m->ctx->stream, m->flow_gen, n_tok, m->flow_cls_type, m->flow_grid, flow_form(m->flow_args));
     if (e == hipSuccess) m->flow_gen += (unsigned)n_tok * (5u * (unsigned)m->c.n_layers + 2u);
     return e;
 }

@@ -118,15 +118,39 @@ __host__ __device__ inline int flow_n_local(const FlowGeom &g, int wg) {
     const int hi = lo + g.rpw < g.n_rows ? lo + g.rpw : g.n_rows;
     return hi > lo ? hi - lo : 0;
 }
+// Rows that end in the middle of a piece (FlowGeom::ppr == 0) come in pairs of flow_half() pieces: rpw and n_rows are
+// even.  H = false: the caller knows that the geometry has none (kernels that are not built for them do not look).
+template <bool H = true>
+__host__ __device__ inline int flow_half(const FlowGeom &g) {
+    return H && g.ppr == 0 ? g.K >> 10 : 0;
+}
+// pieces of a workgroup's rows
+template <bool H = true>
+__host__ __device__ inline int flow_wg_pieces(const FlowGeom &g, int wg) {
+    const int n = flow_n_local(g, wg), h = flow_half<H>(g);
+    return h ? (n >> 1) * h : n * g.ppr;
+}
+// the first logical row that piece j of a workgroup holds super-blocks of
+__host__ __device__ inline int flow_piece_row(const FlowGeom &g, int j) {
+    const int h = flow_half(g);
+    return h ? 2 * (j / h) : j / g.ppr;
+}
+// pieces of a workgroup with a full share of rows
+__host__ __device__ inline int flow_wg_capacity(const FlowGeom &g) {
+    const int h = flow_half(g);
+    return h ? (g.rpw >> 1) * h : g.rpw * g.ppr;
+}
 // pieces of workgroup wg that wavefront `wave` takes: a contiguous run of the workgroup's pieces
 // (consecutive pieces of a row stay in one wavefront where possible), the first np % 16 wavefronts
 // one piece longer than the rest
+template <bool H = true>
 __host__ __device__ inline int flow_wave_pieces(const FlowGeom &g, int wg, int wave) {
-    const int np = flow_n_local(g, wg) * g.ppr;
+    const int np = flow_wg_pieces<H>(g, wg);
     return np / FLOW_NW + (wave < np % FLOW_NW ? 1 : 0);
 }
+template <bool H = true>
 __host__ __device__ inline int flow_wave_start(const FlowGeom &g, int wg, int wave) {
-    const int np = flow_n_local(g, wg) * g.ppr;
+    const int np = flow_wg_pieces<H>(g, wg);
     const int base = np / FLOW_NW, rem = np % FLOW_NW;
     return wave * base + (wave < rem ? wave : rem);
 }
@@ -139,13 +163,15 @@ __host__ __device__ inline int flow_wave_start(const FlowGeom &g, int wg, int wa
 #ifndef FLOW_R
 #define FLOW_R 1
 #endif
+template <bool H = true>
 __host__ __device__ inline int flow_reg_pieces(const FlowGeom &g, int wg, int wave) {
-    const int cnt = flow_wave_pieces(g, wg, wave);
+    const int cnt = flow_wave_pieces<H>(g, wg, wave);
     return cnt < FLOW_R ? cnt : FLOW_R;
 }
 // pieces of a layer phase that go through the ring
+template <bool H = true>
 __host__ __device__ inline int flow_ring_pieces(const FlowGeom &g, int wg, int wave) {
-    return flow_wave_pieces(g, wg, wave) - flow_reg_pieces(g, wg, wave);
+    return flow_wave_pieces<H>(g, wg, wave) - flow_reg_pieces<H>(g, wg, wave);
 }
 
 // logical row L of a phase -> (tensor of the phase, row in it).  Logical rows put the two rows an
@@ -218,12 +244,15 @@ __device__ __forceinline__ void flow_decode_field(uint32_t f, int &sc_a, int &sc
 }
 
 // geometry of layer phase `kind`, field by field (scalar selects of scalar loads)
+// (HALF: only a kernel built for rows that end inside a piece looks at that field; for the others it is a constant zero)
+template <bool HALF = false>
 __device__ __forceinline__ FlowGeom flow_geom(const FlowArgs &a, int kind) {
     FlowGeom g;
     g.n_rows = kind == 0 ? a.qkv.n_rows : (kind == 1 ? a.wo.n_rows : (kind == 2 ? a.w13.n_rows : a.w2.n_rows));
     g.rpw = kind == 0 ? a.qkv.rpw : (kind == 1 ? a.wo.rpw : (kind == 2 ? a.w13.rpw : a.w2.rpw));
     g.ppr = kind == 0 ? a.qkv.ppr : (kind == 1 ? a.wo.ppr : (kind == 2 ? a.w13.ppr : a.w2.ppr));
     g.K = 0;
+    if (HALF) g.K = kind == 0 ? a.qkv.K : (kind == 1 ? a.wo.K : (kind == 2 ? a.w13.K : a.w2.K));
     return g;
 }
 
@@ -620,7 +649,7 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
     asm volatile("" : "+v"(lane));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
-    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    const int cnt = uni(flow_wave_pieces<false>(g, wg, wave)), start = uni(flow_wave_start<false>(g, wg, wave));
     RingLoop<FLOW_SLOT, FLOW_D, 2> q;
     q.begin(r);
     const int left0 = q.left;
@@ -739,7 +768,7 @@ __device__ __forceinline__ void flow_top_up_q6(Ring &r, unsigned char *ring_base
 __device__ __forceinline__ void flow_loop_q6(const FlowGeom &g, Ring &r, unsigned char *ring_base, int wg) {
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int ppr = uni(g.ppr);
-    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    const int cnt = uni(flow_wave_pieces<false>(g, wg, wave)), start = uni(flow_wave_start<false>(g, wg, wave));
     const int b = lane >> 2, c = lane & 3, n = c >> 1, h = c & 1;
     const XLds x = flow_x();
     RingLoop<FLOW_Q6_PIECE, FLOW_Q6_D, 5> q;
@@ -894,13 +923,16 @@ __device__ __forceinline__ double flow_q6_term(const uint4 ql, const uint4 qh, u
 }
 
 // the streaming loop over typed pieces; partial sums as in flow_loop_q4<., true> (four doubles per piece)
+template <bool HALF = false>
 __device__ __forceinline__ void flow_loop_mixed(const FlowGeom &g, MRing &r, unsigned char *ring_base, int wg) {
     int lane = threadIdx.x & 63;
     asm volatile("" : "+v"(lane));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int ppr = uni(g.ppr);
-    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
-    int part = uni(start % ppr);
+    // rows that end in the middle of a piece (flow_half() pieces per pair of rows): the lane's super-block is number
+    // 8 part + blk of the pair's 2 nb_row; from nb_row on it belongs to the odd row
+    const int half = uni(flow_half<HALF>(g)), unit = half ? half : uni(g.ppr), mid = half >> 1, nb_row = 4 * half;
+    const int cnt = uni(flow_wave_pieces<HALF>(g, wg, wave)), start = uni(flow_wave_start<HALF>(g, wg, wave));
+    int part = uni(start % unit);
     const int blk = lane >> 3, c8 = lane & 7;
     // q4_K / q5_K: sub-block pair c8 / 2, half c8 % 2.  q6_K: n = c8 / 4, w = (c8 / 2) % 2, h = c8 % 2.
     const int pair = c8 >> 1, w32 = (c8 >> 1) & 1;
@@ -935,9 +967,10 @@ __device__ __forceinline__ void flow_loop_mixed(const FlowGeom &g, MRing &r, uns
         const unsigned a_w = sl + (t == 0 ? 144u : (t == 1 ? 400u : 672u)) + lane * 16;
         const unsigned a_h = sl + blk * 16;
         const unsigned a_q = sl + (six ? q6h : q5h);
-        const unsigned a_xlo = (six ? x6 : x45) + po * 64, a_xhi = a_xlo + (six ? 64u : 32u);
-        const unsigned a_bsa = (six ? bs6 : bs45) + po * 8, a_bsb = a_bsa + (six ? 8u : 4u);
-        const unsigned a_yd = xd0 + po, a_tag = sl + 128, a_d = sl + 144 + 2 * blk;
+        const unsigned back = (half && 8 * part + blk >= nb_row) ? (unsigned)(4 * nb_row) : 0u;  // (the odd row starts anew)
+        const unsigned a_xlo = (six ? x6 : x45) + (po - back) * 64, a_xhi = a_xlo + (six ? 64u : 32u);
+        const unsigned a_bsa = (six ? bs6 : bs45) + (po - back) * 8, a_bsb = a_bsa + (six ? 8u : 4u);
+        const unsigned a_yd = xd0 + (po - back), a_tag = sl + 128, a_d = sl + 144 + 2 * blk;
         uint4 w, hdr, qh, xlo, xhi;
         int bs_a, bs_b;
         float yd;
@@ -973,15 +1006,30 @@ __device__ __forceinline__ void flow_loop_mixed(const FlowGeom &g, MRing &r, uns
             else
                 acc += flow_q4_term(w, hdr.x, sc_a, sc_b, m_a, m_b, xlo, xhi, bs_a, bs_b, yd);
         }
-        // (as FLOW_PIECE_DONE of flow_loop_q4)
+        // (as FLOW_PIECE_DONE of flow_loop_q4.)  Rows that end inside a piece: the upper half of the lanes goes over to
+        // the odd row behind piece mid - 1 and the lower half behind piece mid, and each hands in its sums of the even row
+        // there; what a piece's four quarter sums belong to is thereby fixed: to the even row up to the middle piece's
+        // second quarter, to the odd row from its third.
+        const int done = part;
         part++;
         po += 32;
         double v_ = 0.0;
-        if (k == 1 || part == ppr) {
-            v_ = row16_sum_f64_dpp(acc);
-            acc = 0.0;
-            po = 0;
-            part = 0;
+        if constexpr (!HALF) {
+            if (k == 1 || part == unit) {
+                v_ = row16_sum_f64_dpp(acc);
+                acc = 0.0;
+                po = 0;
+                part = 0;
+            }
+        } else {
+            const bool last = k == 1 || part == unit;
+            if (last || (half && (done == mid || done + 1 == mid))) {
+                const double red = row16_sum_f64_dpp(acc);
+                const bool mine = last || (done == mid ? lane < 32 : lane >= 32);
+                v_ = mine ? red : 0.0;
+                acc = mine ? 0.0 : acc;
+                if (!half || part == unit) po = 0, part = 0;  // (a wavefront's last piece ends the loop)
+            }
         }
         *out = v_;
         out += 4;
@@ -1015,7 +1063,17 @@ __device__ __forceinline__ void flow_row_values(int n_local, int ppr) {
 }
 
 // the same for one row, straight from the partial sums (the layer epilogues: one barrier instead of two)
-__device__ __forceinline__ float flow_row_value4(int lr, int ppr) {
+// (HALF: the geometry may have rows that end inside a piece; see flow_loop_mixed for what belongs to which row)
+template <bool HALF = false>
+__device__ __forceinline__ float flow_row_value4(int lr, int ppr, int half = 0) {
+    if (HALF && half) {
+        const int mid = half >> 1, odd = lr & 1;
+        const double *h4 = s_part + 4 * (lr >> 1) * half;
+        double v = 0.0;
+        for (int p = odd ? mid + 1 : 0; p < (odd ? half : mid); p++) v += (h4[4 * p] + h4[4 * p + 1]) + (h4[4 * p + 2] + h4[4 * p + 3]);
+        v += h4[4 * mid + 2 * odd] + h4[4 * mid + 2 * odd + 1];
+        return (float)v;
+    }
     const double *q4 = s_part + 4 * lr * ppr;
     double v = 0.0;
     // (the quarter sums of up to four pieces are read before any is added: one LDS latency per four pieces, not per piece)
@@ -1041,7 +1099,7 @@ __device__ __forceinline__ float flow_pair_value(float own) { return dpp_f32<DPP
 // a round trip to memory that would stand between the publication of a phase's results and the next
 // phase's requests.)
 // rope! (reference src/inference.jl:112-157) and the cache append (:259-260)
-template <bool ANY_HS = false>
+template <bool ANY_HS = false, bool HALF = false>
 __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned e_q) {
     l = uni(l), wg = uni(wg), pos = uni(pos), e_q = uni(e_q);
     const FlowArgs &a = c_flow;
@@ -1054,7 +1112,7 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
     int seg, row;
     flow_row_src(0, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row, ANY_HS);
     // (rows come in pairs and a workgroup's run of them is even, so the partner's thread is here too)
-    const float val = flow_row_value4(tid, a.qkv.ppr), other = flow_pair_value(val);
+    const float val = flow_row_value4<HALF>(tid, a.qkv.ppr, flow_half<HALF>(a.qkv)), other = flow_pair_value(val);
     const int hs_log = 31 - __builtin_clz(a.hs);  // (a power of two unless ANY_HS)
     const int hh = ANY_HS ? row / a.hs : row >> hs_log, e = ANY_HS ? row - hh * a.hs : row & (a.hs - 1);
     if (seg == 2) {
@@ -1089,6 +1147,7 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
 
 // dst = old + result (x .+= ..., :284,305); which = 1 after wo (-> x_b), 3 after w2 (-> x_a); `old` is
 // this thread's row of the other buffer, fetched before the loop (the same thread wrote it)
+template <bool HALF = false>
 __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned oldw) {
     which = uni(which), wg = uni(wg);
     const FlowArgs &a = c_flow;
@@ -1102,13 +1161,14 @@ __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned ol
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
     const float old = bare_read(src + row, oldw);
-    bare_store(dst + row, bare_of(old + flow_row_value4(tid, g.ppr)));
+    bare_store(dst + row, bare_of(old + flow_row_value4<HALF>(tid, g.ppr, flow_half<HALF>(g))));
     bare_store(src + row, FLOW_EMPTY);  // (its readers are through: see FLOW_EMPTY)
 }
 
 // SwiGLU (:295-299): logical rows (2u, 2u+1) are w1 row u and w3 row u.  The arithmetic (an fp64 exp) is a
 // function of its own for the registers it takes; the stores are the caller's: a function that stores
 // waits before it returns until the stores are acknowledged.
+template <bool HALF = false>
 __device__ __noinline__ unsigned flow_w13_word(int wg) {
     wg = uni(wg);
     const FlowArgs &a = c_flow;
@@ -1117,13 +1177,14 @@ __device__ __noinline__ unsigned flow_w13_word(int wg) {
     asm volatile("" : "+v"(tid));
     flow_barrier_lds();
     if (tid >= n_local) return 0u;
-    const float own = flow_row_value4(tid, a.w13.ppr), next = flow_pair_value(own);  // (w1 row u | w3 row u, threads 2u | 2u+1)
+    const float own = flow_row_value4<HALF>(tid, a.w13.ppr, flow_half<HALF>(a.w13)), next = flow_pair_value(own);  // (w1 row u | w3 row u, threads 2u | 2u+1)
     if (tid & 1) return 0u;
     return bare_of(swiglu_val(own, next));
 }
+template <bool HALF = false>
 __device__ __forceinline__ void flow_finish_w13(int wg, unsigned e_out) {
     const FlowArgs &a = c_flow;
-    const unsigned v = flow_w13_word(wg);
+    const unsigned v = flow_w13_word<HALF>(wg);
     int tid = threadIdx.x;
     asm volatile("" : "+v"(tid));
     if (tid >= flow_n_local(a.w13, wg) || (tid & 1)) return;
@@ -1790,7 +1851,8 @@ __device__ __noinline__ bool flow_attention_split(int layer, int pos, unsigned e
 // pieces follow them in the stream in their usual form, and the ring starts afresh for them.
 // n_tok: steps of the token loop (reference src/inference.jl:349-386) that this launch runs, one after the other; the
 // epochs of step t start at gen0 + t * (5 * n_layers + 2).
-template <int T_CLS, bool MIXED>
+// HALF (with MIXED): the layer matrices' rows of dim inputs end in the middle of a piece (FlowGeom::half)
+template <int T_CLS, bool MIXED, bool HALF = false>
 __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int n_tok) {
     const FlowArgs &a = c_flow;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1837,8 +1899,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
     if constexpr (MIXED) {
         mr.gptr = r.gptr;
         mr.lds = (unsigned)(size_t)mring_base;
-        mr.left = a.n_layers * (flow_wave_pieces(a.qkv, wg, wave) + flow_wave_pieces(a.wo, wg, wave) +
-                                flow_wave_pieces(a.w13, wg, wave) + flow_wave_pieces(a.w2, wg, wave));
+        mr.left = a.n_layers * (flow_wave_pieces<HALF>(a.qkv, wg, wave) + flow_wave_pieces<HALF>(a.wo, wg, wave) +
+                                flow_wave_pieces<HALF>(a.w13, wg, wave) + flow_wave_pieces<false>(a.w2, wg, wave));
         {
             const unsigned long long p = (unsigned long long)mr.gptr;
             mr.gptr = (const unsigned char *)(((unsigned long long)uni((unsigned)(p >> 32)) << 32) | uni((unsigned)p));
@@ -1848,13 +1910,13 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
         flowm_start(mr, mring_base, uni(a.wave_types[wg * FLOW_NW + wave]), lane);
     } else {
         // the layers' pieces and, where the classifier is q4_K too, its pieces behind them: one stream
-        const int ring_layer = flow_ring_pieces(a.qkv, wg, wave) + flow_ring_pieces(a.wo, wg, wave) +
-                               flow_ring_pieces(a.w13, wg, wave) + flow_ring_pieces(a.w2, wg, wave);
-        r.left = a.n_layers * ring_layer + (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces(a.cls, wg, wave) : 0);
+        const int ring_layer = flow_ring_pieces<false>(a.qkv, wg, wave) + flow_ring_pieces<false>(a.wo, wg, wave) +
+                               flow_ring_pieces<false>(a.w13, wg, wave) + flow_ring_pieces<false>(a.w2, wg, wave);
+        r.left = a.n_layers * ring_layer + (T_CLS == L2H_TYPE_Q4_K ? flow_wave_pieces<false>(a.cls, wg, wave) : 0);
         ring_uniform(r);  // values that came through vector loads are the same on every lane: make them scalar
         // the register pieces follow the ring's part of the stream, in the order in which they are used
         reg_ptr = uni(r.gptr + (int64_t)a.n_layers * ring_layer * FLOW_SLOT +
-                      (int64_t)flow_wave_pieces(a.cls, wg, wave) * (T_CLS == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT));
+                      (int64_t)flow_wave_pieces<false>(a.cls, wg, wave) * (T_CLS == L2H_TYPE_Q6_K ? FLOW_Q6_PIECE : FLOW_SLOT));
         flow_top_up_q4(r, ring_base, lane);
     }
     FTL();
@@ -1903,8 +1965,8 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
             int tid = threadIdx.x;
             asm volatile("" : "+v"(tid));
             const int lane = tid & 63;
-            const FlowGeom g = flow_geom(a, kind);
-            const int n_reg = MIXED ? 0 : uni(flow_reg_pieces(g, wg, wave));
+            const FlowGeom g = flow_geom<HALF>(a, kind);
+            const int n_reg = MIXED ? 0 : uni(flow_reg_pieces<false>(g, wg, wave));
             if (!MIXED && kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
 #ifdef L2H_TIMELINE
             if (tid == 0) s_tl_fine = ((int)gridDim.x > 101 && wg == 101 && l == 2) ? 256 * 64 + 512 + kind * 8 : -1;
@@ -1949,7 +2011,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
             if (kind == 0 && is_att && pos < FLOW_ATT_SHORT && !(MIXED && a.kv16)) flow_touch_cache(l, att_h, pos);
             if constexpr (MIXED) {
                 // rows of dim inputs padded to whole pieces: the q8_K blocks beyond dim are zero (d = 0, no quants)
-                if (kind != 3 && a.dim_pad > a.dim) {
+                if (kind != 3 && a.dim_pad > a.dim && !flow_half<HALF>(g)) {
                     const int b0 = a.dim >> 8, nbz = (a.dim_pad - a.dim) >> 8;
                     unsigned char *q8 = (unsigned char *)s_act;
                     for (int i = tid; i < nbz * 64; i += 1024) ((uint32_t *)(q8 + 256 * b0))[i] = 0u;
@@ -1957,20 +2019,20 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
                     if (tid < nbz) ((float *)(q8 + 14336 + 1792))[b0 + tid] = 0.f;
                     __syncthreads();
                 }
-                flow_loop_mixed(g, mr, mring_base, wg);
+                flow_loop_mixed<HALF>(g, mr, mring_base, wg);
             } else {
                 flow_loop_q4<true, true>(g, r, ring_base, wg, rp, n_reg);
             }
             FTL();
             FTLS();
             if (kind == 0)
-                flow_finish_qkv<MIXED>(l, wg, pos, e_q);
+                flow_finish_qkv<MIXED, HALF>(l, wg, pos, e_q);
             else if (kind == 1)
-                flow_finish_resid(1, wg, oldw);
+                flow_finish_resid<HALF>(1, wg, oldw);
             else if (kind == 2)
-                flow_finish_w13(wg, e_w13);
+                flow_finish_w13<HALF>(wg, e_w13);
             else
-                flow_finish_resid(3, wg, oldw);
+                flow_finish_resid<HALF>(3, wg, oldw);
             FTL();
         }
     }
@@ -1983,7 +2045,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
         if constexpr (MIXED) r.gptr = mr.gptr;
         r.issued = r.consumed = r.drain_mark = 0;
         r.off = 0;
-        r.left = flow_wave_pieces(a.cls, wg, wave);
+        r.left = flow_wave_pieces<false>(a.cls, wg, wave);
         ring_uniform(r);
         if (T_CLS == L2H_TYPE_Q6_K)
             flow_top_up_q6(r, ring_base, lane);
@@ -2113,7 +2175,7 @@ __device__ __forceinline__ void flow_f32_request(F32Pre &pre, const FlowGeom &g,
     int lane = threadIdx.x & 63;
     asm volatile("" : "+v"(lane));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    const int cnt = uni(flow_wave_pieces<false>(g, wg, wave)), start = uni(flow_wave_start<false>(g, wg, wave));
     if (cnt <= 0) return;
     const int n4 = (K / g.ppr) >> 2;
 #pragma unroll
@@ -2130,7 +2192,7 @@ __device__ __forceinline__ void flow_loop_f32(const F32Pre &pre, const FlowGeom 
     int lane = threadIdx.x & 63;
     asm volatile("" : "+v"(lane));
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int cnt = uni(flow_wave_pieces(g, wg, wave)), start = uni(flow_wave_start(g, wg, wave));
+    const int cnt = uni(flow_wave_pieces<false>(g, wg, wave)), start = uni(flow_wave_start<false>(g, wg, wave));
     const int n4 = (K / g.ppr) >> 2;
 #define F32_FMA4(ACC_, W_, X_)                       \
     ACC_ = fma((double)W_.x, (double)X_.x, ACC_);    \
@@ -2316,14 +2378,14 @@ struct FlowRepackArgs {
 // one 64-thread workgroup copies one piece from the per-tensor field streams into its place
 __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
     const FlowGeom g = p.kind == 4 ? p.cls : (p.kind == 0 ? p.g4[0] : (p.kind == 1 ? p.g4[1] : (p.kind == 2 ? p.g4[2] : p.g4[3])));
-    const int per_wg = g.rpw * g.ppr;
+    const int per_wg = flow_wg_capacity(g);
     const int wg = blockIdx.x / per_wg, j = blockIdx.x % per_wg;
-    if (j >= flow_n_local(g, wg) * g.ppr) return;
-    const int np = flow_n_local(g, wg) * g.ppr, base = np / FLOW_NW, rem = np % FLOW_NW;
+    if (j >= flow_wg_pieces(g, wg)) return;
+    const int np = flow_wg_pieces(g, wg), base = np / FLOW_NW, rem = np % FLOW_NW;
     const int wave = j < rem * (base + 1) ? j / (base + 1) : rem + (j - rem * (base + 1)) / base;
     const int idx = j - flow_wave_start(g, wg, wave);
-    const int L = wg * g.rpw + j / g.ppr;
-    const int part = j % g.ppr;
+    const int L = wg * g.rpw + flow_piece_row(g, j);
+    const int half = flow_half(g), part = half ? j % half : j % g.ppr;
     int seg, row32;
     flow_row_src(p.kind == 4 ? 1 : p.kind, L, p.dim, p.kv_dim, p.hs, p.neox, seg, row32, true);
     const int64_t row = row32;
@@ -2340,29 +2402,43 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
         }
         const int64_t e = p.typed.piece_base[wg * FLOW_NW + wave] + (int64_t)p.layer * per_layer + before + idx;
         uint4 *dst = (uint4 *)(p.stream + p.wave_off[wg * FLOW_NW + wave] + p.typed.piece_off[e]);
-        const int64_t blk0 = row * t.nb + part * 8;
-        // super-blocks of the piece that the row has (fewer than 8 where the row is padded to whole pieces: the
-        // others are written as zeros, d = 0)
-        const int nbv = (int)min((int64_t)8, max((int64_t)0, t.nb - (int64_t)part * 8));
+        // super-block b of the piece: which tensor and which of its super-blocks (valid: the row has it; a row that is
+        // padded to whole pieces has fewer than 8 in its last piece, and the others are written as zeros, d = 0).
+        // Rows that end inside a piece: super-block 8 part + b of the pair's, the odd row's from t.nb on.
+        auto at = [&](int b_, const DevTensor *&tt, int64_t &bi) -> bool {
+            if (half) {
+                const int pb = 8 * part + b_, odd = pb >= (int)t.nb ? 1 : 0;
+                int sg, rw;
+                flow_row_src(p.kind, L + odd, p.dim, p.kv_dim, p.hs, p.neox, sg, rw, true);
+                tt = sg == 0 ? &p.w[0] : (sg == 1 ? &p.w[1] : &p.w[2]);
+                bi = (int64_t)rw * tt->nb + (pb - odd * (int)t.nb);
+                return true;
+            }
+            tt = &t;
+            bi = row * t.nb + part * 8 + b_;
+            return (int64_t)part * 8 + b_ < t.nb;
+        };
         const uint4 z4 = make_uint4(0u, 0u, 0u, 0u);
+        const DevTensor *tt;
+        int64_t bi;
         if (lane == 0) dst[8] = make_uint4((uint32_t)p.typed.piece_tag[e], 0u, 0u, 0u);
         if (t.type == L2H_TYPE_Q4_K) {
-            if (lane < 8) dst[lane] = lane < nbv ? flow_encode_hdr(t.hdr[blk0 + lane]) : z4;
-            dst[9 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
+            if (lane < 8) dst[lane] = at(lane, tt, bi) ? flow_encode_hdr(tt->hdr[bi]) : z4;
+            dst[9 + lane] = at(lane >> 3, tt, bi) ? ((const uint4 *)(tt->qs + bi * 128))[lane & 7] : z4;
         } else if (t.type == L2H_TYPE_Q5_K) {
-            if (lane < 8) dst[lane] = lane < nbv ? flow_encode_hdr(t.hdr[blk0 + lane]) : z4;
-            if (lane < 16) dst[9 + lane] = (lane >> 1) < nbv ? ((const uint4 *)(t.qh + blk0 * 32))[lane] : z4;
-            dst[25 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
+            if (lane < 8) dst[lane] = at(lane, tt, bi) ? flow_encode_hdr(tt->hdr[bi]) : z4;
+            if (lane < 16) dst[9 + lane] = at(lane >> 1, tt, bi) ? ((const uint4 *)(tt->qh + bi * 32))[lane & 1] : z4;
+            dst[25 + lane] = at(lane >> 3, tt, bi) ? ((const uint4 *)(tt->qs + bi * 128))[lane & 7] : z4;
         } else {  // q6_K
-            if (lane < 8) dst[lane] = lane < nbv ? ((const uint4 *)(t.sc6 + blk0 * 4))[lane] : z4;
+            if (lane < 8) dst[lane] = at(lane, tt, bi) ? ((const uint4 *)(tt->sc6 + bi * 4))[0] : z4;
             if (lane == 1) {
                 uint16_t dd[8];
-                for (int b = 0; b < 8; b++) dd[b] = b < nbv ? t.d6[blk0 + b] : (uint16_t)0;
+                for (int b_ = 0; b_ < 8; b_++) dd[b_] = at(b_, tt, bi) ? tt->d6[bi] : (uint16_t)0;
                 dst[9] = make_uint4(dd[0] | (uint32_t)dd[1] << 16, dd[2] | (uint32_t)dd[3] << 16, dd[4] | (uint32_t)dd[5] << 16,
                                     dd[6] | (uint32_t)dd[7] << 16);
             }
-            if (lane < 32) dst[10 + lane] = (lane >> 2) < nbv ? ((const uint4 *)(t.qh + blk0 * 64))[lane] : z4;
-            dst[42 + lane] = (lane >> 3) < nbv ? ((const uint4 *)(t.qs + blk0 * 128))[lane] : z4;
+            if (lane < 32) dst[10 + lane] = at(lane >> 2, tt, bi) ? ((const uint4 *)(tt->qh + bi * 64))[lane & 3] : z4;
+            dst[42 + lane] = at(lane >> 3, tt, bi) ? ((const uint4 *)(tt->qs + bi * 128))[lane & 7] : z4;
         }
         return;
     }
@@ -2407,7 +2483,7 @@ __global__ __launch_bounds__(64) void flow_repack_kernel(FlowRepackArgs p) {
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
-static FlowGeom make_geom(int64_t n_rows, int64_t K, int type, int grid) {
+static FlowGeom make_geom(int64_t n_rows, int64_t K, int type, int grid, bool halves = false) {
     FlowGeom g{};
     g.n_rows = (int)n_rows;
     g.K = (int)K;
@@ -2422,6 +2498,7 @@ static FlowGeom make_geom(int64_t n_rows, int64_t K, int type, int grid) {
         g.ppr = ppr;
     } else {
         g.ppr = (int)(K / 256) / (type == L2H_TYPE_Q6_K ? 16 : 8);
+        if (halves) g.ppr = 0;  // K = 256 * (8 i + 4): a piece and a half per row (or 2 1/2, ...), whole pieces per pair of rows
     }
     return g;
 }
@@ -2472,9 +2549,12 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     for (int l = 0; l * 7 + 6 < n_layer_types; l++)  // (w1 and w3 rows alternate within a workgroup's pieces)
         if (layer_types[l * 7 + 4] != layer_types[l * 7 + 6]) return no("w1 and w3 of a layer must have one type");
     if (cls_type != L2H_TYPE_Q4_K && cls_type != L2H_TYPE_Q6_K) return no("classifier must be q4_K or q6_K");
-    // rows of dim inputs may be padded with zero super-blocks to whole pieces if that adds a third at most (dim 3072
-    // -> 4096); such a model, and one with head size 96, runs as typed pieces
+    // rows of dim inputs may be padded with zero super-blocks to whole pieces if that adds a third at most (dim 3584
+    // -> 4096); such a model, and one with head size 96, runs as typed pieces.  Where half a piece is missing (dim 3072)
+    // the layer matrices are not padded: their rows go in pairs, a pair's middle piece shared by the two (the
+    // classifier's rows, which are not paired, stay padded).
     a.dim_pad = (a.dim + 2047) / 2048 * 2048;
+    const bool halves = a.dim % 2048 == 1024;
     if (a.dim % 256 != 0 || (int64_t)a.dim * 4 < (int64_t)a.dim_pad * 3 || a.hidden % 2048 != 0)
         return no("dim must be a multiple of 2048 (or of 256 and within a quarter below one), hidden_dim a multiple of 2048");
     if (a.dim_pad != a.dim) a.mixed = 1;
@@ -2492,16 +2572,17 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     const size_t run = (size_t)((((a.seq_len + G - 1) / G) + 63) & ~63);
     const size_t att = (size_t)a.hs * 8 + (size_t)std::max(FLOW_NW * a.hs, 1024) * 8 + run * 4 + (size_t)a.hs * 8 + 64 * 8;
     if (att > FLOW_ACT_BYTES) return no("sequence too long for the attention area");
-    a.qkv = make_geom(a.dim + 2 * a.kv_dim, a.dim_pad, L2H_TYPE_Q4_K, grid);
-    a.wo = make_geom(a.dim, a.dim_pad, L2H_TYPE_Q4_K, grid);
-    a.w13 = make_geom(2 * (int64_t)a.hidden, a.dim_pad, L2H_TYPE_Q4_K, grid);
+    a.qkv = make_geom(a.dim + 2 * a.kv_dim, halves ? a.dim : a.dim_pad, L2H_TYPE_Q4_K, grid, halves);
+    a.wo = make_geom(a.dim, halves ? a.dim : a.dim_pad, L2H_TYPE_Q4_K, grid, halves);
+    a.w13 = make_geom(2 * (int64_t)a.hidden, halves ? a.dim : a.dim_pad, L2H_TYPE_Q4_K, grid, halves);
     a.w2 = make_geom(a.dim, a.hidden, L2H_TYPE_Q4_K, grid);
     a.cls = make_geom(a.vocab, a.dim_pad, cls_type, grid);
     const FlowGeom *gs[5] = {&a.qkv, &a.wo, &a.w13, &a.w2, &a.cls};
     for (const FlowGeom *g : gs)
-        if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
+        if (g->rpw > FLOW_MAX_ROWS || flow_wg_capacity(*g) > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
             return no("too many rows per workgroup");  // (layer phases keep four partial sums per piece)
-    if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
+    if ((a.dim + 2 * a.kv_dim) % 2 != 0 || (halves && (a.dim % 2 != 0 || a.kv_dim % 2 != 0)))
+        return no("odd row count");
     if (a.wo.rpw != a.w2.rpw) return no("row split of wo and w2 differs");  // (a row of x has one owner)
     return true;
 }
@@ -2545,7 +2626,7 @@ void k_flow_typed_tables(const FlowArgs &a, const int *layer_types, int cls_type
                     const FlowGeom &g = g4[kind];
                     const int cnt = flow_wave_pieces(g, wg, w), start = flow_wave_start(g, wg, w);
                     for (int i = 0; i < cnt; i++) {
-                        const int L = wg * g.rpw + (start + i) / g.ppr;
+                        const int L = wg * g.rpw + flow_piece_row(g, start + i);
                         int seg, row;
                         flow_row_src(kind, L, a.dim, a.kv_dim, a.hs, a.neox, seg, row, true);
                         const int slot = kind == 0 ? seg : (kind == 1 ? 3 : (kind == 2 ? 4 : 5));
@@ -2590,7 +2671,7 @@ hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream
     p.mixed = a.mixed;
     p.typed = typed;
     const FlowGeom &g = kind == 4 ? a.cls : p.g4[kind];
-    hipLaunchKernelGGL(flow_repack_kernel, dim3((unsigned)(grid * g.rpw * g.ppr)), dim3(64), 0, s, p);
+    hipLaunchKernelGGL(flow_repack_kernel, dim3((unsigned)(grid * flow_wg_capacity(g))), dim3(64), 0, s, p);
     return hipGetLastError();
 }
 
@@ -2605,17 +2686,21 @@ hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a) {
 // else.  The kernel has no grid-wide barrier and every wait in it is bounded, so residency is what makes it
 // fast, not what makes it correct: workgroups that had to wait for a CU would let the others run into their
 // wait limit, and the launch would end with the error that l2h_model_set_wait_limit describes.
-static const void *flow_kernel_fn(int cls_type, bool mixed) {
+// form: 0 q4_K pieces, 1 typed pieces, 2 typed pieces and rows that end inside a piece
+static const void *flow_kernel_fn(int cls_type, int form) {
     if (cls_type == L2H_TYPE_F32) return (const void *)flow_f32_kernel;
-    if (mixed)
+    if (form == 2)
+        return cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K, true, true>
+                                         : (const void *)flow_token_kernel<L2H_TYPE_Q4_K, true, true>;
+    if (form == 1)
         return cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K, true>
                                          : (const void *)flow_token_kernel<L2H_TYPE_Q4_K, true>;
     return cls_type == L2H_TYPE_Q6_K ? (const void *)flow_token_kernel<L2H_TYPE_Q6_K, false>
                                      : (const void *)flow_token_kernel<L2H_TYPE_Q4_K, false>;
 }
 
-bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed) {
-    const void *fn = flow_kernel_fn(cls_type, mixed);
+bool k_flow_fits(int cls_type, int grid, int n_cu, int form) {
+    const void *fn = flow_kernel_fn(cls_type, form);
     int per_cu = 0;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, fn, 1024, 0) != hipSuccess) return false;
     return per_cu >= 1 && (int64_t)per_cu * n_cu >= grid;
@@ -2623,8 +2708,8 @@ bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed) {
 
 // A plain launch: a cooperative one costs about 20 µs more per token on this stack, and all it would add is the
 // residency check that k_flow_fits makes once.
-hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int n_tok, int cls_type, int grid, bool mixed) {
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int n_tok, int cls_type, int grid, int form) {
     void *args[] = {&gen0, &n_tok};
-    const void *fn = flow_kernel_fn(cls_type, mixed);
+    const void *fn = flow_kernel_fn(cls_type, form);
     return hipLaunchKernel(fn, dim3(grid), dim3(1024), args, 0, s);
 }

@@ -133,7 +133,8 @@ struct MegaArgs {
 struct FlowGeom {
     int n_rows;  // logical rows
     int rpw;     // rows per workgroup (even)
-    int ppr;     // pieces per row
+    int ppr;     // pieces per row; 0: rows of K = 1024 (2 i + 1) inputs end in the middle of a piece and go in pairs of
+                 // K / 1024 pieces, the pair's middle piece holding the end of the even row and the start of the odd one
     int K;       // input length
 };
 struct FlowArgs {
@@ -198,8 +199,10 @@ hipError_t k_flow_repack(hipStream_t s, const FlowArgs &a, unsigned char *stream
                          int layer, const DevTensor *w, int nw, int grid, int cls_type, const FlowTypedDev &typed);
 hipError_t k_flow_bind(hipStream_t s, const FlowArgs &a);
 // one launch runs n_tok steps of the token loop; the epochs of the launch start at gen0 and take 5 * n_layers + 2 per step
-hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int n_tok, int cls_type, int grid, bool mixed);
-bool k_flow_fits(int cls_type, int grid, int n_cu, bool mixed);
+// form: 0 q4_K pieces, 1 typed pieces, 2 typed pieces and rows that end inside a piece (flow_form)
+hipError_t k_flow_launch(hipStream_t s, unsigned int gen0, int n_tok, int cls_type, int grid, int form);
+bool k_flow_fits(int cls_type, int grid, int n_cu, int form);
+inline int flow_form(const FlowArgs &a) { return a.mixed ? (a.qkv.ppr == 0 ? 2 : 1) : 0; }
 
 // ---- launchers (kernel files) ----------------------------------------------------------------
 // Each returns hipGetLastError() of its launch.

@@ -88,6 +88,7 @@ class DeviceModel:
             self.ctx.check(_lib.lib().l2h_model_finalize(self.handle))
             self.path = _lib.lib().l2h_model_path(self.handle)  # 1 = kernel per phase, 2 = persistent kernel, 3 = streaming
             self.path_reason = _lib.lib().l2h_model_path_reason(self.handle).decode()  # why not 3 ("" if 3)
+            self.steps_per_launch = _lib.lib().l2h_model_steps_per_launch(self.handle)  # token-loop steps per kernel launch
         except Exception:
             self.close()
             raise

@@ -49,8 +49,25 @@ static void check_shape(int dim, int hidden, int n_layers, int n_heads, int n_kv
                 EXPECT(flow_wave_start(g4[k], wg, w) == pieces);
                 pieces += flow_wave_pieces(g4[k], wg, w);
             }
-            EXPECT(pieces == n * g4[k].ppr);
+            EXPECT(pieces == flow_wg_pieces(g4[k], wg));
+            EXPECT(flow_half(g4[k]) ? pieces * 2 == n * flow_half(g4[k]) : pieces == n * g4[k].ppr);
             EXPECT(n <= FLOW_MAX_ROWS && pieces <= FLOW_MAX_PIECES / 4);
+            if (flow_half(g4[k])) {
+                // rows that end inside a piece: the pieces of a pair of rows hold every super-block of both rows once
+                const int nb = 4 * flow_half(g4[k]);
+                EXPECT(nb * 256 == dim && n % 2 == 0 && flow_half(g4[k]) % 2 == 1);
+                std::vector<char> seen((size_t)n * nb, 0);
+                for (int j = 0; j < pieces; j++) {
+                    const int lr = flow_piece_row(g4[k], j), part = j % flow_half(g4[k]);
+                    for (int b = 0; b < 8; b++) {
+                        const int pb = 8 * part + b, odd = pb >= nb, blk = pb - odd * nb;
+                        EXPECT(lr + odd < n && blk < nb);
+                        EXPECT(!seen[(size_t)(lr + odd) * nb + blk]);
+                        seen[(size_t)(lr + odd) * nb + blk] = 1;
+                    }
+                }
+                for (char c : seen) EXPECT(c);
+            }
         }
         EXPECT(rows == g4[k].n_rows);
     }
@@ -113,11 +130,12 @@ int main() {
     check_shape(4096, 14336, 32, 32, 8, 128256, 512, q4, 14, 0, true);    // the headline model
     check_shape(4096, 14336, 32, 32, 8, 128256, 4096, q5m, 14, 0, true);  // q5_K_M mix: typed pieces
     check_shape(4096, 14336, 4, 32, 8, 128256, 512, mix, 12, 0, true);    // q4_K classifier behind typed pieces
-    check_shape(3072, 8192, 32, 32, 32, 32064, 4096, q4, 12, 0, true);    // Phi-3: padded rows, head size 96
+    check_shape(3072, 8192, 32, 32, 32, 32064, 4096, q4, 12, 0, true);    // Phi-3: a piece and a half per row, head size 96
     check_shape(3072, 8192, 2, 32, 32, 32064, 4096, q4, 12, 1, true);     // the same with an fp16 cache
     check_shape(2048, 4096, 3, 16, 4, 1000, 160, q4, 14, 0, false);       // q6_K classifier needs 4096
     check_shape(2048, 4096, 3, 16, 4, 1000, 160, q4, 12, 0, true);
-    check_shape(1536, 2048, 2, 16, 16, 999, 96, q4, 12, 0, true);         // a quarter below 2048
+    check_shape(1536, 2048, 2, 16, 16, 999, 96, q4, 12, 0, true);         // a quarter below 2048: padded rows
+    check_shape(3072, 8192, 2, 32, 8, 32064, 512, mix, 12, 0, true);      // halves with typed pieces and grouped heads
     check_shape(1024, 2048, 2, 16, 16, 999, 96, q4, 12, 0, false);        // half below: refused
     check_shape(512, 1376, 8, 8, 8, 32000, 1024, f32, 0, 0, true);        // llama2.c shape
     check_shape(4096, 14336, 2, 32, 8, 32000, 512, bad, 14, 0, false);    // w1 and w3 of different types

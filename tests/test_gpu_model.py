@@ -150,10 +150,16 @@ FLOW_CASES = {
     "q4ks_headline_widths": ("PLAN_Q4_K_S", dict(dim=4096, hidden_dim=14336, n_layers=2, n_heads=32, n_kv_heads=8,
                                                  vocab_size=32000, seq_len=192, rope_freq_base=500000.0,
                                                  rope_is_neox=False)),
-    # the Phi-3 shape: dim 3072 is 1.5 pieces per row (rows padded with zero super-blocks to 4096 in the streams), head
-    # size 96 is not a power of two, neox RoPE, no GQA
+    # the Phi-3 shape: dim 3072 is 1.5 pieces per row (a pair of rows shares its middle piece in the streams; the
+    # classifier's rows are padded with zero super-blocks to 4096), head size 96 is not a power of two, neox RoPE, no GQA
     "phi3_widths": ("PLAN_Q4_K", dict(dim=3072, hidden_dim=2048, n_layers=2, n_heads=32, n_kv_heads=32, vocab_size=512,
                                       seq_len=128, rope_freq_base=10000.0, rope_is_neox=True)),
+    # the same row length with every type in every role and grouped heads: a pair's two rows come from different tensors
+    # (w1 | w3) and the shared piece may be of any type
+    "halves_all_types": (dict(emb=12, output=12, wq=[14, 12, 13], wk=[13, 14, 12], wv=[12, 13, 14], wo=[14, 13, 12],
+                              w1=[13, 12, 14], w3=[13, 12, 14], w2=[13, 14, 12]),
+                         dict(dim=3072, hidden_dim=2048, n_layers=3, n_heads=32, n_kv_heads=8, vocab_size=600, seq_len=96,
+                              rope_freq_base=10000.0, rope_is_neox=False)),
     # fp32 matrices (llama2.c checkpoints): no streams, rows read where the tensors lie; hidden_dim not a multiple of 256,
     # classifier shared with the embedding
     "f32_rows": ("PLAN_F32", dict(dim=256, hidden_dim=344, n_layers=3, n_heads=8, n_kv_heads=4, vocab_size=500, seq_len=96,
