@@ -156,7 +156,10 @@ def main():
         prefill = {"positions": n_prompt, "ms": round(pf_dt * 1e3, 2), "tok_s": round(n_prompt / pf_dt, 1),
                    "TFLOP/s": round((gemm_flop + attn_flop) / pf_dt / 1e12, 1), "gemm_TFLOP": round(gemm_flop / 1e12, 2),
                    "attention_TFLOP": round(attn_flop / 1e12, 2), "peak_bf16_TFLOP/s": 2500.0,
-                   "frac_of_mfma_peak": round((gemm_flop + attn_flop) / pf_dt / 2.5e15, 4)}
+                   "frac_of_mfma_peak": round((gemm_flop + attn_flop) / pf_dt / 2.5e15, 4),
+                   # q|k|v, wo and w2 through hipBLASLt (the default where it can be opened; L2H_PF_LIBRARY=0: own kernels);
+                   # w1|w3 + SwiGLU and the attention are this library's kernels either way
+                   "plain_products": "hipBLASLt" if dev.prefill_library else "own kernels"}
         log("prompt pass:", json.dumps(prefill))
         prompt = np.array([nxt], np.int32)
         n_pre = n_prompt  # the cache now holds the whole prompt; decoding starts at the next position

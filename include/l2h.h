@@ -135,8 +135,19 @@ int l2h_model_set_wait_limit(l2h_model *m, unsigned int spins);
 /* l2h_prefill keeps a bf16 copy of the layer matrices (2 bytes per weight, made at its first call
  * when that fits beside 2 GiB of free device memory) and multiplies from it; on = 0 makes it
  * expand the quantized blocks inside the product kernel on every call instead (no extra memory,
- * slower).  The results are the same bit for bit.  Default 1.  No counterpart in the reference. */
+ * slower).  With this library's own product kernels (l2h_model_set_prefill_library 0) the results are
+ * the same bit for bit.  Default 1.  No counterpart in the reference. */
 int l2h_model_set_prefill_copy(l2h_model *m, int on);
+/* The products of l2h_prefill that have no arithmetic behind them (q | k | v; wo and w2, whose residual add is the
+ * product's beta = 1) go through hipBLASLt, ROCm's GEMM library, when the bf16 copy above exists and the library can be
+ * opened at run time (on = 1, the default; the environment variable L2H_PF_LIBRARY=0 has the effect of on = 0); w1 | w3
+ * with SwiGLU, the attention and everything else stay with this library's kernels.  on = 0: this library's product
+ * kernels throughout.  Same operands (bf16) and fp32 sums either way; the order of the sums differs, so results agree
+ * to rounding, not bit for bit.  Takes effect at the next l2h_prefill (the copy's layout is rewritten, a few ms).
+ * l2h_model_prefill_library: 1 if the last l2h_prefill ran those products through hipBLASLt.  No counterpart in the
+ * reference (matmul! on a matrix of activations is BLAS there too: src/matmul.jl:3-11 for dense matrices). */
+int l2h_model_set_prefill_library(l2h_model *m, int on);
+int l2h_model_prefill_library(l2h_model *m);
 /* RunState(config) (src/inference.jl:88-100): checks every tensor is present, allocates
  * activations and the zeroed KV cache, records the per-token launch sequence. */
 int l2h_model_finalize(l2h_model *m);

@@ -51,6 +51,8 @@ SIGNATURES = {
     "l2h_model_set_path": (_I, [_P, _I]),
     "l2h_model_set_wait_limit": (_I, [_P, C.c_uint]),
     "l2h_model_set_prefill_copy": (_I, [_P, _I]),
+    "l2h_model_set_prefill_library": (_I, [_P, _I]),
+    "l2h_model_prefill_library": (_I, [_P]),
     "l2h_model_path": (_I, [_P]),
     "l2h_model_steps_per_launch": (_I, [_P]),
     "l2h_model_finalize": (_I, [_P]),

@@ -20,7 +20,7 @@ OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libl2hip.so")
 LIB_TIMELINE = os.path.join(HERE, "libl2hip_tl.so")
 
-SOURCES = ["api.cpp", "synth.cpp", "k_misc.hip", "k_matvec.hip", "k_attn.hip", "k_mega.hip", "k_prefill.hip", "k_flow.hip"]
+SOURCES = ["api.cpp", "synth.cpp", "pf_lt.cpp", "k_misc.hip", "k_matvec.hip", "k_attn.hip", "k_mega.hip", "k_prefill.hip", "k_flow.hip"]
 
 COMMON = [
     "-O3", "-fPIC", "-std=c++17", "-ffp-contract=off", "-Wall", "-Wno-unused-function",
@@ -65,7 +65,8 @@ def build(force=True, verbose=True, timeline=False):
             if verbose and text.strip():
                 print("[%s]\n%s" % (src, text))
             objs.append(obj)
-    cmd = [_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", lib] + objs
+    # (hipBLASLt is opened at run time by pf_lt.cpp: -ldl, no link-time dependency on it)
+    cmd = [_hipcc(), "-shared", "-fPIC", "--offload-arch=gfx950", "-o", lib] + objs + ["-ldl"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stdout + r.stderr)

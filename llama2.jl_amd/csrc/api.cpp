@@ -258,6 +258,12 @@ struct l2h_model {
     int pf_copy_mode = 1;          // 0 never, 1 when it fits
     bool pf_copy_tried = false;
     uint16_t *pf_wbf = nullptr;
+    // the plain products of the prompt pass (q | k | v, wo, w2) through hipBLASLt: asked for (default) / opened / the
+    // layout the copy's three matrices have now (plain rows for the library, tiles for the own kernels)
+    int pf_library_mode = 1;
+    PfLt *pf_lt = nullptr;
+    bool pf_lt_tried = false, pf_plain = false;
+    std::string pf_lt_why, pf_lt_err;
     int64_t pf_wbf_layer = 0, pf_off_wo = 0, pf_off_w13 = 0, pf_off_w2 = 0;  // elements
     std::vector<void *> allocs;
     std::vector<void *> uc_allocs;  // blocks of the uncached pool (uncached_alloc), handed back with the model
@@ -314,6 +320,10 @@ static void model_free_state(l2h_model *m) {
     m->pf_cap = 0;
     m->pf_wbf = nullptr;
     m->pf_copy_tried = false;
+    pf_lt_close(m->pf_lt);
+    m->pf_lt = nullptr;
+    m->pf_lt_tried = false;
+    m->pf_plain = false;
     m->sample_p = nullptr;
     m->sample_out = nullptr;
     m->finalized = false;
@@ -395,6 +405,15 @@ extern "C" int l2h_model_set_prefill_copy(l2h_model *m, int on) {
     m->pf_copy_mode = on;
     return L2H_OK;
 }
+
+extern "C" int l2h_model_set_prefill_library(l2h_model *m, int on) {
+    if (!m) return L2H_EINVAL;
+    if (on != 0 && on != 1) return set_err(m->ctx, L2H_EINVAL, "on must be 0 or 1");
+    m->pf_library_mode = on;
+    return L2H_OK;
+}
+
+extern "C" int l2h_model_prefill_library(l2h_model *m) { return (m && m->pf_wbf && m->pf_copy_mode && m->pf_plain) ? 1 : 0; }
 
 extern "C" int l2h_model_set_kv_type(l2h_model *m, int kv_type) {
     if (!m) return L2H_EINVAL;
@@ -1235,8 +1254,42 @@ static int prefill_buffers(l2h_model *m, int cap) {
 // that later prompt passes run plain bf16 products.  2 bytes per weight stay resident; when that does
 // not fit beside 2 GiB of head room, or dim or hidden_dim is not a multiple of 64, the fused kernels
 // stay in use.
+// (re)writes the copy: w1 | w3 always as the product kernel's tiles, the three plain products' matrices as tiles or as
+// plain rows
+static int prefill_expand(l2h_model *m, bool plain) {
+    const l2h_config &c = m->c;
+    const int64_t dim = c.dim, kvd = m->kv_dim, hid = c.hidden_dim;
+    hipStream_t s = m->ctx->stream;
+    const int pl = plain ? 1 : 0;
+    for (int l = 0; l < c.n_layers; l++) {
+        uint16_t *base = m->pf_wbf + (int64_t)l * m->pf_wbf_layer;
+        const DevTensor w[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
+        const int64_t row0[3] = {0, dim, dim + kvd};
+        for (int i = 0; i < 3; i++) HIPCHK(m->ctx, k_pf_expand(s, w + i, 1, 0, dim, base, row0[i], i == 2, pl));
+        const DevTensor wo = m->L(l, L2H_WO), w2 = m->L(l, L2H_W2);
+        const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
+        HIPCHK(m->ctx, k_pf_expand(s, &wo, 1, 0, dim, base + m->pf_off_wo, 0, 1, pl));
+        HIPCHK(m->ctx, k_pf_expand(s, w13, 2, 1, dim, base + m->pf_off_w13, 0, 1, 0));
+        HIPCHK(m->ctx, k_pf_expand(s, &w2, 1, 0, hid, base + m->pf_off_w2, 0, 1, pl));
+    }
+    HIPCHK(m->ctx, hipStreamSynchronize(s));
+    m->pf_plain = plain;
+    return L2H_OK;
+}
+
 static int prefill_weights(l2h_model *m) {
-    if (m->pf_copy_tried) return L2H_OK;
+    // the library for the plain products: opened once; L2H_PF_LIBRARY=0 keeps every product in this library's kernels
+    const char *env = getenv("L2H_PF_LIBRARY");
+    const bool want = m->pf_library_mode != 0 && !(env && atoi(env) == 0);
+    if (want && !m->pf_lt_tried) {
+        m->pf_lt_tried = true;
+        m->pf_lt = pf_lt_open(&m->pf_lt_why);
+    }
+    const bool plain = want && m->pf_lt != nullptr;
+    if (m->pf_copy_tried) {
+        if (m->pf_wbf && plain != m->pf_plain) return prefill_expand(m, plain);
+        return L2H_OK;
+    }
     m->pf_copy_tried = true;
     const l2h_config &c = m->c;
     const int64_t dim = c.dim, kvd = m->kv_dim, hid = c.hidden_dim;
@@ -1253,20 +1306,11 @@ static int prefill_weights(l2h_model *m) {
     uint16_t *buf = nullptr;
     int rc;
     if ((rc = dalloc(m, &buf, (int64_t)(bytes / 2), false))) return rc;
-    hipStream_t s = m->ctx->stream;
-    for (int l = 0; l < c.n_layers; l++) {
-        uint16_t *base = buf + (int64_t)l * m->pf_wbf_layer;
-        const DevTensor w[3] = {m->L(l, L2H_WQ), m->L(l, L2H_WK), m->L(l, L2H_WV)};
-        const int64_t row0[3] = {0, dim, dim + kvd};
-        for (int i = 0; i < 3; i++) HIPCHK(m->ctx, k_pf_expand(s, w + i, 1, 0, dim, base, row0[i], i == 2));
-        const DevTensor wo = m->L(l, L2H_WO), w2 = m->L(l, L2H_W2);
-        const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
-        HIPCHK(m->ctx, k_pf_expand(s, &wo, 1, 0, dim, base + m->pf_off_wo, 0, 1));
-        HIPCHK(m->ctx, k_pf_expand(s, w13, 2, 1, dim, base + m->pf_off_w13, 0, 1));
-        HIPCHK(m->ctx, k_pf_expand(s, &w2, 1, 0, hid, base + m->pf_off_w2, 0, 1));
-    }
-    HIPCHK(m->ctx, hipStreamSynchronize(s));
     m->pf_wbf = buf;
+    if ((rc = prefill_expand(m, plain))) {
+        m->pf_wbf = nullptr;
+        return rc;
+    }
     return L2H_OK;
 }
 
@@ -1287,7 +1331,10 @@ static hipError_t prefill_chunk(l2h_model *m, int M, int pos0) {
         float *vc = m->vc + (int64_t)l * m->cache_layer_elems;
         CK(k_pf_rmsnorm(s, m->pf_x, m->L(l, L2H_RMS_ATT).f32, m->pf_xn, M, dim));
         const uint16_t *wb = (m->pf_wbf && m->pf_copy_mode) ? m->pf_wbf + (int64_t)l * m->pf_wbf_layer : nullptr;
-        if (wb) {
+        const bool lib = wb && m->pf_plain;  // (plain rows in the copy: the plain products go through hipBLASLt)
+        if (lib) {
+            CK(pf_lt_gemm(m->pf_lt, s, wb, m->pf_xn, m->pf_raw, M, dim + 2 * kvd, dim, dim + 2 * kvd, false, &m->pf_lt_err));
+        } else if (wb) {
             CK(k_pf_gemm(s, nullptr, 0, 0, wb, dim + 2 * kvd, m->pf_xn, M, dim, PF_STORE, m->pf_raw, dim + 2 * kvd, 0,
                          nullptr, 0));
         } else {
@@ -1307,15 +1354,21 @@ static hipError_t prefill_chunk(l2h_model *m, int M, int pos0) {
         CK(k_pf_kv_tiles(s, kc, vc, m->pf_kvt, (pos0 + M + 31) / 32, m->pf_kvt_tiles, m->hs, c.n_kv_heads, c.seq_len));
         CK(k_pf_attention(s, m->pf_q, m->pf_att, m->pf_kvt, m->pf_kvt_tiles, M, pos0, m->hs, c.n_heads, c.n_kv_heads, dim));
         const DevTensor wo = m->L(l, L2H_WO);
-        CK(k_pf_gemm(s, &wo, 1, 0, wb ? wb + m->pf_off_wo : nullptr, dim, m->pf_att, M, dim, PF_RESID, m->pf_x, dim, 0,
-                     nullptr, 0));
+        if (lib)
+            CK(pf_lt_gemm(m->pf_lt, s, wb + m->pf_off_wo, m->pf_att, m->pf_x, M, dim, dim, dim, true, &m->pf_lt_err));
+        else
+            CK(k_pf_gemm(s, &wo, 1, 0, wb ? wb + m->pf_off_wo : nullptr, dim, m->pf_att, M, dim, PF_RESID, m->pf_x, dim, 0,
+                         nullptr, 0));
         CK(k_pf_rmsnorm(s, m->pf_x, m->L(l, L2H_RMS_FFN).f32, m->pf_xn, M, dim));
         const DevTensor w13[2] = {m->L(l, L2H_W1), m->L(l, L2H_W3)};
         CK(k_pf_gemm(s, w13, 2, 1, wb ? wb + m->pf_off_w13 : nullptr, 2 * (int64_t)c.hidden_dim, m->pf_xn, M, dim,
                      PF_SWIGLU, nullptr, 0, 0, m->pf_hb, c.hidden_dim));
         const DevTensor w2 = m->L(l, L2H_W2);
-        CK(k_pf_gemm(s, &w2, 1, 0, wb ? wb + m->pf_off_w2 : nullptr, dim, m->pf_hb, M, c.hidden_dim, PF_RESID, m->pf_x,
-                     dim, 0, nullptr, 0));
+        if (lib)
+            CK(pf_lt_gemm(m->pf_lt, s, wb + m->pf_off_w2, m->pf_hb, m->pf_x, M, dim, c.hidden_dim, dim, true, &m->pf_lt_err));
+        else
+            CK(k_pf_gemm(s, &w2, 1, 0, wb ? wb + m->pf_off_w2 : nullptr, dim, m->pf_hb, M, c.hidden_dim, PF_RESID, m->pf_x,
+                         dim, 0, nullptr, 0));
     }
 #undef CK
     return hipSuccess;
@@ -1349,7 +1402,9 @@ extern "C" int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0,
         M = std::min(m->pf_cap, n - c0);
         HIPCHK(ctx, hipMemcpyAsync(m->pf_tok, tokens + c0, (size_t)M * 4, hipMemcpyHostToDevice, ctx->stream));
         hipError_t e = prefill_chunk(m, M, pos0 + c0);
-        if (e != hipSuccess) return set_err(ctx, L2H_EHIP, "prompt pass launch failed: %s", hipGetErrorString(e));
+        if (e != hipSuccess)
+            return set_err(ctx, L2H_EHIP, "prompt pass launch failed: %s%s%s", hipGetErrorString(e),
+                           m->pf_lt_err.empty() ? "" : "; ", m->pf_lt_err.c_str());
     }
     // last position: its hidden state becomes the decode state; classifier and argmax as in a decode step
     HIPCHK(ctx, hipMemcpyAsync(m->x, m->pf_x + (int64_t)(M - 1) * m->c.dim, (size_t)m->c.dim * 4,

@@ -326,8 +326,10 @@ __device__ __forceinline__ void pf_row_ptr(const PfGemmArgs &a, int64_t L, PfRow
 // rows 256 nt.. x inputs 64 kt.. at ((nt K/64) + kt) * 16384 elements, and inside a tile the image the
 // product kernel keeps in LDS: the 16-byte chunk c of row r at chunk index 8 r + (c ^ pf_swz(r)).  Logical
 // row L goes to row dst_row0 + L; rows from n_rows up to rows_end (padding of the last tile) are zero.
+// plain: row R is K values in a row at dst + R K instead (the layout a library product takes).
 template <int TYPE>
-__global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *dst, int64_t dst_row0, int64_t rows_end) {
+__global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *dst, int64_t dst_row0, int64_t rows_end,
+                                                        int plain) {
     const int64_t groups = a.K >> 5, nk = a.K >> 6;
     const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (idx >= rows_end * groups) return;
@@ -340,6 +342,12 @@ __global__ __launch_bounds__(256) void pf_expand_kernel(PfGemmArgs a, uint16_t *
     uint4 wv[4];
     pf_convert<TYPE>(raw, rp, lr.row, k0, a.K, wv);
     const int64_t R = dst_row0 + L, nt = R >> 8, kt = g >> 1;
+    if (plain) {
+        uint4 *row = (uint4 *)(dst + R * a.K + k0);
+#pragma unroll
+        for (int cc = 0; cc < 4; cc++) row[cc] = wv[cc];
+        return;
+    }
     const int r = (int)(R & 255);
     uint4 *tile = (uint4 *)(dst + (nt * nk + kt) * 16384);
 #pragma unroll
@@ -1102,7 +1110,7 @@ hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave
 // bf16 into the tiled matrix dst (see pf_expand_kernel) from row dst_row0 on; with pad the rows up to the
 // next multiple of 256 are zeroed.  K a multiple of 64.
 hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interleave, int64_t K, uint16_t *dst,
-                       int64_t dst_row0, int pad) {
+                       int64_t dst_row0, int pad, int plain) {
     PfGemmArgs a{};
     const hipError_t e = pf_weight_args(a, w, nseg, interleave, K);
     if (e != hipSuccess) return e;
@@ -1111,7 +1119,7 @@ hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interlea
     if (pad) rows_end = (dst_row0 + a.n_rows + 255) / 256 * 256 - dst_row0;
     const int64_t n = rows_end * (K >> 5);
     const dim3 grid((unsigned)((n + 255) / 256));
-#define GO(T) hipLaunchKernelGGL((pf_expand_kernel<T>), grid, dim3(256), 0, s, a, dst, dst_row0, rows_end)
+#define GO(T) hipLaunchKernelGGL((pf_expand_kernel<T>), grid, dim3(256), 0, s, a, dst, dst_row0, rows_end, plain)
     switch (w[0].type) {
     case L2H_TYPE_Q4_K: GO(L2H_TYPE_Q4_K); break;
     case L2H_TYPE_Q5_K: GO(L2H_TYPE_Q5_K); break;

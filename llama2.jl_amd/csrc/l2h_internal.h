@@ -254,8 +254,16 @@ hipError_t k_pf_rope_scatter(hipStream_t s, const float *raw, const float *cs, u
 hipError_t k_pf_gemm(hipStream_t s, const DevTensor *w, int nseg, int interleave, const uint16_t *wbf, int64_t n_rows_bf,
                      const uint16_t *act, int M, int64_t K, int epi, float *out, int64_t ldo, int64_t out_col0,
                      uint16_t *out_bf, int64_t ldb);
+// plain: rows of K bf16 values one after the other (what pf_lt_gemm multiplies from) instead of the product kernels' tiles
 hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interleave, int64_t K, uint16_t *dst,
-                       int64_t dst_row0, int pad);
+                       int64_t dst_row0, int pad, int plain);
+// hipBLASLt for the plain products of the prompt pass (pf_lt.cpp): D[M][0..N) (fp32, row stride ldd) = X[M][K] W[N][K]^T
+// (+ D if accumulate), bf16 operands, fp32 sums.  pf_lt_open returns nullptr, and says why, where the library cannot be used.
+struct PfLt;
+PfLt *pf_lt_open(std::string *why);
+void pf_lt_close(PfLt *lt);
+hipError_t pf_lt_gemm(PfLt *lt, hipStream_t s, const uint16_t *W, const uint16_t *X, float *D, int M, int64_t N, int64_t K,
+                      int64_t ldd, bool accumulate, std::string *err);
 bool k_pf_attention_supported(int hs);
 int64_t k_pf_kv_tile_bytes(int hs);
 hipError_t k_pf_kv_tiles(hipStream_t s, const float *kc, const float *vc, unsigned char *tiles, int n_tiles,

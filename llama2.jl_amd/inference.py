@@ -135,6 +135,15 @@ class DeviceModel:
         """Whether prefill multiplies from a resident bf16 copy of the weights (l2h_model_set_prefill_copy)."""
         self.ctx.check(_lib.lib().l2h_model_set_prefill_copy(self.handle, 1 if on else 0))
 
+    def set_prefill_library(self, on):
+        """Whether prefill runs its plain products (q|k|v, wo, w2) through hipBLASLt (l2h_model_set_prefill_library)."""
+        self.ctx.check(_lib.lib().l2h_model_set_prefill_library(self.handle, 1 if on else 0))
+
+    @property
+    def prefill_library(self):
+        """True if the last prefill ran those products through hipBLASLt (l2h_model_prefill_library)."""
+        return bool(_lib.lib().l2h_model_prefill_library(self.handle))
+
     def forward(self, token, pos, want_logits=True):
         """transformer!(token, pos, ...) (src/inference.jl:222-315): returns (logits, argmax)."""
         logits = np.empty(self.config.vocab_size, np.float32) if want_logits else None

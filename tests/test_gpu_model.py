@@ -519,6 +519,7 @@ def test_full_size_model_launch_paths_agree(pkg):
             # 2048 positions: the shapes at which the product kernels split a matrix over two tile sizes
             long_prompt = synth.seeded_prompt(8, 2048, kw["vocab_size"])
             pf = []
+            dev.set_prefill_library(False)  # (this library's product kernels: the copy changes nothing, bit for bit)
             for on in (True, False):
                 dev.set_prefill_copy(on)
                 dev.reset()
@@ -528,6 +529,17 @@ def test_full_size_model_launch_paths_agree(pkg):
             assert pf[0][1] == pf[1][1]
             assert np.array_equal(pf[0][0], pf[1][0])
             assert np.array_equal(pf[0][2], pf[1][2]) and np.array_equal(pf[0][3], pf[1][3])
+            # the plain products through hipBLASLt (the default): the same sums in another order
+            dev.set_prefill_library(True)
+            dev.set_prefill_copy(True)
+            dev.reset()
+            pl, nxt = dev.prefill(long_prompt, 0)
+            assert dev.prefill_library
+            k, v = dev.kv_read(31, 0, 2048)
+            d_l, d_k, d_v = _rel(pl, pf[0][0]), _rel(k, pf[0][2]), _rel(v, pf[0][3])
+            print("\n[full size] 2048-position prompt pass, hipBLASLt products against own products: logits rel diff %.3g, "
+                  "layer-31 K %.3g, V %.3g; same next token: %s" % (d_l, d_k, d_v, nxt == pf[0][1]))
+            assert max(d_l, d_k, d_v) <= 2e-2
             # the prompt pass against the state the token loop leaves (src/inference.jl:349-358: the reference feeds a
             # prompt token by token): the same 2048 tokens decoded one after the other, last logits and the last
             # layer's cache rows.  bf16 products of float activations against q8_K integer products: two roundings of
