@@ -160,6 +160,26 @@ def main():
                    # q|k|v, wo and w2 through hipBLASLt (the default where it can be opened; L2H_PF_LIBRARY=0: own kernels);
                    # w1|w3 + SwiGLU and the attention are this library's kernels either way
                    "plain_products": "hipBLASLt" if dev.prefill_library else "own kernels"}
+        # the other forms of the same pass, one call each after a warm-up call: this library's product kernels for every
+        # product, and the quantized blocks expanded inside the product kernel (no bf16 copy read)
+        def other_form(library, copy):
+            dev.set_prefill_library(library)
+            dev.set_prefill_copy(copy)
+            ts = []
+            for _ in range(2):
+                dev.reset()
+                ctx.sync()
+                t0 = time.perf_counter()
+                dev.prefill(prompt, 0, want_logits=False)
+                ts.append(time.perf_counter() - t0)
+            return round(min(ts) * 1e3, 2)
+        was_library = dev.prefill_library
+        prefill["own_product_kernels_ms"] = other_form(False, True) if was_library else prefill["ms"]
+        prefill["dequantized_in_the_product_kernel_ms"] = other_form(False, False)
+        dev.set_prefill_library(True)
+        dev.set_prefill_copy(True)
+        dev.reset()
+        _, nxt = dev.prefill(prompt, 0, want_logits=False)  # (the cache the decode steps continue from: the default form's)
         log("prompt pass:", json.dumps(prefill))
         prompt = np.array([nxt], np.int32)
         n_pre = n_prompt  # the cache now holds the whole prompt; decoding starts at the next position
