@@ -327,12 +327,20 @@ def test_several_steps_per_launch(pkg, monkeypatch, case, steps):
         lm._device = None
         dev = lm.device(path=3 if env is not None else 1)
         assert dev.path == (3 if env is not None else 1)
+        assert dev.steps_per_launch == (int(env["L2H_FLOW_STEPS"]) if env else 1)  # l2h_model_steps_per_launch
         ids, logits = dev.generate_greedy(prompt, n_new, want_logits=True)
         got.append((np.asarray(ids).tolist(), logits.copy()))
         dev.close()
     for other in got[1:]:
         assert other[0] == got[0][0]
         assert np.array_equal(other[1].view(np.uint32), got[0][1].view(np.uint32))
+    # the library's own choice: eight steps where no two heads share a cache row, one otherwise
+    for k in ("L2H_KV_UNCACHED", "L2H_FLOW_STEPS"):
+        monkeypatch.delenv(k, raising=False)
+    lm._device = None
+    dev = lm.device(path=3)
+    assert dev.steps_per_launch == (8 if kw["n_heads"] == kw["n_kv_heads"] else 1)
+    dev.close()
 
 
 def test_streaming_kernel_gives_up_and_recovers(pkg):
