@@ -71,6 +71,11 @@ __shared__ int s_tl_fine;
 #endif
 __shared__ __attribute__((aligned(16))) unsigned char s_sink[256];  // target of fetches made only to warm the L2
 __shared__ int s_tok;  // the token of a launch's next step (flow_next_token)
+// The rows of the residual stream x that this workgroup adds to after wo and after w2 (the same rows, the same threads:
+// k_flow_plan checks it): thread t keeps its row's current value here, so that the addition needs no load of the word
+// the thread itself published a phase ago.
+#define FLOW_RESID_ROWS 64
+__shared__ float s_resid[FLOW_RESID_ROWS];
 #define FLOW_TOK_COPIES 8
 
 __device__ __forceinline__ void tag_store(u64 *p, float v, unsigned epoch) {
@@ -105,12 +110,6 @@ __device__ __forceinline__ void bare_store(unsigned *p, unsigned v) {
 __device__ __forceinline__ unsigned bare_of(float v) {
     const unsigned u = __float_as_uint(v);
     return u == FLOW_EMPTY ? 0x7FC00000u : u;
-}
-// one bare word, waited for (the caller has usually seen it already)
-__device__ __forceinline__ float bare_read(const unsigned *p, unsigned seen) {
-    unsigned w = seen, spins = 0;
-    while (w == FLOW_EMPTY && ++spins <= c_flow.spin_limit) w = bare_load(p);
-    return __uint_as_float(w);
 }
 
 __host__ __device__ inline int flow_n_local(const FlowGeom &g, int wg) {
@@ -1146,9 +1145,9 @@ __device__ __forceinline__ void flow_finish_qkv(int l, int wg, int pos, unsigned
 }
 
 // dst = old + result (x .+= ..., :284,305); which = 1 after wo (-> x_b), 3 after w2 (-> x_a); `old` is
-// this thread's row of the other buffer, fetched before the loop (the same thread wrote it)
+// this thread's row of the other buffer, which the same thread wrote and kept in s_resid
 template <bool HALF = false>
-__device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned oldw) {
+__device__ __forceinline__ void flow_finish_resid(int which, int wg) {
     which = uni(which), wg = uni(wg);
     const FlowArgs &a = c_flow;
     const FlowGeom &g = which == 1 ? a.wo : a.w2;
@@ -1160,8 +1159,9 @@ __device__ __forceinline__ void flow_finish_resid(int which, int wg, unsigned ol
     flow_barrier_lds();
     if (tid >= n_local) return;
     const int row = wg * g.rpw + tid;
-    const float old = bare_read(src + row, oldw);
-    bare_store(dst + row, bare_of(old + flow_row_value4<HALF>(tid, g.ppr, flow_half<HALF>(g))));
+    const unsigned neww = bare_of(s_resid[tid] + flow_row_value4<HALF>(tid, g.ppr, flow_half<HALF>(g)));
+    bare_store(dst + row, neww);
+    s_resid[tid] = __uint_as_float(neww);  // (the value as the other workgroups read it)
     bare_store(src + row, FLOW_EMPTY);  // (its readers are through: see FLOW_EMPTY)
 }
 
@@ -1946,7 +1946,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
     // the rows of x this workgroup adds to after wo (layer 0): straight from the embedding (:236)
     {
         const int lo = wg * a.wo.rpw, n = flow_n_local(a.wo, wg);
-        if (tid < n) bare_store(a.x_a + lo + tid, bare_of(dequant_elem(a.emb, tok, lo + tid)));
+        if (tid < n) s_resid[tid] = __uint_as_float(bare_of(dequant_elem(a.emb, tok, lo + tid)));
     }
 
     for (int l = 0; l < a.n_layers; l++) {
@@ -1997,9 +1997,6 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
             if (!uni(ok)) LEAVE();
             FTL();
             reg_ptr += n_reg * FLOW_SLOT;
-            // the row of x this thread adds to after wo / w2: fetched now, used after the loop
-            unsigned oldw = 0;
-            if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = bare_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
             // what the ring holds has landed by now: after this wait the first FLOW_D pieces need none,
             // and the cache lines requested next do not stand between the loop and its pieces
             flow_drain(r);
@@ -2028,11 +2025,11 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
             if (kind == 0)
                 flow_finish_qkv<MIXED, HALF>(l, wg, pos, e_q);
             else if (kind == 1)
-                flow_finish_resid<HALF>(1, wg, oldw);
+                flow_finish_resid<HALF>(1, wg);
             else if (kind == 2)
                 flow_finish_w13<HALF>(wg, e_w13);
             else
-                flow_finish_resid<HALF>(3, wg, oldw);
+                flow_finish_resid<HALF>(3, wg);
             FTL();
         }
     }
@@ -2279,7 +2276,7 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0, int n
     const bool is_att = uni((int)(att_h < a.n_heads && wg % att_stride == att_h % att_stride)) != 0;
     {
         const int lo = wg * a.wo.rpw, n = flow_n_local(a.wo, wg);
-        if (tid < n) bare_store(a.x_a + lo + tid, bare_of(dequant_elem(a.emb, tok, lo + tid)));
+        if (tid < n) s_resid[tid] = __uint_as_float(bare_of(dequant_elem(a.emb, tok, lo + tid)));
     }
     for (int l = 0; l < a.n_layers; l++) {
         const unsigned e_x = E0 + 5u * (unsigned)l;
@@ -2313,19 +2310,17 @@ __global__ __launch_bounds__(1024) void flow_f32_kernel(unsigned int gen0, int n
             }
             if (!uni(ok)) return;
             XTL();
-            unsigned oldw = 0;
-            if ((kind & 1) && tid < flow_n_local(g, wg)) oldw = bare_load((kind == 1 ? a.x_a : a.x_b) + wg * g.rpw + tid);
             if (kind == 0 && is_att && pos < FLOW_ATT_SHORT) flow_touch_cache(l, att_h, pos);
             flow_loop_f32<false>(pre, g, kind, l, wg, K);
             XTL();
             if (kind == 0)
                 flow_finish_qkv(l, wg, pos, e_q);
             else if (kind == 1)
-                flow_finish_resid(1, wg, oldw);
+                flow_finish_resid(1, wg);
             else if (kind == 2)
                 flow_finish_w13(wg, e_w13);
             else
-                flow_finish_resid(3, wg, oldw);
+                flow_finish_resid(3, wg);
             XTL();
         }
     }
@@ -2536,6 +2531,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
                 if (g->rpw > FLOW_MAX_ROWS || g->rpw * g->ppr > (g == &a.cls ? FLOW_MAX_PIECES : FLOW_MAX_PIECES / 4))
                     return no("too many rows per workgroup");
             if ((a.dim + 2 * a.kv_dim) % 2 != 0) return no("odd row count");
+            if (a.wo.rpw != a.w2.rpw || a.wo.rpw > FLOW_RESID_ROWS) return no("too many rows of x per workgroup");
             a.f32 = 1;
             a.dim_pad = a.dim;
             return true;
@@ -2584,6 +2580,7 @@ bool k_flow_plan(FlowArgs &a, const int *layer_types, int n_layer_types, int cls
     if ((a.dim + 2 * a.kv_dim) % 2 != 0 || (halves && (a.dim % 2 != 0 || a.kv_dim % 2 != 0)))
         return no("odd row count");
     if (a.wo.rpw != a.w2.rpw) return no("row split of wo and w2 differs");  // (a row of x has one owner)
+    if (a.wo.rpw > FLOW_RESID_ROWS) return no("too many rows of x per workgroup");
     return true;
 }
 
