@@ -62,6 +62,8 @@ __shared__ int s_flag;
 #ifdef L2H_TIMELINE
 // profiling build: flow_stage's own stamps (thread 0 of one workgroup, one layer) go to a.timeline[s_tl_fine++]
 __shared__ int s_tl_fine;
+// ... and where lane 0 of every wavefront of that workgroup stamps the end of its streaming loop (-1: nowhere)
+__shared__ int s_tl_wave;
 #define STG()                                                                                          \
     do {                                                                                               \
         if (threadIdx.x == 0 && a.timeline && s_tl_fine >= 0) a.timeline[s_tl_fine++] = wall_clock64(); \
@@ -735,6 +737,9 @@ __device__ __forceinline__ void flow_loop_q4(const FlowGeom &g, Ring &r, unsigne
             }
     }
 #undef FLOW_PIECE_DONE
+#ifdef L2H_TIMELINE
+    if (c_flow.timeline && lane == 0 && s_tl_wave >= 0) c_flow.timeline[s_tl_wave + wave] = wall_clock64();
+#endif
 }
 
 // classifier pieces (q6_K): 16 super-blocks per piece, lane = (block lane/4, chunk lane%4); the ring
@@ -1970,6 +1975,7 @@ __global__ __launch_bounds__(1024) void flow_token_kernel(unsigned int gen0, int
             if (!MIXED && kind != 1) flow_reg_fetch(rp, reg_ptr, n_reg, lane);
 #ifdef L2H_TIMELINE
             if (tid == 0) s_tl_fine = ((int)gridDim.x > 101 && wg == 101 && l == 2) ? 256 * 64 + 512 + kind * 8 : -1;
+            if (tid == 0) s_tl_wave = ((int)gridDim.x > 101 && wg == 101 && l == 2) ? 256 * 64 + 600 + kind * 16 : -1;
 #endif
             if (kind == 0) {
                 const float *nw = a.rms_att + (int64_t)l * a.norm_stride;

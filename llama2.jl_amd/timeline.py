@@ -96,6 +96,16 @@ def main():
             f = (fine[k][:len(labels)] - t0) * 0.01 - last
             print("staging for %-3s (workgroup 101, layer 2), us after the last workgroup's previous epilogue: " % ph +
                   ", ".join("%s %+.2f" % (lab, float(v)) for lab, v in zip(labels, f)))
+        # the end of every wavefront's streaming loop in that workgroup and layer, relative to the drained stamp of the phase
+        # (the moment the loops start); the all-q4_K loop only
+        waves = buf[n_wg * 64 + 600:n_wg * 64 + 600 + 64].reshape(4, 16)
+        for k, ph in enumerate(PHASES):
+            if waves[k].min() <= 0:
+                continue
+            start = float(us[101, names.index("%s drained l2" % ph)])
+            w = (waves[k] - t0) * 0.01 - start
+            print("loop of %-3s (workgroup 101, layer 2), us after the loops started, wavefronts 0..15: " % ph +
+                  " ".join("%.2f" % float(v) for v in w))
     dev.close()
 
 
