@@ -573,7 +573,7 @@ def test_streaming_kernel_soak_against_per_phase_path(pkg, case, reps, n_new):
     """The streaming kernel's exchange of activations between workgroups rests on timing-independent
     reasoning (every buffer is rewritten two phases after its last read); this repeats it: generations of
     up to 128 tokens (30 of them at the benchmark's widths, two layers; a dozen for each other form of the
-    kernel: typed pieces, padded rows with head size 96, fp32 rows), different prompts, each compared bit for
+    kernel: typed pieces, rows of a piece and a half with head size 96, fp32 rows), different prompts, each compared bit for
     bit (tokens and final logits) with the per-phase path, stopping at the first difference or error."""
     from llama2_jl_amd import synth
     from llama2_jl_amd.inference import DeviceModel
