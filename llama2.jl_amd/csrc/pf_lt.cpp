@@ -8,6 +8,7 @@
 // of its calls fails at set-up, pf_lt_open returns nullptr with the reason and the prompt pass runs its own product
 // kernels throughout.
 #include <dlfcn.h>
+#include <stdlib.h>
 #include <hipblaslt/hipblaslt.h>
 
 #include <map>
@@ -77,9 +78,19 @@ PfLt *pf_lt_open(std::string *why) {
     };
     PfLt *lt = new PfLt();
     LtApi &a = lt->api;
-    a.so = dlopen("libhipblaslt.so.1", RTLD_NOW | RTLD_LOCAL);
-    if (!a.so) a.so = dlopen("libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
-    if (!a.so) return fail(lt, std::string("hipBLASLt not found: ") + (dlerror() ? dlerror() : ""));
+    // L2H_HIPBLASLT names the shared object to open instead of the system's (another build of the library; a name that
+    // does not exist leaves the own product kernels in charge, which is how the fallback is tested)
+    const char *named = getenv("L2H_HIPBLASLT");
+    if (named && *named) {
+        a.so = dlopen(named, RTLD_NOW | RTLD_LOCAL);
+    } else {
+        a.so = dlopen("libhipblaslt.so.1", RTLD_NOW | RTLD_LOCAL);
+        if (!a.so) a.so = dlopen("libhipblaslt.so", RTLD_NOW | RTLD_LOCAL);
+    }
+    if (!a.so) {
+        const char *e = dlerror();
+        return fail(lt, std::string("hipBLASLt not found: ") + (e ? e : ""));
+    }
 #define LT_SYM(name)                                                                   \
     do {                                                                               \
         a.name = (decltype(a.name))dlsym(a.so, "hipblasLt" #name);                     \

@@ -135,6 +135,30 @@ def test_prefill_weight_copy_changes_nothing(pkg, case):
     assert not dev.prefill_library and nxt == got[0][1] and np.array_equal(logits, got[0][0])
 
 
+def test_prefill_without_the_gemm_library(pkg, monkeypatch):
+    """Where hipBLASLt cannot be opened (here: L2H_HIPBLASLT names a file that does not exist) the prompt pass runs this
+    library's product kernels and says so; same results, bit for bit, as with the library switched off by the caller."""
+    from llama2_jl_amd import synth
+    plan, kw = CASES["q4ks_gqa"]
+    lm = _model(pkg, plan, **kw)
+    prompt = synth.seeded_prompt(5, lm.config.seq_len - 7, lm.config.vocab_size)
+    got = []
+    for missing in (True, False):
+        if missing:
+            monkeypatch.setenv("L2H_HIPBLASLT", "/nonexistent/libhipblaslt.so")
+        else:
+            monkeypatch.delenv("L2H_HIPBLASLT", raising=False)
+        lm._device = None
+        dev = lm.device()
+        if not missing:
+            dev.set_prefill_library(False)
+        logits, nxt = dev.prefill(prompt, 0)
+        assert not dev.prefill_library
+        got.append((logits.copy(), nxt))
+        dev.close()
+    assert got[0][1] == got[1][1] and np.array_equal(got[0][0], got[1][0])
+
+
 def test_prefill_longer_than_one_chunk(pkg, orc):
     """More positions than one internal chunk (2048): the second chunk's queries attend to the first's keys."""
     from llama2_jl_amd import synth
