@@ -455,23 +455,28 @@ __device__ __forceinline__ void q8k_quantize_rows16(const float (&v)[16], q8k_u3
 #pragma unroll
     for (int k = 0; k < 2; k++) c[k] = fabsf(c[2 * k + 1]) > fabsf(c[2 * k]) ? c[2 * k + 1] : c[2 * k];
     const float mx = fabsf(c[1]) > fabsf(c[0]) ? c[1] : c[0], amax = fabsf(mx);
-    float rmax = amax;
-    rmax = fmaxf(rmax, dpp_f32<DPP_QUAD_SWAP1>(rmax));
-    rmax = fmaxf(rmax, dpp_f32<DPP_QUAD_SWAP2>(rmax));
-    rmax = fmaxf(rmax, dpp_f32<DPP_ROW_HALF_MIRROR>(rmax));
-    rmax = fmaxf(rmax, dpp_f32<DPP_ROW_MIRROR>(rmax));
-    // lowest lane of the row whose own extreme reaches the block's: its first such element is the block's first
-    // (on the scalar unit, a row at a time; a row's set is empty only where the block has a NaN: the row's lane 0 then
-    // stands in, so that `first` is always a lane of the row)
-    const unsigned long long holders = __ballot(amax == rmax);
-    float bmx = 0.0f;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-        const unsigned row = (unsigned)(holders >> (16 * r)) & 0xFFFFu;
-        const int first = 16 * r + __builtin_ctz(row | (unsigned)(row == 0u));
-        const float m = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mx), first));
-        bmx = (int)(threadIdx.x & 48u) == 16 * r ? m : bmx;
-    }
+    // The row's first element of largest magnitude: the sixteen lanes of a row agree on the lane with the largest |x| --
+    // among equal ones the lowest, whose first such element is the block's first -- and on that lane's signed value.
+    // (|x| >= 0 compares as an unsigned integer; a NaN compares above everything and then fixes the scale: unspecified
+    // quants, no fault.  The four exchanges leave every lane of the row with the row's winner, as they do for a maximum.)
+    unsigned kb = __float_as_uint(amax), kl = threadIdx.x & 15u;
+    float bmx = mx;
+#define Q8K_ROW_STEP(CTRL)                                                                                        \
+    do {                                                                                                          \
+        const unsigned ob = (unsigned)__builtin_amdgcn_update_dpp((int)kb, (int)kb, CTRL, 0xF, 0xF, true);        \
+        const unsigned ol = (unsigned)__builtin_amdgcn_update_dpp((int)kl, (int)kl, CTRL, 0xF, 0xF, true);        \
+        const float ov = dpp_f32<CTRL>(bmx);                                                                      \
+        const bool take = ob > kb || (ob == kb && ol < kl);                                                       \
+        kb = take ? ob : kb;                                                                                      \
+        kl = take ? ol : kl;                                                                                      \
+        bmx = take ? ov : bmx;                                                                                    \
+    } while (0)
+    Q8K_ROW_STEP(DPP_QUAD_SWAP1);
+    Q8K_ROW_STEP(DPP_QUAD_SWAP2);
+    Q8K_ROW_STEP(DPP_ROW_HALF_MIRROR);
+    Q8K_ROW_STEP(DPP_ROW_MIRROR);
+#undef Q8K_ROW_STEP
+    const float rmax = __uint_as_float(kb);
     const bool zero = rmax == 0.0f;
     const float iscale = zero ? 0.0f : -127.0f / bmx;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
