@@ -101,6 +101,12 @@ end
 "Which of the library's launch paths decodes this model (3 = the one-launch-per-token streaming kernel), and why not 3."
 launch_path(m::DeviceModel) = Int(ccall((:l2h_model_path, lib), Cint, (Ptr{Cvoid},), m.handle))
 launch_path_reason(m::DeviceModel) = unsafe_string(ccall((:l2h_model_path_reason, lib), Cstring, (Ptr{Cvoid},), m.handle))
+"Steps of the token loop (src/inference.jl:349-386) that one kernel launch of `generate` runs."
+steps_per_launch(m::DeviceModel) = Int(ccall((:l2h_model_steps_per_launch, lib), Cint, (Ptr{Cvoid},), m.handle))
+"Whether `prefill!` runs its plain products (q|k|v, wo, w2) through hipBLASLt (default) or through the library's own kernels."
+set_prefill_library!(m::DeviceModel, on::Bool) =
+    check(m.ctx.handle, ccall((:l2h_model_set_prefill_library, lib), Cint, (Ptr{Cvoid}, Cint), m.handle, on ? 1 : 0))
+prefill_library(m::DeviceModel) = ccall((:l2h_model_prefill_library, lib), Cint, (Ptr{Cvoid},), m.handle) != 0
 
 reset!(m::DeviceModel) = check(m.ctx.handle, ccall((:l2h_state_reset, lib), Cint, (Ptr{Cvoid},), m.handle))
 
