@@ -28,10 +28,10 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E datasheet peak
 # timed region):
 #   (8b-q4ks, launch path 1): per matvec launch, 31.23 MB read + 0.04 MB written (profiles/pmc_fetch_write_bench_8b-q4ks.md)
 #   launch path 3, per token launch (profiles/pmc_fetch_write_streaming_kernel_all_workloads.md):
-#     8b-q4ks 4500.9 MB read + 9.3 MB written, 8b-q5km 5760.0 + 9.3, phi3-4k 5316.8 + 40.5 (per step: its launches run
+#     8b-q4ks 4501.1 MB read + 30.3 MB written, 8b-q5km 5760.0 + 9.3, phi3-4k 5316.8 + 40.5 (per step: its launches run
 #     eight), llama2c-f32 172.6 + 0.8,
 #     8b-q4ks-prefill (its decode steps at positions 2048 and up) 5021.0 + 67.1
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4510221000, ("8b-q5km", 3): 5769380000,
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {("8b-q4ks", 1): 31264000, ("8b-q4ks", 3): 4531362000, ("8b-q5km", 3): 5769380000,
                                      ("phi3-4k", 3): 5357300000, ("llama2c-f32", 3): 173480000,
                                      ("8b-q4ks-prefill", 3): 5088146000}
 
