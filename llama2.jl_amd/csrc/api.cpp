@@ -1400,6 +1400,25 @@ extern "C" int l2h_prefill(l2h_model *m, const int32_t *tokens, int n, int pos0,
     int M = 0;
     for (int c0 = 0; c0 < n; c0 += M) {
         M = std::min(m->pf_cap, n - c0);
+        if (m->pf_wbf && m->pf_copy_mode && m->pf_plain) {
+            // The library must have an algorithm for this chunk's three products before anything is computed with it
+            // (it may be installed without the kernels for this device): where it has none, the own kernels take over
+            // for good and the copy's matrices go back to tiles.
+            const int64_t dim = m->c.dim, kvd = m->kv_dim, hid = m->c.hidden_dim;
+            const uint16_t *wb = m->pf_wbf;
+            const bool ok =
+                pf_lt_gemm(m->pf_lt, ctx->stream, wb, m->pf_xn, nullptr, M, dim + 2 * kvd, dim, dim + 2 * kvd, false, &m->pf_lt_err) == hipSuccess &&
+                pf_lt_gemm(m->pf_lt, ctx->stream, wb + m->pf_off_wo, m->pf_att, nullptr, M, dim, dim, dim, true, &m->pf_lt_err) == hipSuccess &&
+                pf_lt_gemm(m->pf_lt, ctx->stream, wb + m->pf_off_w2, m->pf_hb, nullptr, M, dim, hid, dim, true, &m->pf_lt_err) == hipSuccess;
+            if (!ok) {
+                (void)hipGetLastError();
+                m->pf_lt_why = "hipBLASLt has no algorithm for the prompt pass's products: " + m->pf_lt_err;
+                m->pf_lt_err.clear();
+                pf_lt_close(m->pf_lt);
+                m->pf_lt = nullptr;
+                if ((rc = prefill_expand(m, false))) return rc;
+            }
+        }
         HIPCHK(ctx, hipMemcpyAsync(m->pf_tok, tokens + c0, (size_t)M * 4, hipMemcpyHostToDevice, ctx->stream));
         hipError_t e = prefill_chunk(m, M, pos0 + c0);
         if (e != hipSuccess)

@@ -259,6 +259,7 @@ hipError_t k_pf_expand(hipStream_t s, const DevTensor *w, int nseg, int interlea
                        int64_t dst_row0, int pad, int plain);
 // hipBLASLt for the plain products of the prompt pass (pf_lt.cpp): D[M][0..N) (fp32, row stride ldd) = X[M][K] W[N][K]^T
 // (+ D if accumulate), bf16 operands, fp32 sums.  pf_lt_open returns nullptr, and says why, where the library cannot be used.
+// pf_lt_gemm with D == nullptr only prepares the shape (hipErrorNotSupported: the library has no algorithm for it).
 struct PfLt;
 PfLt *pf_lt_open(std::string *why);
 void pf_lt_close(PfLt *lt);

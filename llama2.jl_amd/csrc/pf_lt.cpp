@@ -11,6 +11,7 @@
 #include <stdlib.h>
 #include <hipblaslt/hipblaslt.h>
 
+#include <algorithm>
 #include <map>
 #include <string>
 #include <tuple>
@@ -143,10 +144,14 @@ static bool pf_lt_plan(PfLt *lt, hipStream_t s, LtPlan &p, const uint16_t *W, co
     uint64_t wsz = lt->workspace_bytes;
     hipblasLtMatmulHeuristicResult_t res[PF_LT_CANDIDATES];
     int got = 0;
+    // (L2H_PF_LT_CANDIDATES: how many of the library's proposals to consider, 1 .. 4; 0 = none, which is how the path
+    // "the library is there but has nothing for this product" is tested)
+    int want = PF_LT_CANDIDATES;
+    if (const char *e = getenv("L2H_PF_LT_CANDIDATES")) want = std::max(0, std::min(PF_LT_CANDIDATES, atoi(e)));
     const bool pref_ok = a.MatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsz, sizeof(wsz)) == HIPBLAS_STATUS_SUCCESS;
     const hipblasStatus_t st =
-        pref_ok ? a.MatmulAlgoGetHeuristic(lt->handle, p.desc, p.lw, p.lx, p.ld, p.ld, pref, PF_LT_CANDIDATES, res, &got)
-                : HIPBLAS_STATUS_INTERNAL_ERROR;
+        pref_ok && want > 0 ? a.MatmulAlgoGetHeuristic(lt->handle, p.desc, p.lw, p.lx, p.ld, p.ld, pref, want, res, &got)
+                            : HIPBLAS_STATUS_INTERNAL_ERROR;
     a.MatmulPreferenceDestroy(pref);
     if (st != HIPBLAS_STATUS_SUCCESS || got < 1) return bad("hipBLASLt has no algorithm for this product");
     p.algo = res[0].algo;
@@ -186,6 +191,8 @@ static bool pf_lt_plan(PfLt *lt, hipStream_t s, LtPlan &p, const uint16_t *W, co
     return true;
 }
 
+// D == nullptr: only finds (and keeps) the algorithm for the shape, so that a library that has none is noticed before
+// anything has been computed with it
 hipError_t pf_lt_gemm(PfLt *lt, hipStream_t s, const uint16_t *W, const uint16_t *X, float *D, int M, int64_t N, int64_t K,
                       int64_t ldd, bool accumulate, std::string *err) {
     if (!lt || M < 1 || N < 1 || K < 1 || ldd < N) return hipErrorInvalidValue;
@@ -202,6 +209,7 @@ hipError_t pf_lt_gemm(PfLt *lt, hipStream_t s, const uint16_t *W, const uint16_t
         }
         it = lt->plans.emplace(key, p).first;
     }
+    if (!D) return hipSuccess;
     const LtPlan &p = it->second;
     const float alpha = 1.0f, beta = accumulate ? 1.0f : 0.0f;
     const hipblasStatus_t st = lt->api.Matmul(lt->handle, p.desc, &alpha, W, p.lw, X, p.lx, &beta, D, p.ld, D, p.ld, &p.algo,

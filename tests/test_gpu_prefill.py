@@ -159,6 +159,34 @@ def test_prefill_without_the_gemm_library(pkg, monkeypatch):
     assert got[0][1] == got[1][1] and np.array_equal(got[0][0], got[1][0])
 
 
+def test_prefill_with_a_gemm_library_that_has_no_algorithm(pkg, monkeypatch):
+    """The library opens but offers nothing for the products (L2H_PF_LT_CANDIDATES=0 stands for an installation without
+    the kernels for this device): noticed before anything is computed with it, the own product kernels take over and the
+    copy's matrices are rewritten as tiles; same results, bit for bit, as with the library switched off."""
+    from llama2_jl_amd import synth
+    plan, kw = CASES["q5km"]
+    lm = _model(pkg, plan, **kw)
+    prompt = synth.seeded_prompt(6, lm.config.seq_len - 5, lm.config.vocab_size)
+    got = []
+    for none in (True, False):
+        if none:
+            monkeypatch.setenv("L2H_PF_LT_CANDIDATES", "0")
+        else:
+            monkeypatch.delenv("L2H_PF_LT_CANDIDATES", raising=False)
+        lm._device = None
+        dev = lm.device()
+        if not none:
+            dev.set_prefill_library(False)
+        for rep in range(2):  # (the second call finds the library already given up)
+            dev.reset()
+            logits, nxt = dev.prefill(prompt, 0)
+            assert not dev.prefill_library
+            got.append((logits.copy(), nxt))
+        dev.close()
+    for other in got[1:]:
+        assert other[1] == got[0][1] and np.array_equal(other[0], got[0][0])
+
+
 def test_prefill_longer_than_one_chunk(pkg, orc):
     """More positions than one internal chunk (2048): the second chunk's queries attend to the first's keys."""
     from llama2_jl_amd import synth
